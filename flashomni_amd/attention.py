@@ -1,0 +1,460 @@
+"""``BatchFlashOmniFAWithRaggedKVWrapper``: ragged block-sparse FlashAttention prefill.
+
+The public surface (constructor, ``plan``, ``run``, ``run_return_lse``, the deprecated
+``forward*`` aliases, defaults and error types) is that of the reference
+(flashomni/attention.py:194-869).  Behind it:
+
+* ``plan()`` runs the host planner (fo_prefill_plan) into the wrapper's integer workspace, builds
+  the q-block table and sizes the work-list buffers;
+* ``run()`` first decodes the bit-packed symbols into a compacted work list on the GPU
+  (fo_decode_sparse; skipped when the same symbol tensors were decoded by the previous call) and
+  then launches the sparse FlashAttention kernel over that list (fo_sparse_fa_run).
+
+Only what the reference's shipped build supports is implemented: no causal / custom mask, no
+positional encoding, no logits soft cap, fp32 logits (reference: setup.py:98-111).
+"""
+import functools
+import math
+from typing import Optional, Tuple, Union
+
+import torch
+
+from . import _lib
+from .utils import (MaskMode, PosEncodingMode, TensorLayout, _check_cached_qkv_data_type,  # noqa: F401
+                    _check_kv_layout, _check_pos_encoding_mode, _check_shape_dtype_device,
+                    canonicalize_torch_dtype, is_float8)
+
+
+def _compute_sparse_info_indptr(qo_indptr: torch.Tensor, num_qo_heads, sparse_block_size_for_q: int,
+                                device: torch.device = "cuda") -> torch.Tensor:
+    """Bit-count indptr of ``sparse_info`` (reference: flashomni/attention.py:165-176)."""
+    sparse_info_indptr = torch.empty_like(qo_indptr, device=device)
+    sparse_info_indptr[0] = 0
+    sparse_info_indptr[1:] = torch.cumsum(
+        torch.ceil((qo_indptr[1:] - qo_indptr[:-1]) / sparse_block_size_for_q) * num_qo_heads, 0)
+    return sparse_info_indptr
+
+
+def _compute_sparse_kv_info_indptr(qo_indptr: torch.Tensor, kv_indptr: torch.Tensor, num_qo_heads,
+                                   sparse_block_size_for_q: int, sparse_block_size_for_kv: int,
+                                   device: torch.device = "cuda") -> torch.Tensor:
+    """Bit-count indptr of ``sparse_kv_info`` (reference: flashomni/attention.py:178-191)."""
+    sparse_kv_info_indptr = torch.empty_like(qo_indptr, device=device)
+    sparse_kv_info_indptr[0] = 0
+    sparse_kv_info_indptr[1:] = torch.cumsum(
+        torch.ceil((qo_indptr[1:] - qo_indptr[:-1]) / sparse_block_size_for_q)
+        * torch.ceil((kv_indptr[1:] - kv_indptr[:-1]) / sparse_block_size_for_kv)
+        * num_qo_heads, 0)
+    return sparse_kv_info_indptr
+
+
+class DecodedWorkList:
+    """Device buffers holding one decoded work list (canonical order).
+
+    ``row_req/row_qb/row_head[n_rows]``, ``kv_row_ptr[n_rows+1]``, ``kv_idx[nnz]``, all int32;
+    ``counts = [n_rows, nnz, 0, 0]``.  The sizes live on the device; ``sizes()`` copies them back
+    (one synchronisation) for tests and reports."""
+
+    def __init__(self, max_rows: int, max_nnz: int, device):
+        self.max_rows, self.max_nnz = max_rows, max_nnz
+        n = max(max_rows, 1)
+        self.row_req = torch.empty(n, dtype=torch.int32, device=device)
+        self.row_qb = torch.empty(n, dtype=torch.int32, device=device)
+        self.row_head = torch.empty(n, dtype=torch.int32, device=device)
+        self.kv_row_ptr = torch.empty(n + 1, dtype=torch.int32, device=device)
+        self.kv_idx = torch.empty(max(max_nnz, 1), dtype=torch.int32, device=device)
+        self.counts = torch.zeros(4, dtype=torch.int32, device=device)
+        self.scratch = torch.empty(2 * n + 2, dtype=torch.int32, device=device)
+
+    def sizes(self) -> Tuple[int, int]:
+        c = self.counts.cpu()
+        return int(c[0]), int(c[1])
+
+    def to_host(self):
+        n_rows, nnz = self.sizes()
+        return (self.row_req[:n_rows].cpu(), self.row_qb[:n_rows].cpu(), self.row_head[:n_rows].cpu(),
+                self.kv_row_ptr[:n_rows + 1].cpu(), self.kv_idx[:nnz].cpu())
+
+
+class BatchFlashOmniFAWithRaggedKVWrapper:
+    r"""Wrapper class for block-sparse prefill attention over ragged q/k/v tensors.
+
+    >>> workspace = torch.empty(128 * 1024 * 1024, dtype=torch.uint8, device="cuda:0")
+    >>> wrapper = BatchFlashOmniFAWithRaggedKVWrapper(workspace, "NHD")
+    >>> wrapper.plan(qo_indptr, kv_indptr, num_qo_heads, num_kv_heads, head_dim,
+    ...              sparse_block_size_for_q=128, sparse_block_size_for_kv=128,
+    ...              q_data_type=torch.bfloat16)
+    >>> o = wrapper.run(q, k, v, sparse_info, sparse_kv_info, sparse_info_indptr,
+    ...                 sparse_kv_info_indptr)
+
+    ``sparse_info`` holds one bit per (q-block, head) (1 = compute, 0 = cached: the rows of ``out``
+    are left untouched), ``sparse_kv_info`` one bit per (q-block, head, kv-block) (1 = keep), both
+    packed little-endian per request; the two indptr tensors are the byte offsets returned by
+    ``segment_packbits``.
+    """
+
+    def __init__(
+        self,
+        float_workspace_buffer: torch.Tensor,
+        kv_layout: str = "NHD",
+        use_cuda_graph: bool = False,
+        qo_indptr_buf: Optional[torch.Tensor] = None,
+        kv_indptr_buf: Optional[torch.Tensor] = None,
+        custom_mask_buf: Optional[torch.Tensor] = None,
+        mask_indptr_buf: Optional[torch.Tensor] = None,
+        backend: str = "auto",
+    ) -> None:
+        _check_kv_layout(kv_layout)
+        self._kv_layout = kv_layout
+        self._float_workspace_buffer = float_workspace_buffer
+        self.device = float_workspace_buffer.device
+        if self.device.type != "cuda":
+            raise ValueError("float_workspace_buffer must live on the GPU; there is no CPU path")
+        self._int_workspace_buffer = torch.empty((8 * 1024 * 1024,), dtype=torch.uint8,
+                                                 device=self.device)
+        self._pin_memory_int_workspace_buffer = torch.empty(
+            self._int_workspace_buffer.shape, dtype=torch.uint8, pin_memory=True, device="cpu")
+        self._use_cuda_graph = use_cuda_graph
+        if use_cuda_graph:
+            if not torch.is_tensor(qo_indptr_buf):
+                raise ValueError("qo_indptr_buf should be a torch.Tensor in cuda graph mode")
+            if not torch.is_tensor(kv_indptr_buf):
+                raise ValueError("kv_indptr_buf should be a torch.Tensor in cuda graph mode")
+            self._fixed_batch_size = len(qo_indptr_buf) - 1
+            if len(kv_indptr_buf) != self._fixed_batch_size + 1:
+                raise ValueError(
+                    "The length of kv_indptr_buf ({}) should be the same as qo_indptr_buf ({}).".format(
+                        len(kv_indptr_buf), self._fixed_batch_size))
+        self._qo_indptr_buf = qo_indptr_buf
+        self._kv_indptr_buf = kv_indptr_buf
+        self._custom_mask_buf = custom_mask_buf
+        self._mask_indptr_buf = mask_indptr_buf
+        self._max_total_num_rows = None
+        self._backend = backend  # accepted for compatibility; there is one HIP code path
+        self._plan_info = None
+        self._worklist = None
+        self._decode_key = None
+
+    @property
+    def is_cuda_graph_enabled(self) -> bool:
+        return self._use_cuda_graph
+
+    def reset_workspace_buffer(self, float_workspace_buffer: torch.Tensor,
+                               int_workspace_buffer) -> None:
+        self._float_workspace_buffer = float_workspace_buffer
+        self._int_workspace_buffer = int_workspace_buffer
+        self._pin_memory_int_workspace_buffer = torch.empty(
+            self._int_workspace_buffer.shape, dtype=self._int_workspace_buffer.dtype, device="cpu",
+            pin_memory=True)
+
+    # ------------------------------------------------------------------------------------------
+    def plan(
+        self,
+        qo_indptr: torch.Tensor,
+        kv_indptr: torch.Tensor,
+        num_qo_heads: int,
+        num_kv_heads: int,
+        head_dim_qk: int,
+        sparse_block_size_for_q: int = 128,
+        sparse_block_size_for_kv: int = 128,
+        head_dim_vo: Optional[int] = None,
+        custom_mask: Optional[torch.Tensor] = None,
+        packed_custom_mask: Optional[torch.Tensor] = None,
+        causal: bool = False,
+        pos_encoding_mode: str = "NONE",
+        use_fp16_qk_reduction: bool = False,
+        logits_soft_cap: Optional[float] = None,
+        sm_scale: Optional[float] = None,
+        rope_scale: Optional[float] = None,
+        rope_theta: Optional[float] = None,
+        q_data_type: Union[str, torch.dtype] = "float16",
+        kv_data_type: Optional[Union[str, torch.dtype]] = None,
+    ) -> None:
+        r"""Plan sparse prefill attention for the given ragged batch.
+
+        Same parameters as the reference ``plan``.  The host planner tiles the batch into the
+        integer workspace; in addition the q-block table of the symbol decoder is built and the
+        work-list buffers are sized for the worst case (every bit set).  Cannot be captured in a
+        graph (it copies the indptrs to the host)."""
+        q_data_type = canonicalize_torch_dtype(q_data_type)
+        if kv_data_type is None:
+            kv_data_type = q_data_type
+        kv_data_type = canonicalize_torch_dtype(kv_data_type)
+        if head_dim_vo is None:
+            head_dim_vo = head_dim_qk
+        if logits_soft_cap is None:
+            logits_soft_cap = 0.0
+
+        batch_size = len(qo_indptr) - 1
+        if len(kv_indptr) != batch_size + 1:
+            raise ValueError("The kv_indptr length should be equal to mask_indptr length.")
+        _check_pos_encoding_mode(pos_encoding_mode)
+        if custom_mask is not None or packed_custom_mask is not None or causal:
+            raise NotImplementedError(
+                "causal / custom masks are not part of the sparse prefill path (the reference build "
+                "only instantiates the non-causal kernel)")
+        if PosEncodingMode[pos_encoding_mode] != PosEncodingMode.NONE or logits_soft_cap > 0 \
+                or use_fp16_qk_reduction:
+            raise NotImplementedError(
+                "positional encoding, logits soft cap and fp16 logits are not part of the sparse "
+                "prefill path")
+        if num_qo_heads != num_kv_heads:
+            raise NotImplementedError("grouped-query attention (num_qo_heads != num_kv_heads) is not "
+                                      "supported by the sparse prefill path")
+        if head_dim_qk != 128 or head_dim_vo != 128:
+            raise NotImplementedError("only head_dim 128 is supported")
+        if sparse_block_size_for_q != 128 or sparse_block_size_for_kv != 128:
+            raise NotImplementedError("only 128 x 128 sparse blocks are supported")
+
+        qo_indptr_host = qo_indptr.to("cpu", torch.int32).contiguous()
+        kv_indptr_host = kv_indptr.to("cpu", torch.int32).contiguous()
+        total_num_rows = int(qo_indptr_host[-1])
+
+        if self.is_cuda_graph_enabled:
+            if self._max_total_num_rows is None:
+                self._max_total_num_rows = total_num_rows
+            elif total_num_rows > self._max_total_num_rows:
+                raise ValueError(
+                    "The total number of rows in qo_indptr {} in cuda graph mode cannot "
+                    "exceed the number of rows set during initialization {}.".format(
+                        total_num_rows, self._max_total_num_rows))
+            if batch_size != self._fixed_batch_size:
+                raise ValueError(
+                    "The batch size should be fixed in cudagraph mode, the runtime batch size {} "
+                    " mismatches the batch size set during initialization {}.".format(
+                        batch_size, self._fixed_batch_size))
+            self._qo_indptr_buf.copy_(qo_indptr)
+            self._kv_indptr_buf.copy_(kv_indptr)
+        else:
+            self._qo_indptr_buf = qo_indptr_host.to(self.device)
+            self._kv_indptr_buf = kv_indptr_host.to(self.device)
+
+        self._cached_q_data_type = q_data_type
+        self._cached_kv_data_type = kv_data_type
+
+        L = _lib.lib()
+        stream = _lib.current_stream(self.device)
+        plan_info = torch.empty(15, dtype=torch.int64)
+        with torch.cuda.device(self.device):
+            try:
+                _lib.check(L.fo_prefill_plan(
+                    _lib.ptr(self._float_workspace_buffer),
+                    self._float_workspace_buffer.numel() * self._float_workspace_buffer.element_size(),
+                    _lib.ptr(self._int_workspace_buffer),
+                    _lib.ptr(self._pin_memory_int_workspace_buffer),
+                    self._int_workspace_buffer.numel() * self._int_workspace_buffer.element_size(),
+                    _lib.ptr(qo_indptr_host), _lib.ptr(kv_indptr_host),
+                    self._max_total_num_rows or total_num_rows, batch_size, num_qo_heads,
+                    num_kv_heads, head_dim_qk, head_dim_vo, 1, int(self.is_cuda_graph_enabled),
+                    q_data_type.itemsize, 0, _lib.ptr(plan_info), stream))
+            except RuntimeError as e:  # same wording as csrc/batch_sparseFA.cu:61
+                raise RuntimeError("Failed to plan prefill with error: " + str(e)) from None
+        self._plan_info = plan_info
+
+        # q-block table + block numbering for the decoder / fp8 scales
+        n_blk = torch.zeros(3, dtype=torch.int64)
+        _lib.check(L.fo_decode_sizes(_lib.ptr(qo_indptr_host), _lib.ptr(kv_indptr_host), batch_size,
+                                     num_qo_heads, sparse_block_size_for_q, sparse_block_size_for_kv,
+                                     n_blk[0:].data_ptr(), n_blk[1:].data_ptr(), n_blk[2:].data_ptr()))
+        n_q_blk, max_rows, max_nnz = (int(v) for v in n_blk)
+        if max_nnz >= 2 ** 31:
+            raise RuntimeError("Failed to plan prefill with error: work list too large")
+        table = torch.empty((2, max(n_q_blk, 1)), dtype=torch.int32)
+        _lib.check(L.fo_sparse_block_table(_lib.ptr(qo_indptr_host), batch_size,
+                                           sparse_block_size_for_q, table[0].data_ptr(),
+                                           table[1].data_ptr(), n_q_blk, n_blk[0:].data_ptr()))
+        self._blk_table = table.to(self.device)
+        self._n_q_blk = n_q_blk
+        qlen = (qo_indptr_host[1:] - qo_indptr_host[:-1]).to(torch.int64)
+        klen = (kv_indptr_host[1:] - kv_indptr_host[:-1]).to(torch.int64)
+        q_base = torch.zeros(batch_size + 1, dtype=torch.int64)
+        kv_base = torch.zeros(batch_size + 1, dtype=torch.int64)
+        q_base[1:] = torch.cumsum((qlen + sparse_block_size_for_q - 1) // sparse_block_size_for_q, 0)
+        kv_base[1:] = torch.cumsum((klen + sparse_block_size_for_kv - 1) // sparse_block_size_for_kv, 0)
+        self._q_blk_base = q_base.to(torch.int32).to(self.device)
+        self._kv_blk_base = kv_base.to(torch.int32).to(self.device)
+        self._n_kv_blk = int(kv_base[-1])
+        if (self._worklist is None or self._worklist.max_rows < max_rows
+                or self._worklist.max_nnz < max_nnz):
+            self._worklist = DecodedWorkList(max_rows, max_nnz, self.device)
+        self._max_rows = max_rows
+        self._decode_key = None
+
+        self._num_qo_heads = num_qo_heads
+        self._sparse_block_size_for_q = sparse_block_size_for_q
+        self._sparse_block_size_for_kv = sparse_block_size_for_kv
+        self._causal = causal
+        self._pos_encoding_mode = pos_encoding_mode
+        self._use_fp16_qk_reduction = use_fp16_qk_reduction
+        self._logits_soft_cap = logits_soft_cap
+        self._sm_scale = sm_scale
+        self._rope_scale = rope_scale
+        self._rope_theta = rope_theta
+
+        self._sparse_info_indptr_base = _compute_sparse_info_indptr(
+            self._qo_indptr_buf, num_qo_heads, self._sparse_block_size_for_q, device=self.device)
+        self._sparse_kv_info_indptr_base = _compute_sparse_kv_info_indptr(
+            self._qo_indptr_buf, self._kv_indptr_buf, num_qo_heads, self._sparse_block_size_for_q,
+            self._sparse_block_size_for_kv, device=self.device)
+
+    begin_forward = plan
+
+    # ------------------------------------------------------------------------------------------
+    def decode(self, sparse_info, sparse_kv_info, sparse_info_indptr, sparse_kv_info_indptr,
+               is_full: bool = False) -> DecodedWorkList:
+        """Decode the packed symbols into the wrapper's work list (asynchronous, on the current
+        stream) and return it.  ``run`` calls this itself; calling it directly lets a caller decode
+        once and inspect or reuse the list."""
+        if self._plan_info is None:
+            raise RuntimeError("plan() must be called before decode()/run()")
+        wl = self._worklist
+        if not is_full:
+            if sparse_info is None or sparse_kv_info is None or sparse_info_indptr is None \
+                    or sparse_kv_info_indptr is None:
+                raise ValueError("sparse_info, sparse_kv_info and their indptrs are required unless "
+                                 "is_full=True")
+            tensors = []
+            for name, t, dt in (("sparse_info", sparse_info, torch.uint8),
+                                ("sparse_kv_info", sparse_kv_info, torch.uint8),
+                                ("sparse_info_indptr", sparse_info_indptr, torch.int32),
+                                ("sparse_kv_info_indptr", sparse_kv_info_indptr, torch.int32)):
+                if t.device != self.device:
+                    raise ValueError(f"Invalid device of {name}: expected {self.device}, got {t.device}")
+                tensors.append(t.to(dt).contiguous())
+            key = tuple((t.data_ptr(), t._version, t.numel()) for t in
+                        (sparse_info, sparse_kv_info, sparse_info_indptr, sparse_kv_info_indptr))
+        else:
+            tensors = [None] * 4
+            key = "full"
+        if key == self._decode_key:
+            return wl
+        _lib.check(_lib.lib().fo_decode_sparse(
+            _lib.ptr(tensors[0]), _lib.ptr(tensors[1]), _lib.ptr(tensors[2]), _lib.ptr(tensors[3]),
+            _lib.ptr(self._blk_table[0]), _lib.ptr(self._blk_table[1]), _lib.ptr(self._kv_indptr_buf),
+            self._n_q_blk, self._num_qo_heads, self._sparse_block_size_for_kv, int(bool(is_full)),
+            _lib.ptr(wl.row_req), _lib.ptr(wl.row_qb), _lib.ptr(wl.row_head), _lib.ptr(wl.kv_row_ptr),
+            _lib.ptr(wl.kv_idx), _lib.ptr(wl.counts), _lib.ptr(wl.scratch),
+            _lib.current_stream(self.device)))
+        # the memo holds the tensors alive so a recycled address cannot alias the key
+        self._decode_key = key
+        self._decode_refs = (tensors, sparse_info, sparse_kv_info, sparse_info_indptr,
+                             sparse_kv_info_indptr)
+        return wl
+
+    def run(
+        self,
+        q: torch.Tensor,
+        k: torch.Tensor,
+        v: torch.Tensor,
+        sparse_info: torch.Tensor = None,
+        sparse_kv_info: torch.Tensor = None,
+        sparse_info_indptr: torch.Tensor = None,
+        sparse_kv_info_indptr: torch.Tensor = None,
+        is_full: bool = False,
+        *args,
+        out: Optional[torch.Tensor] = None,
+        lse: Optional[torch.Tensor] = None,
+        return_lse: bool = False,
+        q_scale: Optional[torch.Tensor] = None,
+        k_scale: Optional[torch.Tensor] = None,
+    ) -> Union[torch.Tensor, Tuple[torch.Tensor, torch.Tensor]]:
+        r"""Compute block-sparse prefill attention.
+
+        q ``[qo_indptr[-1], H, D]``, k/v ``[kv_indptr[-1], H, D]`` (``NHD``) or ``[H, nnz, D]``
+        (``HND``).  Rows of q-blocks whose ``sparse_info`` bit is 0 are left untouched in ``out``
+        (a fresh ``out`` is zero-filled, as in the reference).  Returns ``out`` or ``(out, lse)``
+        with the base-2 log-sum-exp ``[nnz_q, H]``.
+
+        ``q_scale`` / ``k_scale`` (keyword-only extension): fp32 ``[H, n_blocks]`` dequantisation
+        scales; with them ``q`` and ``k`` are fp8 e4m3fn, ``v`` and ``out`` are bfloat16.
+        """
+        if self._plan_info is None:
+            raise RuntimeError("plan() must be called before run()")
+        _check_cached_qkv_data_type(q, k, self._cached_q_data_type, self._cached_kv_data_type)
+        sm_scale = self._sm_scale
+        if sm_scale is None:
+            sm_scale = 1.0 / math.sqrt(q.size(-1))
+        fp8 = is_float8(q)
+        if fp8:
+            if q.dtype != torch.float8_e4m3fn or k.dtype != torch.float8_e4m3fn \
+                    or q_scale is None or k_scale is None:
+                raise ValueError("fp8 attention needs float8_e4m3fn q and k with q_scale and k_scale")
+            if v.dtype != torch.bfloat16:
+                raise ValueError("fp8 attention keeps v (and the output) in bfloat16")
+        out_dtype = torch.bfloat16 if fp8 else q.dtype
+        if return_lse:
+            if lse is None:
+                lse = torch.empty((q.size(0), q.size(1)), dtype=torch.float32, device=q.device)
+            else:
+                _check_shape_dtype_device(lse, (q.size(0), q.size(1)), torch.float32, q.device, "lse")
+        if out is None:
+            out = torch.zeros(q.shape[:-1] + v.shape[-1:], dtype=out_dtype, device=q.device)
+        else:
+            _check_shape_dtype_device(out, q.shape[:-1] + v.shape[-1:], out_dtype, q.device, "out")
+        if q.device != self.device:
+            raise ValueError(f"Invalid device of q: expected {self.device}, got {q.device}")
+        if q.size(1) != self._num_qo_heads or q.size(2) != 128:
+            raise ValueError("q does not match the head count / head_dim given to plan()")
+        for name, t in (("q", q), ("k", k), ("v", v), ("out", out)):
+            if t.stride(-1) != 1:
+                raise ValueError(f"{name} must have a contiguous last dimension")
+
+        if self._kv_layout == "NHD":
+            k_sn, k_sh, v_sn, v_sh = k.stride(0), k.stride(1), v.stride(0), v.stride(1)
+        else:
+            k_sh, k_sn, v_sh, v_sn = k.stride(0), k.stride(1), v.stride(0), v.stride(1)
+
+        wl = self.decode(sparse_info, sparse_kv_info, sparse_info_indptr, sparse_kv_info_indptr,
+                         is_full)
+        if fp8:
+            q_scale = q_scale.to(torch.float32).contiguous()
+            k_scale = k_scale.to(torch.float32).contiguous()
+            if q_scale.shape != (q.size(1), self._n_q_blk) or k_scale.shape != (q.size(1), self._n_kv_blk):
+                raise ValueError("q_scale / k_scale must be [H, number of 128-token blocks]")
+        _lib.check(_lib.lib().fo_sparse_fa_run(
+            _lib.ptr(q), _lib.ptr(k), _lib.ptr(v), _lib.ptr(out), _lib.ptr(lse if return_lse else None),
+            _lib.dtype_code(q.dtype), _lib.ptr(q_scale if fp8 else None),
+            _lib.ptr(k_scale if fp8 else None),
+            q.stride(0), q.stride(1), k_sn, k_sh, v_sn, v_sh, out.stride(0), out.stride(1),
+            _lib.ptr(self._qo_indptr_buf), _lib.ptr(self._kv_indptr_buf), _lib.ptr(self._q_blk_base),
+            _lib.ptr(self._kv_blk_base), _lib.ptr(wl.row_req), _lib.ptr(wl.row_qb),
+            _lib.ptr(wl.row_head), _lib.ptr(wl.kv_row_ptr), _lib.ptr(wl.kv_idx), _lib.ptr(wl.counts),
+            self._max_rows, q.size(1), q.size(2), self._sparse_block_size_for_q,
+            self._sparse_block_size_for_kv, float(sm_scale), _lib.current_stream(self.device)))
+        return (out, lse) if return_lse else out
+
+    run_return_lse = functools.partialmethod(run, return_lse=True)
+
+    def forward(self, q, k, v, sparse_info=None, sparse_kv_info=None, sparse_info_indptr=None,
+                sparse_kv_info_indptr=None, is_full=False, causal=False, pos_encoding_mode="NONE",
+                use_fp16_qk_reduction=False, logits_soft_cap=None, sm_scale=None, rope_scale=None,
+                rope_theta=None) -> torch.Tensor:
+        r"""Warning: This function is deprecated, please use :meth:`run` instead."""
+        self._set_forward_options(causal, pos_encoding_mode, use_fp16_qk_reduction, logits_soft_cap,
+                                  sm_scale, rope_scale, rope_theta)
+        return self.run(q, k, v, sparse_info, sparse_kv_info, sparse_info_indptr,
+                        sparse_kv_info_indptr, is_full)
+
+    def forward_return_lse(self, q, k, v, sparse_info=None, sparse_kv_info=None,
+                           sparse_info_indptr=None, sparse_kv_info_indptr=None, is_full=False,
+                           causal=False, pos_encoding_mode="NONE", use_fp16_qk_reduction=False,
+                           logits_soft_cap=None, sm_scale=None, rope_scale=None,
+                           rope_theta=None) -> Tuple[torch.Tensor, torch.Tensor]:
+        r"""Warning: This function is deprecated, please use :meth:`run_return_lse` instead."""
+        self._set_forward_options(causal, pos_encoding_mode, use_fp16_qk_reduction, logits_soft_cap,
+                                  sm_scale, rope_scale, rope_theta)
+        return self.run_return_lse(q, k, v, sparse_info, sparse_kv_info, sparse_info_indptr,
+                                   sparse_kv_info_indptr, is_full)
+
+    def _set_forward_options(self, causal, pos_encoding_mode, use_fp16_qk_reduction,
+                             logits_soft_cap, sm_scale, rope_scale, rope_theta):
+        if causal or pos_encoding_mode != "NONE" or use_fp16_qk_reduction or (logits_soft_cap or 0) > 0:
+            raise NotImplementedError("only non-causal attention without positional encoding or "
+                                      "soft cap is supported")
+        self._sm_scale = sm_scale
+        self._rope_scale = rope_scale
+        self._rope_theta = rope_theta
+
+    def end_forward(self) -> None:
+        r"""Warning: this function is deprecated and has no effect."""
+        pass

@@ -1,0 +1,230 @@
+// Sparse-symbol decoder for gfx950: bit-packed (head, q-block) flags and (head, q-block, kv-block)
+// keep masks -> compacted work list in canonical order (ascending request, q-block, head; kv
+// blocks ascending inside a row).  Three short launches on one stream, no host round trip:
+//   count : one wavefront per (q-block, head) candidate; lanes take one mask byte each, popcount
+//   scan  : one workgroup, exclusive prefix sums of row flags and kv counts (canonical positions)
+//   fill  : one wavefront per candidate again; wave prefix of popcounts places every kv index
+// Integer work, bounded by HBM traffic and launch latency; bit-exact by construction.
+//
+// Symbol semantics (reference: include/flashomni/attention/prefill.cuh:1284-1294, 1380-1403,
+// 1434-1460): bit 1 = compute/keep, little-endian bytes, flag bit index qb*H + h, keep-mask bit
+// index (qb*H + h)*NKV + kvb, per-request byte offsets.
+#include "fo_common.h"
+
+namespace {
+
+constexpr int kWave = 64;
+constexpr int kCountThreads = 256;  // 4 candidates per workgroup
+constexpr int kScanThreads = 1024;
+
+struct Candidate {
+  int32_t req, qb, head, nkv;
+  int64_t base;  // first bit of the row inside the request's keep-mask segment
+  bool active;
+};
+
+__device__ __forceinline__ Candidate load_candidate(
+    int64_t c, int32_t num_heads, int32_t block_kv, int is_full,
+    const uint8_t* __restrict__ sparse_info, const int32_t* __restrict__ sparse_info_indptr,
+    const int32_t* __restrict__ blk_req, const int32_t* __restrict__ blk_qb,
+    const int32_t* __restrict__ kv_indptr) {
+  Candidate cd;
+  const int64_t t = c / num_heads;
+  cd.head = static_cast<int32_t>(c - t * num_heads);
+  cd.req = blk_req[t];
+  cd.qb = blk_qb[t];
+  const int32_t kv_len = kv_indptr[cd.req + 1] - kv_indptr[cd.req];
+  cd.nkv = (kv_len + block_kv - 1) / block_kv;
+  const int64_t flag_bit = static_cast<int64_t>(cd.qb) * num_heads + cd.head;
+  cd.base = flag_bit * cd.nkv;
+  if (is_full) {
+    cd.active = true;
+  } else {
+    const uint8_t byte = sparse_info[sparse_info_indptr[cd.req] + (flag_bit >> 3)];
+    cd.active = (byte >> (flag_bit & 7)) & 1;
+  }
+  return cd;
+}
+
+// bits of mask byte `b` (absolute byte index inside the segment) that belong to [base, base+nkv)
+__device__ __forceinline__ uint32_t masked_byte(const uint8_t* __restrict__ seg, int64_t b,
+                                                int64_t base, int32_t nkv) {
+  uint32_t v = seg[b];
+  const int64_t lo = base - b * 8;             // first valid bit position in this byte
+  const int64_t hi = base + nkv - b * 8;       // one past the last valid bit position
+  if (lo > 0) v &= 0xffu << lo;
+  if (hi < 8) v &= (1u << hi) - 1u;
+  return v;
+}
+
+__global__ void __launch_bounds__(kCountThreads) decode_count_kernel(
+    const uint8_t* __restrict__ sparse_info, const uint8_t* __restrict__ sparse_kv_info,
+    const int32_t* __restrict__ sparse_info_indptr,
+    const int32_t* __restrict__ sparse_kv_info_indptr, const int32_t* __restrict__ blk_req,
+    const int32_t* __restrict__ blk_qb, const int32_t* __restrict__ kv_indptr, int64_t n_cand,
+    int32_t num_heads, int32_t block_kv, int is_full, int32_t* __restrict__ act,
+    int32_t* __restrict__ cnt) {
+  const int lane = threadIdx.x % kWave;
+  const int64_t c = static_cast<int64_t>(blockIdx.x) * (kCountThreads / kWave) + threadIdx.x / kWave;
+  if (c >= n_cand) return;
+  const Candidate cd = load_candidate(c, num_heads, block_kv, is_full, sparse_info,
+                                      sparse_info_indptr, blk_req, blk_qb, kv_indptr);
+  int32_t total = 0;
+  if (cd.active) {
+    if (is_full) {
+      total = cd.nkv;
+    } else if (cd.nkv > 0) {
+      const uint8_t* seg = sparse_kv_info + sparse_kv_info_indptr[cd.req];
+      const int64_t b0 = cd.base >> 3, b1 = (cd.base + cd.nkv - 1) >> 3;
+      int32_t part = 0;
+      for (int64_t b = b0 + lane; b <= b1; b += kWave) part += __popc(masked_byte(seg, b, cd.base, cd.nkv));
+      for (int off = kWave / 2; off > 0; off >>= 1) part += __shfl_xor(part, off, kWave);
+      total = part;
+    }
+  }
+  if (lane == 0) {
+    act[c] = cd.active ? 1 : 0;
+    cnt[c] = total;
+  }
+}
+
+// In place: act[c] -> canonical row position (or -1), cnt[c] -> first kv_idx slot of the row.
+__global__ void __launch_bounds__(kScanThreads) decode_scan_kernel(
+    int64_t n_cand, int32_t* __restrict__ act, int32_t* __restrict__ cnt,
+    int32_t* __restrict__ kv_row_ptr, int32_t* __restrict__ counts) {
+  __shared__ int32_t s_rows[kScanThreads];
+  __shared__ int32_t s_kv[kScanThreads];
+  const int tid = threadIdx.x;
+  const int64_t chunk = (n_cand + kScanThreads - 1) / kScanThreads;
+  const int64_t lo = tid * chunk, hi = (lo + chunk < n_cand) ? lo + chunk : n_cand;
+  int32_t rows = 0, kv = 0;
+  for (int64_t c = lo; c < hi; ++c) {
+    rows += act[c];
+    kv += cnt[c];
+  }
+  s_rows[tid] = rows;
+  s_kv[tid] = kv;
+  __syncthreads();
+  // Hillis-Steele inclusive scan over the 1024 partials
+  for (int off = 1; off < kScanThreads; off <<= 1) {
+    int32_t r = 0, k = 0;
+    if (tid >= off) {
+      r = s_rows[tid - off];
+      k = s_kv[tid - off];
+    }
+    __syncthreads();
+    s_rows[tid] += r;
+    s_kv[tid] += k;
+    __syncthreads();
+  }
+  int32_t row_pos = s_rows[tid] - rows, kv_pos = s_kv[tid] - kv;
+  for (int64_t c = lo; c < hi; ++c) {
+    const int32_t a = act[c], n = cnt[c];
+    act[c] = a ? row_pos : -1;
+    cnt[c] = kv_pos;
+    row_pos += a;
+    kv_pos += n;
+  }
+  if (tid == kScanThreads - 1) {
+    const int32_t n_rows = s_rows[tid], nnz = s_kv[tid];
+    counts[0] = n_rows;
+    counts[1] = nnz;
+    counts[2] = 0;
+    counts[3] = 0;
+    kv_row_ptr[n_rows] = nnz;
+  }
+}
+
+__global__ void __launch_bounds__(kCountThreads) decode_fill_kernel(
+    const uint8_t* __restrict__ sparse_info, const uint8_t* __restrict__ sparse_kv_info,
+    const int32_t* __restrict__ sparse_info_indptr,
+    const int32_t* __restrict__ sparse_kv_info_indptr, const int32_t* __restrict__ blk_req,
+    const int32_t* __restrict__ blk_qb, const int32_t* __restrict__ kv_indptr, int64_t n_cand,
+    int32_t num_heads, int32_t block_kv, int is_full, const int32_t* __restrict__ row_pos,
+    const int32_t* __restrict__ kv_pos, int32_t* __restrict__ row_req,
+    int32_t* __restrict__ row_qb, int32_t* __restrict__ row_head,
+    int32_t* __restrict__ kv_row_ptr, int32_t* __restrict__ kv_idx) {
+  const int lane = threadIdx.x % kWave;
+  const int64_t c = static_cast<int64_t>(blockIdx.x) * (kCountThreads / kWave) + threadIdx.x / kWave;
+  if (c >= n_cand) return;
+  const int32_t pos = row_pos[c];
+  if (pos < 0) return;
+  const Candidate cd = load_candidate(c, num_heads, block_kv, is_full, sparse_info,
+                                      sparse_info_indptr, blk_req, blk_qb, kv_indptr);
+  int32_t out = kv_pos[c];
+  if (lane == 0) {
+    row_req[pos] = cd.req;
+    row_qb[pos] = cd.qb;
+    row_head[pos] = cd.head;
+    kv_row_ptr[pos] = out;
+  }
+  if (cd.nkv <= 0) return;
+  if (is_full) {
+    for (int32_t j = lane; j < cd.nkv; j += kWave) kv_idx[out + j] = j;
+    return;
+  }
+  const uint8_t* seg = sparse_kv_info + sparse_kv_info_indptr[cd.req];
+  const int64_t b0 = cd.base >> 3, b1 = (cd.base + cd.nkv - 1) >> 3;
+  for (int64_t bb = b0; bb <= b1; bb += kWave) {  // uniform trip count for the whole wave
+    const int64_t b = bb + lane;
+    uint32_t m = (b <= b1) ? masked_byte(seg, b, cd.base, cd.nkv) : 0u;
+    const int32_t pc = __popc(m);
+    int32_t incl = pc;
+    for (int off = 1; off < kWave; off <<= 1) {
+      const int32_t up = __shfl_up(incl, off, kWave);
+      if (lane >= off) incl += up;
+    }
+    int32_t w = out + incl - pc;
+    while (m) {
+      const int p = __ffs(m) - 1;
+      m &= m - 1;
+      kv_idx[w++] = static_cast<int32_t>(b * 8 + p - cd.base);
+    }
+    out += __shfl(incl, kWave - 1, kWave);
+  }
+}
+
+}  // namespace
+
+extern "C" int fo_decode_sparse(const uint8_t* sparse_info, const uint8_t* sparse_kv_info,
+                                const int32_t* sparse_info_indptr,
+                                const int32_t* sparse_kv_info_indptr, const int32_t* blk_req,
+                                const int32_t* blk_qb, const int32_t* kv_indptr, int32_t n_blk,
+                                int32_t num_heads, int32_t block_kv, int is_full,
+                                int32_t* row_req, int32_t* row_qb, int32_t* row_head,
+                                int32_t* kv_row_ptr, int32_t* kv_idx, int32_t* counts,
+                                int32_t* scratch, void* stream) {
+  FO_REQUIRE(n_blk >= 0 && num_heads > 0 && block_kv > 0, "decode: bad sizes");
+  FO_REQUIRE(counts && kv_row_ptr, "decode: null output");
+  if (!is_full) {
+    FO_REQUIRE(sparse_info && sparse_kv_info && sparse_info_indptr && sparse_kv_info_indptr,
+               "decode: sparse_info, sparse_kv_info and their indptrs are required unless is_full");
+  }
+  FO_REQUIRE(blk_req && blk_qb && kv_indptr && scratch, "decode: null table");
+  const int64_t n_cand = static_cast<int64_t>(n_blk) * num_heads;
+  FO_REQUIRE(n_cand < (int64_t(1) << 31), "decode: too many (q-block, head) pairs");
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  int32_t* act = scratch;
+  int32_t* cnt = scratch + n_cand;
+  if (n_cand > 0) {
+    FO_REQUIRE(row_req && row_qb && row_head && kv_idx, "decode: null output");
+    const int per_wg = kCountThreads / kWave;
+    const unsigned grid = static_cast<unsigned>((n_cand + per_wg - 1) / per_wg);
+    decode_count_kernel<<<grid, kCountThreads, 0, s>>>(
+        sparse_info, sparse_kv_info, sparse_info_indptr, sparse_kv_info_indptr, blk_req, blk_qb,
+        kv_indptr, n_cand, num_heads, block_kv, is_full, act, cnt);
+    FO_CHECK_LAUNCH();
+  }
+  decode_scan_kernel<<<1, kScanThreads, 0, s>>>(n_cand, act, cnt, kv_row_ptr, counts);
+  FO_CHECK_LAUNCH();
+  if (n_cand > 0) {
+    const int per_wg = kCountThreads / kWave;
+    const unsigned grid = static_cast<unsigned>((n_cand + per_wg - 1) / per_wg);
+    decode_fill_kernel<<<grid, kCountThreads, 0, s>>>(
+        sparse_info, sparse_kv_info, sparse_info_indptr, sparse_kv_info_indptr, blk_req, blk_qb,
+        kv_indptr, n_cand, num_heads, block_kv, is_full, act, cnt, row_req, row_qb, row_head,
+        kv_row_ptr, kv_idx);
+    FO_CHECK_LAUNCH();
+  }
+  return FO_OK;
+}

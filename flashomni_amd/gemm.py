@@ -1,0 +1,119 @@
+"""GEMM-Q (``flashomni_gemm``) and GEMM-O with reduction (``flashomni_gemm_reduction``).
+
+Signatures and defaults are those of the reference (flashomni/gemm.py:156-216); the work runs in
+hand-written MFMA kernels behind the C ABI (fo_gemm_q / fo_gemm_o)."""
+import torch
+
+from . import _lib
+from .utils import _require_gpu_tensor
+
+
+def _check_gemm_operands(A: torch.Tensor, B: torch.Tensor, name: str):
+    _require_gpu_tensor(A, "A")
+    _require_gpu_tensor(B, "B")
+    if A.dim() != 3 or B.dim() != 2:
+        # reference: csrc/gemm.cu:26-31
+        raise RuntimeError(f"{name}: A must be [B, M, K] and B must be [N, K]")
+    if A.shape[2] != B.shape[1]:
+        raise RuntimeError(f"{name}: K mismatch, A is {tuple(A.shape)} and B is {tuple(B.shape)}")
+    if A.dtype != B.dtype or A.dtype not in (torch.bfloat16, torch.float16):
+        raise RuntimeError(f"{name}: A and B must both be bfloat16 or float16")
+    if not (A.is_contiguous() and B.is_contiguous()):
+        raise RuntimeError(f"{name}: A and B must be contiguous")
+
+
+def _symbols(sparse_info, sparse_info_indptr, device):
+    if sparse_info is None:
+        return None, None
+    info = sparse_info.to(device=device, dtype=torch.uint8).contiguous()
+    indptr = sparse_info_indptr.to(device=device, dtype=torch.int32).contiguous()
+    return info, indptr
+
+
+def flashomni_gemm(
+    A: torch.Tensor,
+    B: torch.Tensor,
+    num_qo_heads: int,
+    sparse_info: torch.Tensor = None,
+    sparse_info_indptr: torch.Tensor = None,
+    num_text_tokens: int = 512,
+    bias: torch.Tensor = None,
+    out: torch.Tensor = None,
+    sparse_q_size: int = 128,
+    is_full: bool = False,
+) -> torch.Tensor:
+    """``out[b, tile] = A[b] @ B.T + bias`` for every (128-token block, 128-column) tile whose
+    ``sparse_info`` bit is 1; the other tiles of ``out`` are left untouched (a fresh ``out`` is
+    ``torch.empty``, as in the reference)."""
+    _check_gemm_operands(A, B, "flashomni_gemm")
+    if out is None:
+        out = torch.empty((A.shape[0], A.shape[1], B.shape[0]), device=A.device, dtype=A.dtype)
+    elif out.shape != (A.shape[0], A.shape[1], B.shape[0]) or out.dtype != A.dtype \
+            or not out.is_contiguous() or out.device != A.device:
+        raise RuntimeError("flashomni_gemm: out must be a contiguous [B, M, N] tensor of A's dtype")
+    if bias is not None:
+        if bias.dtype != A.dtype or bias.numel() != B.shape[0] or bias.device != A.device:
+            raise RuntimeError("flashomni_gemm: bias must be [N] with A's dtype on A's device")
+        bias = bias.contiguous()
+    info, indptr = _symbols(sparse_info, sparse_info_indptr, A.device)
+    if not is_full and info is None:
+        raise RuntimeError("flashomni_gemm: sparse_info is required unless is_full=True")
+    _lib.check(_lib.lib().fo_gemm_q(
+        _lib.ptr(A), _lib.ptr(B), _lib.ptr(bias), _lib.ptr(out), _lib.dtype_code(A.dtype),
+        A.shape[0], A.shape[1], B.shape[0], A.shape[2], sparse_q_size, num_qo_heads,
+        _lib.ptr(info), _lib.ptr(indptr), num_text_tokens, int(bool(is_full)),
+        _lib.current_stream(A.device)))
+    return out
+
+
+def flashomni_gemm_reduction(
+    A: torch.Tensor,
+    B: torch.Tensor,
+    num_qo_heads: int,
+    sparse_info: torch.Tensor,
+    sparse_info_indptr: torch.Tensor,
+    num_text_tokens: int,
+    bias: torch.Tensor = None,
+    is_for_cache: bool = False,
+    sparse_q_size: int = 128,
+    out_dtype: torch.dtype = None,
+) -> torch.Tensor:
+    """GEMM-O.  ``is_for_cache=True``: returns ``bias[N] + sum over cached heads (bit 0)`` of
+    ``A[:, :, head slice] @ B[:, head slice].T``.  ``is_for_cache=False``: ``bias`` is the cached
+    ``[B, M, N]`` partial and the heads with bit 1 are added to it.
+
+    ``out_dtype`` (extension; the reference always returns ``A.dtype``): pass ``torch.float32``
+    to keep the cached partial in fp32; the second call accepts an fp32 ``bias`` matrix."""
+    _check_gemm_operands(A, B, "flashomni_gemm_reduction")
+    if sparse_info is None or sparse_info_indptr is None:
+        raise RuntimeError("flashomni_gemm_reduction: sparse_info and sparse_info_indptr are required")
+    out_dtype = A.dtype if out_dtype is None else out_dtype
+    if out_dtype not in (A.dtype, torch.float32):
+        raise RuntimeError("flashomni_gemm_reduction: out_dtype must be A.dtype or float32")
+    Bsz, M, _ = A.shape
+    N = B.shape[0]
+    out = torch.empty((Bsz, M, N), device=A.device, dtype=out_dtype)
+    kind = _lib.FO_BIAS_NONE
+    bias_code = _lib.dtype_code(A.dtype)
+    if bias is not None:
+        if bias.device != A.device:
+            raise RuntimeError("flashomni_gemm_reduction: bias must be on A's device")
+        if is_for_cache:
+            if bias.numel() != N or bias.dtype != A.dtype:
+                raise RuntimeError("flashomni_gemm_reduction: with is_for_cache=True bias must be [N] "
+                                   "with A's dtype")
+            kind = _lib.FO_BIAS_VECTOR
+        else:
+            if bias.numel() != Bsz * M * N or bias.dtype not in (A.dtype, torch.float32):
+                raise RuntimeError("flashomni_gemm_reduction: with is_for_cache=False bias must be "
+                                   "the cached [B, M, N] partial (A's dtype or float32)")
+            kind = _lib.FO_BIAS_MATRIX
+            bias_code = _lib.dtype_code(bias.dtype)
+        bias = bias.contiguous()
+    info, indptr = _symbols(sparse_info, sparse_info_indptr, A.device)
+    _lib.check(_lib.lib().fo_gemm_o(
+        _lib.ptr(A), _lib.ptr(B), _lib.ptr(bias), _lib.ptr(out), _lib.dtype_code(A.dtype), kind,
+        bias_code, _lib.dtype_code(out_dtype), Bsz, M, N, A.shape[2], sparse_q_size, num_qo_heads,
+        _lib.ptr(info), _lib.ptr(indptr), num_text_tokens, int(bool(is_for_cache)),
+        _lib.current_stream(A.device)))
+    return out

@@ -1,0 +1,181 @@
+/*
+ * flashomni_hip.h -- C ABI of the MI355X (gfx950) FlashOmni sparse-attention engine.
+ *
+ * Plain pointers and sizes only; no torch types.  Every entry point that touches the GPU
+ * takes the HIP stream to enqueue on (a hipStream_t passed as void*; NULL = the null stream),
+ * never synchronises and never allocates device memory.  Return value: 0 on success, a
+ * negative FO_ERR_* code otherwise; fo_last_error() then holds a thread-local message.
+ *
+ * Each entry point names the reference interface it stands in for (paths are relative to the
+ * root of qiaolian9/FlashOmni).
+ */
+#ifndef FLASHOMNI_HIP_H_
+#define FLASHOMNI_HIP_H_
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define FO_ABI_VERSION 1
+
+enum {
+  FO_OK = 0,
+  FO_ERR_INVALID = -1,   /* bad argument / unsupported shape (reference: TORCH_CHECK failures) */
+  FO_ERR_WORKSPACE = -2, /* workspace too small (reference: AlignedAllocator overflow) */
+  FO_ERR_HIP = -3        /* a HIP runtime call failed (reference: cudaError_t return codes) */
+};
+
+/* element types of activations */
+enum { FO_BF16 = 0, FO_F16 = 1, FO_FP8_E4M3 = 2, FO_F32 = 3 };
+/* bit orders of packbits */
+enum { FO_BITORDER_BIG = 0, FO_BITORDER_LITTLE = 1 };
+/* kinds of the GEMM-O `bias` operand */
+enum { FO_BIAS_NONE = 0, FO_BIAS_VECTOR = 1, FO_BIAS_MATRIX = 2 };
+
+const char* fo_last_error(void);
+int fo_abi_version(void);
+/* number of compute units of the current device (0 if no device) */
+int fo_num_cu(void);
+
+/* ---------------------------------------------------------------------------------------------
+ * packbits / segment_packbits
+ * replaces: csrc/quantization.cu:22-36 (packbits), :38-57 (segment_packbits);
+ *           kernels include/flashomni/quantization.cuh:39-57, :59-83.
+ * x: n bool bytes (non-zero = 1) on the device; y: ceil(n/8) bytes.
+ * segment form: indptrs are int32 device arrays of num_segments+1 entries; segment i packs
+ * x[in_indptr[i] : in_indptr[i+1]] into y[out_indptr[i] : ...], starting on a byte boundary.
+ * ------------------------------------------------------------------------------------------- */
+int fo_packbits(const uint8_t* x, int64_t n, int bitorder, uint8_t* y, void* stream);
+int fo_segment_packbits(const uint8_t* x, const int32_t* in_indptr, const int32_t* out_indptr,
+                        int32_t num_segments, int bitorder, uint8_t* y, void* stream);
+
+/* ---------------------------------------------------------------------------------------------
+ * Host planner.
+ * replaces: BatchSparseFAWithKVPlan csrc/batch_sparseFA.cu:39-65 and PrefillPlan
+ *           include/flashomni/attention/scheduler.cuh:248-349 (+ :35-168, utils.cuh:293-312,
+ *           allocator.h:32-58).
+ * Pure host arithmetic: fills the pinned mirror `int_ws_host` with request_indices,
+ * qo_tile_indices, kv_tile_indices, o_indptr, kv_chunk_size (and merge_indptr,
+ * block_valid_mask when kv is split) at 16-byte aligned offsets and writes the 15-entry plan
+ * vector in the reference's order (scheduler.cuh:205-221).  When int_ws_dev is not NULL the
+ * used prefix is copied host->device on `stream`.  num_cu <= 0 queries the current device.
+ * ------------------------------------------------------------------------------------------- */
+int fo_prefill_plan(void* float_ws, size_t float_ws_bytes, void* int_ws_dev, void* int_ws_host,
+                    size_t int_ws_bytes, const int32_t* qo_indptr_host,
+                    const int32_t* kv_indptr_host, uint32_t total_num_rows, uint32_t batch_size,
+                    uint32_t num_qo_heads, uint32_t num_kv_heads, uint32_t head_dim_qk,
+                    uint32_t head_dim_vo, uint32_t page_size, int enable_graph,
+                    uint32_t sizeof_dtype_o, int num_cu, int64_t plan_info_out[15], void* stream);
+
+/* ---------------------------------------------------------------------------------------------
+ * Sparse-symbol decoder: packed symbols -> compacted, canonically ordered work list.
+ * replaces the per-CTA bit tests and bit walks of
+ *   include/flashomni/attention/prefill.cuh:1284-1294 (q-block flag),
+ *   :1380-1403 and :1434-1460 (next kept kv block).
+ *
+ * The q-block table (one entry per sparse q-block of every request, request-major) is built on
+ * the host by fo_sparse_block_table(); fo_decode_sizes() tells how large the outputs must be.
+ *
+ * Bit conventions: bit = 1 keep/compute; little-endian in a byte; sparse_info bit index inside
+ * request r is qb*H + h; sparse_kv_info bit index is (qb*H + h)*NKV_r + kvb with
+ * NKV_r = ceil(kv_len_r / block_kv); the two indptr arrays are BYTE offsets per request.
+ *
+ * Outputs (all int32, device):
+ *   row_req,row_qb,row_head [n_rows]  rows with flag 1, ascending (request, q-block, head)
+ *   kv_row_ptr [n_rows+1], kv_idx [nnz]  kept kv blocks of each row, ascending
+ *   counts[0] = n_rows, counts[1] = nnz, counts[2..3] = scratch counters cleared to 0
+ * is_full != 0 ignores the symbol tensors (which may be NULL) and lists everything
+ * (csrc/batch_sparseFA.cu:123-128).
+ * `scratch` needs 2*n_blk*H + 2 int32.
+ * ------------------------------------------------------------------------------------------- */
+int fo_sparse_block_table(const int32_t* qo_indptr_host, uint32_t batch_size, uint32_t block_q,
+                          int32_t* blk_req_host, int32_t* blk_qb_host, int64_t capacity,
+                          int64_t* n_blk_out);
+int fo_decode_sizes(const int32_t* qo_indptr_host, const int32_t* kv_indptr_host,
+                    uint32_t batch_size, uint32_t num_heads, uint32_t block_q, uint32_t block_kv,
+                    int64_t* n_blk_out, int64_t* max_rows_out, int64_t* max_nnz_out);
+int fo_decode_sparse(const uint8_t* sparse_info, const uint8_t* sparse_kv_info,
+                     const int32_t* sparse_info_indptr, const int32_t* sparse_kv_info_indptr,
+                     const int32_t* blk_req, const int32_t* blk_qb, const int32_t* kv_indptr,
+                     int32_t n_blk, int32_t num_heads, int32_t block_kv, int is_full,
+                     int32_t* row_req, int32_t* row_qb, int32_t* row_head, int32_t* kv_row_ptr,
+                     int32_t* kv_idx, int32_t* counts, int32_t* scratch, void* stream);
+
+/* ---------------------------------------------------------------------------------------------
+ * Ragged block-sparse FlashAttention prefill over a decoded work list.
+ * replaces: BatchSparseFAWithRaggedKVRun csrc/batch_sparseFA.cu:67-201 and the kernel
+ *           include/flashomni/attention/prefill.cuh:1203-1531 (mask none, no positional
+ *           encoding, fp32 logits: the only variant the reference builds, setup.py:98-111).
+ *
+ * q [nnz_q,H,D], k,v [nnz_kv,H,D], o [nnz_q,H,D]; strides in elements (the innermost stride is
+ * 1).  dtype FO_BF16 / FO_F16: q,k,v,o share it.  dtype FO_FP8_E4M3: q and k are e4m3fn bytes
+ * with dequantisation scales q_scale[H][n_q_blocks], k_scale[H][n_kv_blocks] (fp32, blocks
+ * numbered request by request); v and o are bf16.  (The fp8 form has no counterpart in the
+ * reference.)
+ * Rows of the list write every output row of their q-block; q-blocks not in the list are left
+ * untouched; a listed row with no kv block writes zeros and lse = -5e4.  lse (optional, fp32
+ * [nnz_q,H]) is base 2: log2(sum 2^(s*c - m*c)) + m*c, c = sm_scale*log2(e).
+ * Supported: D = 128, block_q = 128, block_kv = 128.  max_rows bounds counts[0].
+ * ------------------------------------------------------------------------------------------- */
+int fo_sparse_fa_run(const void* q, const void* k, const void* v, void* o, float* lse, int dtype,
+                     const float* q_scale, const float* k_scale, int64_t q_stride_n,
+                     int64_t q_stride_h, int64_t k_stride_n, int64_t k_stride_h,
+                     int64_t v_stride_n, int64_t v_stride_h, int64_t o_stride_n,
+                     int64_t o_stride_h, const int32_t* qo_indptr, const int32_t* kv_indptr,
+                     const int32_t* q_blk_base, const int32_t* kv_blk_base,
+                     const int32_t* row_req, const int32_t* row_qb, const int32_t* row_head,
+                     const int32_t* kv_row_ptr, const int32_t* kv_idx, int32_t* counts,
+                     int64_t max_rows, int32_t num_heads, int32_t head_dim, int32_t block_q,
+                     int32_t block_kv, float sm_scale, void* stream);
+
+/* ---------------------------------------------------------------------------------------------
+ * GEMM-Q: y[b, tile] = x[b] . w^T + bias for every (128-row, 128-column) tile whose symbol bit
+ * is 1; other tiles keep their bytes.
+ * replaces: FLASHOMNIGEMM csrc/gemm.cu:24-59, FLASHOMNIGEMMRun/kernel
+ *           include/flashomni/gemm/w16a16/gemm.cuh:27-228, :230-357.
+ * x [B,M,K], w [N,K], y [B,M,N] row-major contiguous; bias [N] or NULL; dtype FO_BF16/FO_F16.
+ * Tile (b, iy, ix) tests bit ((num_text_tokens + iy*128)/sparse_q_size)*num_qo_heads
+ * + (ix*128)/(N/num_qo_heads) of sparse_info + sparse_info_indptr[b] (gemm.cuh:50-58).
+ * Requires N % 128 == 0 and K % 32 == 0 (csrc/gemm.cu:36); M may have a tail (the reference
+ * demands M % 128 == 0).
+ * ------------------------------------------------------------------------------------------- */
+int fo_gemm_q(const void* x, const void* w, const void* bias, void* y, int dtype, int32_t batch,
+              int32_t m, int32_t n, int32_t k, int32_t sparse_q_size, int32_t num_qo_heads,
+              const uint8_t* sparse_info, const int32_t* sparse_info_indptr,
+              int32_t num_text_tokens, int is_full, void* stream);
+
+/* ---------------------------------------------------------------------------------------------
+ * GEMM-O with reduction: y[b, row-tile, :] = init + sum over selected head slices of
+ * x[:, h*hd:(h+1)*hd] . w[:, h*hd:(h+1)*hd]^T, hd = N/num_qo_heads.
+ * is_for_cached != 0 selects heads whose bit is 0 and init = bias vector [N];
+ * is_for_cached == 0 selects heads whose bit is 1 and init = bias matrix [B,M,N].
+ * replaces: FLASHOMNIGEMMReduction csrc/gemm_reduction.cu:24-57, kernel
+ *           include/flashomni/gemm/w16a16/gemm_reduction.cuh:27-276 (:77-95 init, :126-160
+ *           slice selection).
+ * bias_dtype: the activation dtype (as in the reference) or FO_F32 for the matrix form;
+ * y_dtype: the activation dtype or FO_F32 (so a cached partial can stay in fp32).
+ * ------------------------------------------------------------------------------------------- */
+int fo_gemm_o(const void* x, const void* w, const void* bias, void* y, int dtype, int bias_kind,
+              int bias_dtype, int y_dtype, int32_t batch, int32_t m, int32_t n, int32_t k,
+              int32_t sparse_q_size, int32_t num_qo_heads, const uint8_t* sparse_info,
+              const int32_t* sparse_info_indptr, int32_t num_text_tokens, int is_for_cached,
+              void* stream);
+
+/* ---------------------------------------------------------------------------------------------
+ * fp8 e4m3fn quantiser with one absmax scale per (head, 128-token block).
+ * No counterpart in the reference (its quantization.cuh only packs bits).
+ * x [nnz,H,D] bf16/f16 (strides in elements), x8 [nnz,H,D] bytes contiguous,
+ * scale fp32 [H][n_blk]: scale = absmax/448 (1 for an all-zero block), x8 = rne(x/scale).
+ * blk_req/blk_tok0/blk_len (int32 [n_blk], device): request, first token and length of each block.
+ * ------------------------------------------------------------------------------------------- */
+int fo_quant_fp8_block(const void* x, int dtype, int64_t x_stride_n, int64_t x_stride_h,
+                       uint8_t* x8, float* scale, const int32_t* blk_tok0, const int32_t* blk_len,
+                       int32_t n_blk, int32_t num_heads, int32_t head_dim, void* stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* FLASHOMNI_HIP_H_ */

@@ -1,0 +1,157 @@
+"""GPU parity: sparse FlashAttention through the wrapper vs the fp32 dense masked oracle.
+
+Tolerances are those stated for the path: bf16/fp16 outputs within max-abs 2e-2 and relative L2
+1e-2 of the fp32 reference; skipped q-blocks byte-identical; listed rows without kv blocks zero."""
+import math
+
+import numpy as np
+import pytest
+import torch
+
+import oracle
+from helpers import make_ragged_masks, max_abs, rel_l2, sentinel_like
+
+pytestmark = pytest.mark.gpu
+
+MAX_ABS, REL_L2 = 2e-2, 1e-2
+
+
+def _run_case(dev, ql, kl, heads, dtype, seed, pa=0.75, pk=0.5, force=None, is_full=False,
+              return_lse=False, layout="NHD"):
+    import flashomni_amd as fo
+    m = make_ragged_masks(ql, kl, heads, pa, pk, seed=seed, force=force)
+    g = torch.Generator().manual_seed(seed)
+    nq, nk = int(m["qo_indptr"][-1]), int(m["kv_indptr"][-1])
+    q = torch.randn(nq, heads, 128, generator=g).to(dtype)
+    k = torch.randn(nk, heads, 128, generator=g).to(dtype)
+    v = torch.randn(nk, heads, 128, generator=g).to(dtype)
+    out0 = sentinel_like((nq, heads, 128), dtype)
+    t = lambda a: torch.from_numpy(a).to(dev)
+    ws = torch.empty(128 << 20, dtype=torch.uint8, device=dev)
+    w = fo.BatchFlashOmniFAWithRaggedKVWrapper(ws, layout)
+    w.plan(t(m["qo_indptr"]), t(m["kv_indptr"]), heads, heads, 128, q_data_type=dtype)
+    kd, vd = k.to(dev), v.to(dev)
+    if layout == "HND":
+        kd, vd = kd.transpose(0, 1).contiguous(), vd.transpose(0, 1).contiguous()
+    out = out0.clone().to(dev)
+    res = w.run(q.to(dev), kd, vd, t(m["packed_info"]), t(m["packed_keep"]), t(m["info_indptr"]),
+                t(m["keep_indptr"]), is_full, out=out, return_lse=return_lse)
+    lse = None
+    if return_lse:
+        res, lse = res
+    assert res.data_ptr() == out.data_ptr()
+    exp_lse = torch.full((nq, heads), float("nan")) if return_lse else None
+    exp = oracle.sparse_attention(q, k, v, m["packed_info"], m["packed_keep"], m["info_indptr"],
+                                  m["keep_indptr"], m["qo_indptr"], m["kv_indptr"], is_full=is_full,
+                                  out=out0.clone(), lse=exp_lse)
+    return out.cpu(), exp, out0, m, (lse.cpu() if lse is not None else None), exp_lse
+
+
+def _check(out, exp, out0, m, heads, is_full=False):
+    # untouched q-blocks: byte-identical to the sentinel
+    touched = torch.zeros(out.shape[:2], dtype=torch.bool)
+    for r, info in enumerate(m["info"]):
+        q0 = int(m["qo_indptr"][r])
+        q1 = int(m["qo_indptr"][r + 1])
+        for qb in range(info.shape[0]):
+            for h in range(heads):
+                if is_full or info[qb, h]:
+                    touched[q0 + qb * 128:min(q1, q0 + (qb + 1) * 128), h] = True
+    assert torch.equal(out[~touched].view(torch.int16), out0[~touched].view(torch.int16))
+    assert torch.equal(exp[~touched].view(torch.int16), out0[~touched].view(torch.int16))
+    if touched.any():
+        assert max_abs(out[touched], exp[touched]) <= MAX_ABS
+        assert rel_l2(out[touched], exp[touched]) <= REL_L2
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+def test_small_single_request(dev, dtype):
+    out, exp, out0, m, _, _ = _run_case(dev, [512], [512], 2, dtype, seed=1)
+    _check(out, exp, out0, m, 2)
+
+
+@pytest.mark.parametrize("layout", ["NHD", "HND"])
+def test_ragged_batch_with_tails(dev, layout):
+    ql, kl = [300, 1, 128, 1000, 129], [77, 513, 128, 1100, 64]
+    out, exp, out0, m, _, _ = _run_case(dev, ql, kl, 3, torch.bfloat16, seed=2, layout=layout)
+    _check(out, exp, out0, m, 3)
+
+
+def test_all_ones_matches_sdpa(dev):
+    """is_full and an all-ones mask both reduce to plain dense attention (a library routine)."""
+    heads = 2
+    for kwargs in (dict(force="ones"), dict(is_full=True)):
+        out, exp, out0, m, _, _ = _run_case(dev, [384], [640], heads, torch.bfloat16, seed=3, **kwargs)
+        _check(out, exp, out0, m, heads, is_full=True)
+
+
+def test_all_cached_leaves_output_untouched(dev):
+    out, exp, out0, m, _, _ = _run_case(dev, [384], [384], 2, torch.bfloat16, seed=4, force="zeros")
+    assert torch.equal(out.view(torch.int16), out0.view(torch.int16))
+
+
+def test_active_row_without_kv_blocks_writes_zeros_and_lse(dev):
+    out, exp, out0, m, lse, exp_lse = _run_case(dev, [256], [256], 2, torch.bfloat16, seed=5, pa=1.0,
+                                                pk=0.0, return_lse=True)
+    assert float(out.abs().max()) == 0.0
+    assert torch.equal(lse, torch.full_like(lse, -5e4))
+
+
+def test_lse_base2(dev):
+    out, exp, out0, m, lse, exp_lse = _run_case(dev, [300, 200], [500, 130], 2, torch.bfloat16, seed=6,
+                                                pa=0.8, pk=0.6, return_lse=True)
+    _check(out, exp, out0, m, 2)
+    ok = ~torch.isnan(exp_lse)
+    assert ok.any()
+    assert float((lse[ok] - exp_lse[ok]).abs().max()) < 2e-2
+
+
+def test_default_out_is_zero_filled(dev):
+    import flashomni_amd as fo
+    heads = 2
+    m = make_ragged_masks([256], [256], heads, 0.5, 0.5, seed=11)
+    t = lambda a: torch.from_numpy(a).to(dev)
+    q = torch.randn(256, heads, 128, device=dev, dtype=torch.bfloat16)
+    w = fo.BatchFlashOmniFAWithRaggedKVWrapper(torch.empty(128 << 20, dtype=torch.uint8, device=dev))
+    w.plan(t(m["qo_indptr"]), t(m["kv_indptr"]), heads, heads, 128, q_data_type=torch.bfloat16)
+    out = w.run(q, q, q, t(m["packed_info"]), t(m["packed_keep"]), t(m["info_indptr"]), t(m["keep_indptr"]))
+    for qb in range(2):
+        for h in range(heads):
+            if not m["info"][0][qb, h]:
+                assert float(out[qb * 128:(qb + 1) * 128, h].abs().max()) == 0.0
+
+
+def test_flux_shape_full_config(dev):
+    """Config 0 at full size (H=24, seq 4608): every active row checked against the oracle."""
+    import flashomni_amd as fo
+    from flashomni_amd.workloads import make_workload, sm_scale
+    wl = make_workload(0)
+    q, k, v = wl.tensors["q"], wl.tensors["k"], wl.tensors["v"]
+    out0 = sentinel_like(q.shape, torch.bfloat16)
+    w = fo.BatchFlashOmniFAWithRaggedKVWrapper(torch.empty(128 << 20, dtype=torch.uint8, device=dev))
+    w.plan(wl.qo_indptr, wl.kv_indptr, 24, 24, 128, q_data_type=torch.bfloat16)
+    out = out0.clone().to(dev)
+    w.run(q.to(dev), k.to(dev), v.to(dev), wl.packed_info.to(dev), wl.packed_kv_info.to(dev),
+          wl.info_indptr.to(dev), wl.kv_info_indptr.to(dev), out=out)
+    exp = oracle.sparse_attention(q, k, v, wl.packed_info, wl.packed_kv_info, wl.info_indptr,
+                                  wl.kv_info_indptr, wl.qo_indptr, wl.kv_indptr, out=out0.clone())
+    out = out.cpu()
+    active = wl.sparse_info.repeat_interleave(128, dim=0)[:4608]       # [seq, H]
+    assert torch.equal(out[~active].view(torch.int16), out0[~active].view(torch.int16))
+    assert max_abs(out[active], exp[active]) <= MAX_ABS
+    assert rel_l2(out[active], exp[active]) <= REL_L2
+
+
+def test_dtype_mismatch_and_missing_symbols_raise(dev):
+    import flashomni_amd as fo
+    w = fo.BatchFlashOmniFAWithRaggedKVWrapper(torch.empty(128 << 20, dtype=torch.uint8, device=dev))
+    ip = torch.tensor([0, 128], dtype=torch.int32, device=dev)
+    w.plan(ip, ip, 1, 1, 128, q_data_type=torch.bfloat16)
+    q = torch.zeros(128, 1, 128, device=dev, dtype=torch.float16)
+    with pytest.raises(ValueError, match="does not match the q_data_type"):
+        w.run(q, q, q, is_full=True)
+    q = q.to(torch.bfloat16)
+    with pytest.raises(ValueError, match="required unless"):
+        w.run(q, q, q)
+    with pytest.raises(ValueError, match="Invalid shape of out"):
+        w.run(q, q, q, is_full=True, out=torch.zeros(64, 1, 128, device=dev, dtype=torch.bfloat16))

@@ -1,0 +1,166 @@
+"""GPU parity: GEMM-Q / GEMM-O vs the fp32 masked-GEMM oracle.
+
+bf16/fp16 outputs: max-abs <= 2e-2 and relative L2 <= 1e-2 of the fp32 reference; tiles whose flag
+is 0 keep their bytes (GEMM-Q)."""
+import numpy as np
+import pytest
+import torch
+import torch.nn.functional as F
+
+import oracle
+from helpers import max_abs, rel_l2, sentinel_like
+
+pytestmark = pytest.mark.gpu
+
+MAX_ABS, REL_L2 = 2e-2, 1e-2
+
+
+def _flags(batch, n_qblocks, heads, p, seed):
+    rng = np.random.default_rng(seed)
+    info = rng.random((batch, n_qblocks, heads)) < p
+    segs = [np.packbits(info[b].reshape(-1).astype(np.uint8), bitorder="little") for b in range(batch)]
+    indptr = np.zeros(batch + 1, dtype=np.int32)
+    indptr[1:] = np.cumsum([len(s) for s in segs])
+    return info, np.concatenate(segs), indptr
+
+
+def _operands(batch, m, n, k, dtype, seed, bias=True):
+    g = torch.Generator().manual_seed(seed)
+    x = torch.randn(batch, m, k, generator=g).to(dtype)
+    w = (torch.randn(n, k, generator=g) * 0.02).to(dtype)
+    b = (torch.randn(n, generator=g) * 0.02).to(dtype) if bias else None
+    return x, w, b
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("shape", [(1, 512, 384, 256, 3, 0), (2, 256, 256, 96, 2, 0),
+                                   (1, 1024, 256, 512, 2, 512), (1, 300, 256, 128, 2, 0)])
+def test_gemm_q_matches_oracle_and_skips_tiles(dev, dtype, shape):
+    import flashomni_amd as fo
+    batch, m, n, k, heads, text = shape
+    nqb = (text + m + 127) // 128
+    info, packed, indptr = _flags(batch, nqb, heads, 0.6, seed=m + n)
+    x, w, b = _operands(batch, m, n, k, dtype, seed=k)
+    out0 = sentinel_like((batch, m, n), dtype)
+    out = out0.clone().to(dev)
+    res = fo.flashomni_gemm(x.to(dev), w.to(dev), heads, torch.from_numpy(packed).to(dev),
+                            torch.from_numpy(indptr).to(dev), text, b.to(dev), out=out)
+    assert res.data_ptr() == out.data_ptr()
+    exp = oracle.gemm_q(x, w, heads, packed, indptr, text, b, out=out0.clone())
+    out = out.cpu()
+    changed = (exp.view(torch.int16) != out0.view(torch.int16))
+    # skipped tiles byte-identical
+    hd = n // heads
+    for bi in range(batch):
+        for iy in range((m + 127) // 128):
+            for ix in range(n // 128):
+                bit = info[bi, (text + iy * 128) // 128, (ix * 128) // hd]
+                tile = (bi, slice(iy * 128, min(m, (iy + 1) * 128)), slice(ix * 128, (ix + 1) * 128))
+                if not bit:
+                    assert torch.equal(out[tile].view(torch.int16), out0[tile].view(torch.int16))
+    assert max_abs(out, exp) <= MAX_ABS
+    assert rel_l2(out[changed], exp[changed]) <= REL_L2
+
+
+def test_gemm_q_is_full_equals_linear(dev):
+    import flashomni_amd as fo
+    x, w, b = _operands(1, 384, 256, 192, torch.bfloat16, seed=9)
+    out = fo.flashomni_gemm(x.to(dev), w.to(dev), 2, bias=b.to(dev), is_full=True).cpu()
+    exp = F.linear(x.float(), w.float(), b.float())
+    assert max_abs(out, exp) <= MAX_ABS and rel_l2(out, exp) <= REL_L2
+
+
+def test_gemm_q_shape_errors(dev):
+    import flashomni_amd as fo
+    x, w, b = _operands(1, 128, 192, 64, torch.bfloat16, seed=1)
+    with pytest.raises(RuntimeError, match="only support"):
+        fo.flashomni_gemm(x.to(dev), w.to(dev), 1, is_full=True)
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("use_bias", [False, True])
+@pytest.mark.parametrize("shape", [(1, 512, 384, 3, 0), (2, 256, 256, 2, 0), (1, 300, 512, 4, 0)])
+def test_gemm_o_two_pass_protocol(dev, dtype, use_bias, shape):
+    """cache pass, then final pass fed with the cached partial: each pass matches its oracle and the
+    end result equals the dense linear layer (the identity the reference's own script checks,
+    benchmark/test_flashomni_gemm_o.py:72-86)."""
+    import flashomni_amd as fo
+    batch, m, n, heads, text = shape
+    k = n
+    nqb = (text + m + 127) // 128
+    info, packed, indptr = _flags(batch, nqb, heads, 0.5, seed=m)
+    x, w, b = _operands(batch, m, n, k, dtype, seed=n, bias=use_bias)
+    pk, ip = torch.from_numpy(packed).to(dev), torch.from_numpy(indptr).to(dev)
+    xd, wd = x.to(dev), w.to(dev)
+    cache = fo.flashomni_gemm_reduction(xd, wd, heads, pk, ip, text, bias=b.to(dev) if use_bias else None,
+                                        is_for_cache=True)
+    exp_cache = oracle.gemm_o(x, w, heads, packed, indptr, text, bias=b, is_for_cache=True)
+    assert cache.dtype == dtype
+    assert max_abs(cache.cpu(), exp_cache) <= MAX_ABS
+    final = fo.flashomni_gemm_reduction(xd, wd, heads, pk, ip, text, bias=cache, is_for_cache=False)
+    exp_final = oracle.gemm_o(x, w, heads, packed, indptr, text, bias=cache.cpu(), is_for_cache=False)
+    assert max_abs(final.cpu(), exp_final) <= MAX_ABS
+    assert rel_l2(final.cpu(), exp_final) <= REL_L2
+    dense = F.linear(x.float(), w.float(), b.float() if use_bias else None)
+    assert rel_l2(final.cpu(), dense) <= REL_L2
+    # fp32 partial keeps the whole chain within the max-abs budget
+    cache32 = fo.flashomni_gemm_reduction(xd, wd, heads, pk, ip, text, bias=b.to(dev) if use_bias else None,
+                                          is_for_cache=True, out_dtype=torch.float32)
+    assert cache32.dtype == torch.float32
+    final32 = fo.flashomni_gemm_reduction(xd, wd, heads, pk, ip, text, bias=cache32, is_for_cache=False)
+    assert max_abs(final32.cpu(), dense) <= MAX_ABS
+
+
+def test_gemm_o_extreme_masks(dev):
+    """all-ones flags: the cache pass returns the broadcast bias and the final pass the full linear
+    layer; all-zero flags: the reverse."""
+    import flashomni_amd as fo
+    x, w, b = _operands(1, 256, 256, 256, torch.bfloat16, seed=4)
+    heads = 2
+    ip = torch.tensor([0, 1], dtype=torch.int32, device=dev)
+    dense = F.linear(x.float(), w.float(), b.float())
+    for byte, cache_is_bias in ((0xFF, True), (0x00, False)):
+        pk = torch.tensor([byte], dtype=torch.uint8, device=dev)
+        cache = fo.flashomni_gemm_reduction(x.to(dev), w.to(dev), heads, pk, ip, 0, bias=b.to(dev),
+                                            is_for_cache=True).cpu()
+        if cache_is_bias:
+            assert torch.equal(cache, b[None, None, :].expand_as(cache))
+        else:
+            assert rel_l2(cache, dense) <= REL_L2
+        final = fo.flashomni_gemm_reduction(x.to(dev), w.to(dev), heads, pk, ip, 0,
+                                            bias=cache.to(dev), is_for_cache=False).cpu()
+        assert rel_l2(final, dense) <= REL_L2
+
+
+def test_flux_gemm_q_full_config(dev):
+    import flashomni_amd as fo
+    from flashomni_amd.workloads import make_workload
+    wl = make_workload(1)
+    x, w, b = wl.tensors["x"], wl.tensors["w"], wl.tensors["bias"]
+    out0 = sentinel_like((1, 4608, 3072), torch.bfloat16)
+    out = out0.clone().to(dev)
+    fo.flashomni_gemm(x.to(dev), w.to(dev), 24, wl.packed_info.to(dev), wl.info_indptr.to(dev), 0,
+                      b.to(dev), out=out)
+    out = out.cpu()
+    exp = oracle.gemm_q(x, w, 24, wl.packed_info, wl.info_indptr, 0, b, out=out0.clone())
+    active = wl.sparse_info.repeat_interleave(128, 0).repeat_interleave(128, 1)[None]
+    assert torch.equal(out[~active].view(torch.int16), out0[~active].view(torch.int16))
+    assert max_abs(out[active], exp[active]) <= MAX_ABS
+    assert rel_l2(out[active], exp[active]) <= REL_L2
+
+
+def test_flux_gemm_o_full_config(dev):
+    import flashomni_amd as fo
+    from flashomni_amd.workloads import make_workload
+    wl = make_workload(2)
+    a, w, b = wl.tensors["a"], wl.tensors["w"], wl.tensors["bias"]
+    pk, ip = wl.packed_info.to(dev), wl.info_indptr.to(dev)
+    cache = fo.flashomni_gemm_reduction(a.to(dev), w.to(dev), 24, pk, ip, 0, bias=b.to(dev),
+                                        is_for_cache=True, out_dtype=torch.float32)
+    final = fo.flashomni_gemm_reduction(a.to(dev), w.to(dev), 24, pk, ip, 0, bias=cache,
+                                        is_for_cache=False).cpu()
+    exp_cache = oracle.gemm_o(a, w, 24, wl.packed_info, wl.info_indptr, 0, bias=b, is_for_cache=True,
+                              out_dtype=torch.float32)
+    assert max_abs(cache.cpu(), exp_cache) <= 1e-3
+    dense = F.linear(a.float(), w.float(), b.float())
+    assert max_abs(final, dense) <= MAX_ABS and rel_l2(final, dense) <= REL_L2

@@ -1,0 +1,110 @@
+"""GPU parity: packbits / segment_packbits / sparse-symbol decoder vs the oracle (bit-exact)."""
+import numpy as np
+import pytest
+import torch
+
+import oracle
+from helpers import make_ragged_masks
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.mark.parametrize("n", [0, 1, 7, 8, 9, 64, 1000, 31104, 1 << 20])
+@pytest.mark.parametrize("bitorder", ["big", "little"])
+def test_packbits_matches_oracle(dev, n, bitorder):
+    import flashomni_amd as fo
+    rng = np.random.default_rng(n + 1)
+    x = rng.random(n) < 0.5
+    y = fo.packbits(torch.from_numpy(x).to(dev), bitorder)
+    assert y.dtype == torch.uint8 and y.numel() == (n + 7) // 8
+    np.testing.assert_array_equal(y.cpu().numpy(), oracle.packbits(x, bitorder))
+
+
+def test_packbits_docstring_vectors(dev):
+    import flashomni_amd as fo
+    x = torch.tensor([1, 0, 1, 1, 0, 0, 1, 1], dtype=torch.bool, device=dev)
+    assert fo.packbits(x).tolist() == [0b10110011]
+    x = torch.tensor([1, 0, 1, 1, 0, 0, 1, 1, 1, 0, 1], dtype=torch.bool, device=dev)
+    y, p = fo.segment_packbits(x, torch.tensor([0, 4, 7, 11], device=dev), bitorder="big")
+    assert y.tolist() == [0b10110000, 0b100000, 0b11010000]
+    assert p.tolist() == [0, 1, 2, 3]
+
+
+def test_packbits_nonbool_input_and_bad_bitorder(dev):
+    import flashomni_amd as fo
+    x = torch.tensor([3, 0, 255, 0, 0, 0, 0, 1, 2], dtype=torch.uint8, device=dev)
+    assert fo.packbits(x, "little").tolist() == [0b10000101, 0b1]
+    with pytest.raises(RuntimeError, match="bitorder must be 'big' or 'little'"):
+        fo.packbits(x, "middle")
+
+
+@pytest.mark.parametrize("bitorder", ["big", "little"])
+def test_segment_packbits_ragged(dev, bitorder):
+    import flashomni_amd as fo
+    rng = np.random.default_rng(5)
+    lens = [0, 1, 8, 13, 4000, 0, 77, 31104]
+    indptr = np.zeros(len(lens) + 1, dtype=np.int32)
+    indptr[1:] = np.cumsum(lens)
+    x = rng.random(indptr[-1]) < 0.4
+    y, p = fo.segment_packbits(torch.from_numpy(x).to(dev), torch.from_numpy(indptr).to(dev), bitorder)
+    ey, ep = oracle.segment_packbits(x, indptr, bitorder)
+    np.testing.assert_array_equal(p.cpu().numpy(), ep)
+    np.testing.assert_array_equal(y.cpu().numpy(), ey)
+
+
+def _decode_on_gpu(dev, m, heads, is_full=False):
+    import flashomni_amd as fo
+    ws = torch.empty(128 << 20, dtype=torch.uint8, device=dev)
+    w = fo.BatchFlashOmniFAWithRaggedKVWrapper(ws)
+    w.plan(torch.from_numpy(m["qo_indptr"]), torch.from_numpy(m["kv_indptr"]), heads, heads, 128,
+           q_data_type=torch.bfloat16)
+    t = lambda a: torch.from_numpy(a).to(dev)
+    wl = w.decode(t(m["packed_info"]), t(m["packed_keep"]), t(m["info_indptr"]), t(m["keep_indptr"]),
+                  is_full)
+    return [a.numpy() for a in wl.to_host()]
+
+
+CASES = [
+    ([4608], [4608], 24, 0.75, 0.5),                 # FLUX shape
+    ([300, 1, 128, 1000], [77, 513, 128, 4096], 3, 0.6, 0.3),   # ragged, NKV not multiple of 8
+    ([129], [128 * 67 + 5], 5, 0.9, 0.02),           # long rows crossing many bytes
+    ([256, 256], [256, 256], 1, 0.5, 0.5),
+]
+
+
+@pytest.mark.parametrize("case", CASES)
+@pytest.mark.parametrize("force", [None, "ones", "zeros"])
+def test_decoder_matches_bruteforce(dev, case, force):
+    ql, kl, heads, pa, pk = case
+    m = make_ragged_masks(ql, kl, heads, pa, pk, seed=len(ql) + heads, force=force)
+    got = _decode_on_gpu(dev, m, heads)
+    exp = oracle.decode_kv_csr(m["packed_info"], m["packed_keep"], m["info_indptr"],
+                               m["keep_indptr"], m["qo_indptr"], m["kv_indptr"], heads, 128, 128)
+    for g, e, name in zip(got, exp, ["row_req", "row_qb", "row_head", "kv_row_ptr", "kv_idx"]):
+        np.testing.assert_array_equal(g, e, err_msg=name)
+
+
+def test_decoder_is_full_lists_everything(dev):
+    ql, kl, heads = [300, 128], [500, 64], 2
+    m = make_ragged_masks(ql, kl, heads, 0.5, 0.5, seed=3)
+    got = _decode_on_gpu(dev, m, heads, is_full=True)
+    exp = oracle.decode_kv_csr(None, None, None, None, m["qo_indptr"], m["kv_indptr"], heads, 128, 128,
+                               is_full=True)
+    for g, e in zip(got, exp):
+        np.testing.assert_array_equal(g, e)
+
+
+@pytest.mark.parametrize("index", [3, 4])
+def test_decoder_full_size_configs(dev, index):
+    """Hunyuan / Wan shaped masks at full size: bit-exact against the brute-force enumeration."""
+    from flashomni_amd.workloads import make_workload
+    wl = make_workload(index, tensors=False)
+    m = dict(packed_info=wl.packed_info.numpy(), packed_keep=wl.packed_kv_info.numpy(),
+             info_indptr=wl.info_indptr.numpy(), keep_indptr=wl.kv_info_indptr.numpy(),
+             qo_indptr=wl.qo_indptr.numpy(), kv_indptr=wl.kv_indptr.numpy())
+    got = _decode_on_gpu(dev, m, wl.shape.heads)
+    exp = oracle.decode_kv_csr(m["packed_info"], m["packed_keep"], m["info_indptr"], m["keep_indptr"],
+                               m["qo_indptr"], m["kv_indptr"], wl.shape.heads, 128, 128)
+    for g, e in zip(got, exp):
+        np.testing.assert_array_equal(g, e)
+    assert len(got[0]) == wl.active_rows and len(got[4]) == wl.computed_blocks
