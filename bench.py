@@ -1,0 +1,322 @@
+#!/usr/bin/env python3
+"""Benchmark of the sparse-attention hot path on one MI355X.
+
+One *step* is one sparse pass of a FLUX-shaped layer (configs 0-2 of the baseline):
+GEMM-Q over the flagged (token-block, head) tiles -> symbol decode + block-sparse FlashAttention
+-> GEMM-O that adds the non-cached heads to the cached partial.  ``value`` is the effective
+TFLOP/s of that chain, counting only computed blocks / tiles / head slices.
+
+The JSON line also carries
+  * ``kernels``: per-kernel latency and effective TFLOP/s (or GB/s) for every config, each as a
+    fraction of the MI355X peak that bounds it,
+  * ``roofline``: the dominant kernel (sparse FlashAttention at the FLUX shape) measured with HIP
+    events on the launch stream,
+  * ``cpu_baseline``: the fp32 dense-masked CPU path (the oracle) timed on this box's host cores.
+
+Usage: python bench.py [--gpus 1] [--steps K] [--warmup W] [--configs 0,1,2,3,4] [--no-cpu]
+"""
+import argparse
+import json
+import os
+import sys
+import time
+
+import torch
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+
+PEAK_BF16 = 2516.6   # TFLOP/s dense
+PEAK_FP8 = 5033.2
+PEAK_HBM = 8000.0    # GB/s
+
+
+def log(*a):
+    print(*a, file=sys.stderr, flush=True)
+
+
+def time_gpu(fn, iters, warmup):
+    """Average milliseconds per call, HIP events on the current stream."""
+    for _ in range(warmup):
+        fn()
+    torch.cuda.synchronize()
+    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    e0.record()
+    for _ in range(iters):
+        fn()
+    e1.record()
+    e1.synchronize()
+    return e0.elapsed_time(e1) / iters
+
+
+def entry(ms, flops=None, nbytes=None, peak=None):
+    d = {"ms": round(ms, 5)}
+    if flops is not None:
+        d["tflops"] = round(flops / (ms * 1e-3) / 1e12, 2)
+        d["frac_of_peak"] = round(d["tflops"] / (peak or PEAK_BF16), 4)
+    if nbytes is not None:
+        d["gbps"] = round(nbytes / (ms * 1e-3) / 1e9, 2)
+        d["frac_of_peak"] = round(d["gbps"] / PEAK_HBM, 4)
+    return d
+
+
+class FluxLayer:
+    """Configs 0-2 on the device + the wrappers needed to run the chain."""
+
+    def __init__(self, dev):
+        import flashomni_amd as fo
+        from flashomni_amd.workloads import make_workload
+        self.fo = fo
+        self.w0, self.w1, self.w2 = make_workload(0), make_workload(1), make_workload(2)
+        d = lambda t: t.to(dev)
+        self.q, self.k, self.v = (d(self.w0.tensors[n]) for n in "qkv")
+        self.x, self.wq, self.bq = d(self.w1.tensors["x"]), d(self.w1.tensors["w"]), d(self.w1.tensors["bias"])
+        self.a, self.wo, self.bo = d(self.w2.tensors["a"]), d(self.w2.tensors["w"]), d(self.w2.tensors["bias"])
+        self.info, self.kv_info = d(self.w0.packed_info), d(self.w0.packed_kv_info)
+        self.info_ip, self.kv_ip = d(self.w0.info_indptr), d(self.w0.kv_info_indptr)
+        self.ws = torch.empty(128 << 20, dtype=torch.uint8, device=dev)
+        self.wrapper = fo.BatchFlashOmniFAWithRaggedKVWrapper(self.ws)
+        self.wrapper.plan(self.w0.qo_indptr, self.w0.kv_indptr, 24, 24, 128, q_data_type=torch.bfloat16)
+        self.out_q = torch.zeros(1, 4608, 3072, dtype=torch.bfloat16, device=dev)
+        self.out_fa = torch.zeros(4608, 24, 128, dtype=torch.bfloat16, device=dev)
+        self.cache = fo.flashomni_gemm_reduction(self.a, self.wo, 24, self.info, self.info_ip, 0,
+                                                 bias=self.bo, is_for_cache=True)
+
+    def gemm_q(self):
+        return self.fo.flashomni_gemm(self.x, self.wq, 24, self.info, self.info_ip, 0, self.bq,
+                                      out=self.out_q)
+
+    def decode(self):
+        self.wrapper._decode_key = None
+        return self.wrapper.decode(self.info, self.kv_info, self.info_ip, self.kv_ip)
+
+    def attention(self, fresh_decode=True):
+        if fresh_decode:
+            self.wrapper._decode_key = None
+        return self.wrapper.run(self.q, self.k, self.v, self.info, self.kv_info, self.info_ip,
+                                self.kv_ip, out=self.out_fa)
+
+    def gemm_o_cache(self):
+        return self.fo.flashomni_gemm_reduction(self.a, self.wo, 24, self.info, self.info_ip, 0,
+                                                bias=self.bo, is_for_cache=True)
+
+    def gemm_o_final(self):
+        return self.fo.flashomni_gemm_reduction(self.a, self.wo, 24, self.info, self.info_ip, 0,
+                                                bias=self.cache, is_for_cache=False)
+
+    def step(self):
+        self.gemm_q()
+        self.attention(fresh_decode=True)
+        self.gemm_o_final()
+
+    def chain_flops(self):
+        return self.w1.gemm_q_flops() + self.w0.attention_flops() + self.w2.gemm_o_flops(False)
+
+
+def bench_big_attention(dev, index, iters, warmup):
+    """Configs 3 / 4 attention at full size (tensors drawn on the GPU: the CPU draw of 10^9 normals
+    would dominate the run; masks are the seeded CPU ones)."""
+    import flashomni_amd as fo
+    from flashomni_amd.workloads import make_workload
+    wl = make_workload(index, tensors=False)
+    s = wl.shape
+    g = torch.Generator(device=dev).manual_seed(1000 + index)
+    mk = lambda: torch.randn(s.seq, s.heads, 128, generator=g, device=dev, dtype=torch.float32).to(torch.bfloat16)
+    q, k, v = mk(), mk(), mk()
+    ws = torch.empty(128 << 20, dtype=torch.uint8, device=dev)
+    w = fo.BatchFlashOmniFAWithRaggedKVWrapper(ws)
+    w.plan(wl.qo_indptr, wl.kv_indptr, s.heads, s.heads, 128, q_data_type=torch.bfloat16)
+    args = [t.to(dev) for t in (wl.packed_info, wl.packed_kv_info, wl.info_indptr, wl.kv_info_indptr)]
+    out = torch.zeros_like(q)
+
+    def dec():
+        w._decode_key = None
+        w.decode(*args)
+
+    res = {}
+    ms = time_gpu(dec, iters, warmup)
+    rows, nnz = w._worklist.sizes()
+    dec_bytes = wl.packed_info.numel() + wl.packed_kv_info.numel() + 4 * (4 * rows + 1 + nnz)
+    res["decode"] = entry(ms, nbytes=dec_bytes)
+    res["decode"]["rows"], res["decode"]["kv_blocks"] = rows, nnz
+    ms = time_gpu(lambda: w.run(q, k, v, *args, out=out), iters, warmup)
+    res["sparse_fa_bf16"] = entry(ms, flops=wl.attention_flops())
+    res["sparse_fa_bf16"]["computed_blocks"] = wl.computed_blocks
+    del q, k, v, out
+    torch.cuda.empty_cache()
+    return res
+
+
+def bench_big_gemms(dev, index, iters, warmup):
+    import flashomni_amd as fo
+    from flashomni_amd.workloads import make_workload
+    wl = make_workload(index, tensors=False)
+    s = wl.shape
+    g = torch.Generator(device=dev).manual_seed(2000 + index)
+    x = torch.randn(1, s.seq, s.hidden, generator=g, device=dev).to(torch.bfloat16)
+    wq = (torch.randn(s.hidden, s.hidden, generator=g, device=dev) * 0.02).to(torch.bfloat16)
+    bq = (torch.randn(s.hidden, generator=g, device=dev) * 0.02).to(torch.bfloat16)
+    info, ip = wl.packed_info.to(dev), wl.info_indptr.to(dev)
+    out = torch.zeros(1, s.seq, s.hidden, dtype=torch.bfloat16, device=dev)
+    res = {}
+    ms = time_gpu(lambda: fo.flashomni_gemm(x, wq, s.heads, info, ip, 0, bq, out=out), iters, warmup)
+    res["gemm_q"] = entry(ms, flops=wl.gemm_q_flops())
+    ms = time_gpu(lambda: fo.flashomni_gemm_reduction(x, wq, s.heads, info, ip, 0, bias=bq,
+                                                      is_for_cache=True), iters, warmup)
+    res["gemm_o_cache"] = entry(ms, flops=wl.gemm_o_flops(True))
+    cache = fo.flashomni_gemm_reduction(x, wq, s.heads, info, ip, 0, bias=bq, is_for_cache=True)
+    ms = time_gpu(lambda: fo.flashomni_gemm_reduction(x, wq, s.heads, info, ip, 0, bias=cache,
+                                                      is_for_cache=False), iters, warmup)
+    res["gemm_o_final"] = entry(ms, flops=wl.gemm_o_flops(False))
+    # fp8 quantiser: 2 bytes read + 1 written per element (+ scales)
+    q = out.view(s.seq, s.heads, 128)
+    blocks = tuple(t.to(dev) for t in fo.token_blocks(wl.qo_indptr))
+    ms = time_gpu(lambda: fo.quant_fp8_block(q, wl.qo_indptr, blocks=blocks), iters, warmup)
+    res["quant_fp8"] = entry(ms, nbytes=3 * q.numel() + 4 * s.heads * s.n_blocks)
+    del x, wq, out, cache
+    torch.cuda.empty_cache()
+    return res
+
+
+def cpu_baseline(layer):
+    """The oracle (fp32 dense-masked CPU path) on the FLUX layer, same masks; bounded sample:
+    every 4th active attention row, GEMM-Q on the first 8 row blocks, GEMM-O final on the first 8."""
+    import oracle
+    threads = torch.get_num_threads()
+    w0, w1, w2 = layer.w0, layer.w1, layer.w2
+    rows = list(range(0, w0.active_rows, 4))
+    kept = (w0.sparse_kv_info & w0.sparse_info[:, :, None])
+    # flops of the sampled rows
+    act = w0.sparse_info.reshape(-1).nonzero().squeeze(1)
+    per_row = kept.reshape(-1, kept.shape[-1]).sum(1)[act].double() * 4 * 128 * 128 * 128
+    fa_flops = float(per_row[rows].sum())
+    t0 = time.perf_counter()
+    oracle.sparse_attention(w0.tensors["q"], w0.tensors["k"], w0.tensors["v"], w0.packed_info,
+                            w0.packed_kv_info, w0.info_indptr, w0.kv_info_indptr, w0.qo_indptr,
+                            w0.kv_indptr, rows=rows)
+    t_fa = time.perf_counter() - t0
+    nblk = 8
+    x, a = w1.tensors["x"][:, :nblk * 128], w2.tensors["a"][:, :nblk * 128]
+    t0 = time.perf_counter()
+    oracle.gemm_q(x, w1.tensors["w"], 24, w1.packed_info, w1.info_indptr, 0, w1.tensors["bias"])
+    t_q = time.perf_counter() - t0
+    q_flops = float(w1.sparse_info[:nblk].sum()) * 2 * 128 * 128 * 3072
+    cache = torch.zeros(1, nblk * 128, 3072, dtype=torch.bfloat16)
+    t0 = time.perf_counter()
+    oracle.gemm_o(a, w2.tensors["w"], 24, w2.packed_info, w2.info_indptr, 0, bias=cache, is_for_cache=False)
+    t_o = time.perf_counter() - t0
+    o_flops = float(w2.sparse_info[:nblk].sum()) * 2 * 128 * 3072 * 128
+    total_t, total_f = t_fa + t_q + t_o, fa_flops + q_flops + o_flops
+    return {
+        "value": round(total_f / total_t / 1e12, 4), "unit": "TFLOP/s", "cores": threads, "kind": "port",
+        "sample": "FLUX layer, fp32 torch: every 4th active attention row (%d rows, %.2fs), GEMM-Q and "
+                  "GEMM-O final on the first %d of 36 row blocks (%.2fs, %.2fs)" % (len(rows), t_fa, nblk, t_q, t_o),
+        "sparse_fa_tflops": round(fa_flops / t_fa / 1e12, 4),
+        "gemm_q_tflops": round(q_flops / t_q / 1e12, 4),
+        "gemm_o_tflops": round(o_flops / t_o / 1e12, 4),
+    }
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=50)
+    ap.add_argument("--warmup", type=int, default=10)
+    ap.add_argument("--configs", default="0,1,2,3,4")
+    ap.add_argument("--no-cpu", action="store_true")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        sys.exit("bench.py measures one GPU: this path runs on a single MI355X (heads shard without "
+                 "communication; nothing here uses a second GPU). Run with --gpus 1.")
+    if not torch.cuda.is_available():
+        sys.exit("bench.py needs a GPU")
+    dev = torch.device("cuda:0")
+    torch.cuda.set_device(dev)
+    configs = {int(c) for c in args.configs.split(",") if c != ""}
+    K, W = args.steps, args.warmup
+
+    log("[bench] building FLUX layer inputs (configs 0-2)")
+    layer = FluxLayer(dev)
+    kernels = {}
+
+    # ---- the timed region: K steps of the chain ----
+    for _ in range(W):
+        layer.step()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(K):
+        layer.step()
+    torch.cuda.synchronize()
+    ms_per_step = (time.perf_counter() - t0) * 1e3 / K
+    chain_flops = layer.chain_flops()
+    value = chain_flops / (ms_per_step * 1e-3) / 1e12
+    log("[bench] chain %.4f ms/step -> %.1f TFLOP/s" % (ms_per_step, value))
+
+    # ---- per-kernel, HIP events ----
+    w0 = layer.w0
+    c0 = {}
+    ms = time_gpu(layer.decode, K, W)
+    rows, nnz = layer.wrapper._worklist.sizes()
+    c0["decode"] = entry(ms, nbytes=w0.packed_info.numel() + w0.packed_kv_info.numel() + 4 * (4 * rows + 1 + nnz))
+    c0["decode"]["rows"], c0["decode"]["kv_blocks"] = rows, nnz
+    fa_ms = time_gpu(lambda: layer.attention(fresh_decode=False), K, W)
+    c0["sparse_fa_bf16"] = entry(fa_ms, flops=w0.attention_flops())
+    c0["sparse_fa_bf16"]["computed_blocks"] = w0.computed_blocks
+    kernels[w0.shape.name] = c0
+    ms = time_gpu(layer.gemm_q, K, W)
+    kernels[layer.w1.shape.name] = {"gemm_q": entry(ms, flops=layer.w1.gemm_q_flops())}
+    kernels[layer.w1.shape.name]["gemm_q"]["tiles"] = layer.w1.active_rows
+    c2 = {}
+    c2["gemm_o_cache"] = entry(time_gpu(layer.gemm_o_cache, K, W), flops=layer.w2.gemm_o_flops(True))
+    c2["gemm_o_final"] = entry(time_gpu(layer.gemm_o_final, K, W), flops=layer.w2.gemm_o_flops(False))
+    kernels[layer.w2.shape.name] = c2
+    # packbits at the config-0 mask size and at 16 Mi flags
+    pk = {}
+    for n in (31104, 1 << 24):
+        xb = (torch.rand(n, device=dev) < 0.5)
+        pk["n=%d" % n] = entry(time_gpu(lambda: layer.fo.packbits(xb, "little"), K, W), nbytes=n + n // 8)
+    kernels["packbits"] = pk
+    for name, d in kernels.items():
+        log("[bench]", name, json.dumps(d))
+
+    big_iters, big_warm = max(3, min(K, 10)), 2
+    for idx in (3, 4):
+        if idx in configs:
+            from flashomni_amd.workloads import SHAPES
+            log("[bench] config %d attention (bf16)" % idx)
+            res = bench_big_attention(dev, idx, big_iters, big_warm)
+            if idx == 4:
+                log("[bench] config 4 GEMMs + quantiser")
+                res.update(bench_big_gemms(dev, idx, big_iters, big_warm))
+            kernels[SHAPES[idx].name] = res
+            log("[bench]", SHAPES[idx].name, json.dumps(res))
+
+    fa_flops = w0.attention_flops()
+    roofline = {
+        "kernel": "sparse_fa_kernel<bf16> (config 0, FLUX shape)", "bound": "mfma",
+        "achieved": round(fa_flops / (fa_ms * 1e-3) / 1e12, 2), "peak": PEAK_BF16, "unit": "TFLOP/s",
+        "frac": round(fa_flops / (fa_ms * 1e-3) / 1e12 / PEAK_BF16, 4), "traffic": None,
+        "launch_ms": round(fa_ms, 5), "algorithmic_flop_per_launch": fa_flops,
+    }
+    cpu = None
+    if not args.no_cpu:
+        log("[bench] CPU baseline (oracle, %d threads)" % torch.get_num_threads())
+        cpu = cpu_baseline(layer)
+
+    line = {
+        "metric": "sparse-FA + GEMM-Q/O effective TFLOP/s on computed blocks, FLUX-shaped sparse layer "
+                  "(GEMM-Q c1 -> decode + sparse FA c0 -> GEMM-O final c2), 1 GPU",
+        "value": round(value, 2), "unit": "TFLOP/s", "n_gpus": 1, "steps": K, "warmup": W,
+        "ms_per_step": round(ms_per_step, 5), "higher_is_better": True, "scaling": "weak",
+        "vs_baseline": None, "dtype": "bf16", "data": "synthetic",
+        "config": {"workload": "FLUX layer: c1_flux_gemm_q + c0_flux_sparse_fa + c2_flux_gemm_o(final)",
+                   "seq": 4608, "heads": 24, "head_dim": 128, "hidden": 3072, "block": 128,
+                   "p_cached": 0.25, "kv_density": round(float(w0.sparse_kv_info.float().mean()), 3),
+                   "frac_of_bf16_peak": round(value / PEAK_BF16, 4)},
+        "roofline": roofline, "cpu_baseline": cpu, "kernels": kernels,
+    }
+    print(json.dumps(line), flush=True)
+
+
+if __name__ == "__main__":
+    main()
