@@ -47,7 +47,7 @@ class _Bump:
 
 
 def prefill_plan(qo_indptr, kv_indptr, num_qo_heads, num_kv_heads, head_dim_vo, num_cu,
-                 int_ws_bytes=8 * 1024 * 1024, page_size=1, enable_graph=False, total_num_rows=None):
+                 int_ws_bytes=8 * 1024 * 1024, float_ws_bytes=128 * 1024 * 1024, page_size=1, enable_graph=False, total_num_rows=None):
     """Returns dict with the 15 plan_info entries (scheduler.cuh:205-221) and the arrays."""
     if num_qo_heads % num_kv_heads:
         raise RuntimeError("num_qo_heads should be divisible by num_kv_heads")
@@ -93,12 +93,16 @@ def prefill_plan(qo_indptr, kv_indptr, num_qo_heads, num_kv_heads, head_dim_vo, 
     off["kv_chunk_size_ptr"] = bump.alloc(4, 1)
     off["total_num_rows"] = bump.alloc(4, 16) if enable_graph else 0
     off["merge_indptr"] = off["block_valid_mask"] = 0
+    v_off = s_off = 0
     if split_kv:
+        fb = _Bump(float_ws_bytes)
+        v_off = fb.alloc(num_qo_heads * padded * cta_tile_q * head_dim_vo * 4, 16)
+        s_off = fb.alloc(num_qo_heads * padded * cta_tile_q * 4, 16)
         off["merge_indptr"] = bump.alloc(4 * (total_num_rows + 1), 16)
         off["block_valid_mask"] = bump.alloc(padded, 16)
     info = [padded, total_num_rows, off["total_num_rows"], cta_tile_q, off["request_indices"],
             off["qo_tile_indices"], off["kv_tile_indices"], off["merge_indptr"], off["o_indptr"],
-            off["kv_chunk_size_ptr"], 0, 0, off["block_valid_mask"], int(enable_graph), int(split_kv)]
+            off["kv_chunk_size_ptr"], v_off, s_off, off["block_valid_mask"], int(enable_graph), int(split_kv)]
     return dict(plan_info=info, request_indices=req, qo_tile_indices=qt, kv_tile_indices=kt,
                 o_indptr=o_indptr, merge_indptr=merge, kv_chunk_size=kv_chunk, split_kv=split_kv,
                 cta_tile_q=cta_tile_q, padded_batch_size=padded, used_bytes=bump.cur)
