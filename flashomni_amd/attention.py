@@ -52,10 +52,11 @@ class DecodedWorkList:
     """Device buffers holding one decoded work list (canonical order).
 
     ``row_req/row_qb/row_head[n_rows]``, ``kv_row_ptr[n_rows+1]``, ``kv_idx[nnz]``, all int32;
-    ``counts = [n_rows, nnz, 0, 0]``.  The sizes live on the device; ``sizes()`` copies them back
-    (one synchronisation) for tests and reports."""
+    ``counts = [n_rows, nnz, 0, 0]``; ``order[n_rows]`` / ``sched[32]`` are the execution order
+    and queue words the attention kernel schedules from.  The sizes live on the device;
+    ``sizes()`` copies them back (one synchronisation) for tests and reports."""
 
-    def __init__(self, max_rows: int, max_nnz: int, device):
+    def __init__(self, max_rows: int, max_nnz: int, num_heads: int, device):
         self.max_rows, self.max_nnz = max_rows, max_nnz
         n = max(max_rows, 1)
         self.row_req = torch.empty(n, dtype=torch.int32, device=device)
@@ -64,7 +65,9 @@ class DecodedWorkList:
         self.kv_row_ptr = torch.empty(n + 1, dtype=torch.int32, device=device)
         self.kv_idx = torch.empty(max(max_nnz, 1), dtype=torch.int32, device=device)
         self.counts = torch.zeros(4, dtype=torch.int32, device=device)
-        self.scratch = torch.empty(2 * n + 2, dtype=torch.int32, device=device)
+        self.order = torch.empty(n, dtype=torch.int32, device=device)
+        self.sched = torch.zeros(32, dtype=torch.int32, device=device)
+        self.scratch = torch.empty(2 * n + num_heads, dtype=torch.int32, device=device)
 
     def sizes(self) -> Tuple[int, int]:
         c = self.counts.cpu()
@@ -276,7 +279,7 @@ class BatchFlashOmniFAWithRaggedKVWrapper:
         self._n_kv_blk = int(kv_base[-1])
         if (self._worklist is None or self._worklist.max_rows < max_rows
                 or self._worklist.max_nnz < max_nnz):
-            self._worklist = DecodedWorkList(max_rows, max_nnz, self.device)
+            self._worklist = DecodedWorkList(max_rows, max_nnz, num_qo_heads, self.device)
         self._max_rows = max_rows
         self._decode_key = None
 
@@ -333,8 +336,8 @@ class BatchFlashOmniFAWithRaggedKVWrapper:
             _lib.ptr(self._blk_table[0]), _lib.ptr(self._blk_table[1]), _lib.ptr(self._kv_indptr_buf),
             self._n_q_blk, self._num_qo_heads, self._sparse_block_size_for_kv, int(bool(is_full)),
             _lib.ptr(wl.row_req), _lib.ptr(wl.row_qb), _lib.ptr(wl.row_head), _lib.ptr(wl.kv_row_ptr),
-            _lib.ptr(wl.kv_idx), _lib.ptr(wl.counts), _lib.ptr(wl.scratch),
-            _lib.current_stream(self.device)))
+            _lib.ptr(wl.kv_idx), _lib.ptr(wl.counts), _lib.ptr(wl.order), _lib.ptr(wl.sched),
+            _lib.ptr(wl.scratch), _lib.current_stream(self.device)))
         # the memo holds the tensors alive so a recycled address cannot alias the key
         self._decode_key = key
         self._decode_refs = (tensors, sparse_info, sparse_kv_info, sparse_info_indptr,
@@ -418,8 +421,8 @@ class BatchFlashOmniFAWithRaggedKVWrapper:
             q.stride(0), q.stride(1), k_sn, k_sh, v_sn, v_sh, out.stride(0), out.stride(1),
             _lib.ptr(self._qo_indptr_buf), _lib.ptr(self._kv_indptr_buf), _lib.ptr(self._q_blk_base),
             _lib.ptr(self._kv_blk_base), _lib.ptr(wl.row_req), _lib.ptr(wl.row_qb),
-            _lib.ptr(wl.row_head), _lib.ptr(wl.kv_row_ptr), _lib.ptr(wl.kv_idx), _lib.ptr(wl.counts),
-            self._max_rows, q.size(1), q.size(2), self._sparse_block_size_for_q,
+            _lib.ptr(wl.row_head), _lib.ptr(wl.kv_row_ptr), _lib.ptr(wl.kv_idx), _lib.ptr(wl.order),
+            _lib.ptr(wl.sched), self._max_rows, q.size(1), q.size(2), self._sparse_block_size_for_q,
             self._sparse_block_size_for_kv, float(sm_scale), _lib.current_stream(self.device)))
         return (out, lse) if return_lse else out
 

@@ -2,8 +2,16 @@
 // keep masks -> compacted work list in canonical order (ascending request, q-block, head; kv
 // blocks ascending inside a row).  Three short launches on one stream, no host round trip:
 //   count : one wavefront per (q-block, head) candidate; lanes take one mask byte each, popcount
-//   scan  : one workgroup, exclusive prefix sums of row flags and kv counts (canonical positions)
+//   scan  : one workgroup, exclusive prefix sums of row flags and kv counts (canonical positions),
+//           plus a per-head histogram that lays out the execution order
 //   fill  : one wavefront per candidate again; wave prefix of popcounts places every kv index
+//
+// Besides the canonical list the decoder emits an execution order for the attention kernel:
+// `order` lists row positions grouped by head, heads dealt to the 8 XCDs round-robin (head % 8), so
+// that the workgroups of one XCD (which share an L2) walk the rows of the same few heads and find
+// that head's K/V in their L2.  sched[0..8] delimit the 8 per-XCD queues inside `order`,
+// sched[16..23] are the queue cursors and sched[24] a completion counter (all cleared here).
+// The order inside a head is not deterministic (atomic cursors); results do not depend on it.
 // Integer work, bounded by HBM traffic and launch latency; bit-exact by construction.
 //
 // Symbol semantics (reference: include/flashomni/attention/prefill.cuh:1284-1294, 1380-1403,
@@ -16,6 +24,8 @@ namespace {
 constexpr int kWave = 64;
 constexpr int kCountThreads = 256;  // 4 candidates per workgroup
 constexpr int kScanThreads = 1024;
+constexpr int kMaxHeads = 1024;
+constexpr int kXcds = 8;
 
 struct Candidate {
   int32_t req, qb, head, nkv;
@@ -90,17 +100,23 @@ __global__ void __launch_bounds__(kCountThreads) decode_count_kernel(
 
 // In place: act[c] -> canonical row position (or -1), cnt[c] -> first kv_idx slot of the row.
 __global__ void __launch_bounds__(kScanThreads) decode_scan_kernel(
-    int64_t n_cand, int32_t* __restrict__ act, int32_t* __restrict__ cnt,
-    int32_t* __restrict__ kv_row_ptr, int32_t* __restrict__ counts) {
+    int64_t n_cand, int32_t num_heads, int32_t* __restrict__ act, int32_t* __restrict__ cnt,
+    int32_t* __restrict__ kv_row_ptr, int32_t* __restrict__ counts,
+    int32_t* __restrict__ head_cursor, int32_t* __restrict__ sched) {
   __shared__ int32_t s_rows[kScanThreads];
   __shared__ int32_t s_kv[kScanThreads];
+  __shared__ int32_t s_hist[kMaxHeads];
   const int tid = threadIdx.x;
+  for (int h = tid; h < num_heads; h += kScanThreads) s_hist[h] = 0;
+  __syncthreads();
   const int64_t chunk = (n_cand + kScanThreads - 1) / kScanThreads;
   const int64_t lo = tid * chunk, hi = (lo + chunk < n_cand) ? lo + chunk : n_cand;
   int32_t rows = 0, kv = 0;
   for (int64_t c = lo; c < hi; ++c) {
-    rows += act[c];
+    const int32_t a = act[c];
+    rows += a;
     kv += cnt[c];
+    if (a) atomicAdd(&s_hist[c % num_heads], 1);
   }
   s_rows[tid] = rows;
   s_kv[tid] = kv;
@@ -133,6 +149,19 @@ __global__ void __launch_bounds__(kScanThreads) decode_scan_kernel(
     counts[3] = 0;
     kv_row_ptr[n_rows] = nnz;
   }
+  // execution order layout: queue x holds heads x, x+8, x+16, ... back to back
+  if (tid == 0) {
+    int32_t pos = 0;
+    for (int x = 0; x < kXcds; ++x) {
+      sched[x] = pos;
+      for (int h = x; h < num_heads; h += kXcds) {
+        head_cursor[h] = pos;
+        pos += s_hist[h];
+      }
+    }
+    sched[kXcds] = pos;
+    for (int i = kXcds + 1; i < 32; ++i) sched[i] = 0;
+  }
 }
 
 __global__ void __launch_bounds__(kCountThreads) decode_fill_kernel(
@@ -143,7 +172,8 @@ __global__ void __launch_bounds__(kCountThreads) decode_fill_kernel(
     int32_t num_heads, int32_t block_kv, int is_full, const int32_t* __restrict__ row_pos,
     const int32_t* __restrict__ kv_pos, int32_t* __restrict__ row_req,
     int32_t* __restrict__ row_qb, int32_t* __restrict__ row_head,
-    int32_t* __restrict__ kv_row_ptr, int32_t* __restrict__ kv_idx) {
+    int32_t* __restrict__ kv_row_ptr, int32_t* __restrict__ kv_idx,
+    int32_t* __restrict__ head_cursor, int32_t* __restrict__ order) {
   const int lane = threadIdx.x % kWave;
   const int64_t c = static_cast<int64_t>(blockIdx.x) * (kCountThreads / kWave) + threadIdx.x / kWave;
   if (c >= n_cand) return;
@@ -157,6 +187,7 @@ __global__ void __launch_bounds__(kCountThreads) decode_fill_kernel(
     row_qb[pos] = cd.qb;
     row_head[pos] = cd.head;
     kv_row_ptr[pos] = out;
+    order[atomicAdd(&head_cursor[cd.head], 1)] = pos;
   }
   if (cd.nkv <= 0) return;
   if (is_full) {
@@ -193,9 +224,10 @@ extern "C" int fo_decode_sparse(const uint8_t* sparse_info, const uint8_t* spars
                                 int32_t num_heads, int32_t block_kv, int is_full,
                                 int32_t* row_req, int32_t* row_qb, int32_t* row_head,
                                 int32_t* kv_row_ptr, int32_t* kv_idx, int32_t* counts,
-                                int32_t* scratch, void* stream) {
-  FO_REQUIRE(n_blk >= 0 && num_heads > 0 && block_kv > 0, "decode: bad sizes");
-  FO_REQUIRE(counts && kv_row_ptr, "decode: null output");
+                                int32_t* order, int32_t* sched, int32_t* scratch, void* stream) {
+  FO_REQUIRE(n_blk >= 0 && num_heads > 0 && num_heads <= kMaxHeads && block_kv > 0,
+             "decode: bad sizes");
+  FO_REQUIRE(counts && kv_row_ptr && order && sched, "decode: null output");
   if (!is_full) {
     FO_REQUIRE(sparse_info && sparse_kv_info && sparse_info_indptr && sparse_kv_info_indptr,
                "decode: sparse_info, sparse_kv_info and their indptrs are required unless is_full");
@@ -206,6 +238,7 @@ extern "C" int fo_decode_sparse(const uint8_t* sparse_info, const uint8_t* spars
   hipStream_t s = static_cast<hipStream_t>(stream);
   int32_t* act = scratch;
   int32_t* cnt = scratch + n_cand;
+  int32_t* head_cursor = scratch + 2 * n_cand;
   if (n_cand > 0) {
     FO_REQUIRE(row_req && row_qb && row_head && kv_idx, "decode: null output");
     const int per_wg = kCountThreads / kWave;
@@ -215,7 +248,8 @@ extern "C" int fo_decode_sparse(const uint8_t* sparse_info, const uint8_t* spars
         kv_indptr, n_cand, num_heads, block_kv, is_full, act, cnt);
     FO_CHECK_LAUNCH();
   }
-  decode_scan_kernel<<<1, kScanThreads, 0, s>>>(n_cand, act, cnt, kv_row_ptr, counts);
+  decode_scan_kernel<<<1, kScanThreads, 0, s>>>(n_cand, num_heads, act, cnt, kv_row_ptr, counts,
+                                                head_cursor, sched);
   FO_CHECK_LAUNCH();
   if (n_cand > 0) {
     const int per_wg = kCountThreads / kWave;
@@ -223,7 +257,7 @@ extern "C" int fo_decode_sparse(const uint8_t* sparse_info, const uint8_t* spars
     decode_fill_kernel<<<grid, kCountThreads, 0, s>>>(
         sparse_info, sparse_kv_info, sparse_info_indptr, sparse_kv_info_indptr, blk_req, blk_qb,
         kv_indptr, n_cand, num_heads, block_kv, is_full, act, cnt, row_req, row_qb, row_head,
-        kv_row_ptr, kv_idx);
+        kv_row_ptr, kv_idx, head_cursor, order);
     FO_CHECK_LAUNCH();
   }
   return FO_OK;

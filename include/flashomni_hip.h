@@ -86,10 +86,15 @@ int fo_prefill_plan(void* float_ws, size_t float_ws_bytes, void* int_ws_dev, voi
  * Outputs (all int32, device):
  *   row_req,row_qb,row_head [n_rows]  rows with flag 1, ascending (request, q-block, head)
  *   kv_row_ptr [n_rows+1], kv_idx [nnz]  kept kv blocks of each row, ascending
- *   counts[0] = n_rows, counts[1] = nnz, counts[2..3] = scratch counters cleared to 0
+ *   counts[0] = n_rows, counts[1] = nnz, counts[2..3] = 0
+ *   order [n_rows]   execution order for the attention kernel: canonical row positions grouped by
+ *                    head, heads dealt round-robin to 8 queues (head % 8, one queue per XCD); the
+ *                    order inside one head is unspecified
+ *   sched [32]       sched[0..8] = queue boundaries inside `order`, sched[16..23] = queue cursors
+ *                    and sched[24] = completion counter, both cleared to 0
  * is_full != 0 ignores the symbol tensors (which may be NULL) and lists everything
  * (csrc/batch_sparseFA.cu:123-128).
- * `scratch` needs 2*n_blk*H + 2 int32.
+ * `scratch` needs 2*n_blk*H + H int32.
  * ------------------------------------------------------------------------------------------- */
 int fo_sparse_block_table(const int32_t* qo_indptr_host, uint32_t batch_size, uint32_t block_q,
                           int32_t* blk_req_host, int32_t* blk_qb_host, int64_t capacity,
@@ -102,7 +107,8 @@ int fo_decode_sparse(const uint8_t* sparse_info, const uint8_t* sparse_kv_info,
                      const int32_t* blk_req, const int32_t* blk_qb, const int32_t* kv_indptr,
                      int32_t n_blk, int32_t num_heads, int32_t block_kv, int is_full,
                      int32_t* row_req, int32_t* row_qb, int32_t* row_head, int32_t* kv_row_ptr,
-                     int32_t* kv_idx, int32_t* counts, int32_t* scratch, void* stream);
+                     int32_t* kv_idx, int32_t* counts, int32_t* order, int32_t* sched,
+                     int32_t* scratch, void* stream);
 
 /* ---------------------------------------------------------------------------------------------
  * Ragged block-sparse FlashAttention prefill over a decoded work list.
@@ -118,7 +124,10 @@ int fo_decode_sparse(const uint8_t* sparse_info, const uint8_t* sparse_kv_info,
  * Rows of the list write every output row of their q-block; q-blocks not in the list are left
  * untouched; a listed row with no kv block writes zeros and lse = -5e4.  lse (optional, fp32
  * [nnz_q,H]) is base 2: log2(sum 2^(s*c - m*c)) + m*c, c = sm_scale*log2(e).
- * Supported: D = 128, block_q = 128, block_kv = 128.  max_rows bounds counts[0].
+ * Rows are taken from the queues described by `order` / `sched` (see fo_decode_sparse); the
+ * kernel leaves the queue cursors rewound, so one decoded list can be run any number of times,
+ * but two launches sharing one `sched` must not overlap in time.
+ * Supported: D = 128, block_q = 128, block_kv = 128.  max_rows bounds the number of rows.
  * ------------------------------------------------------------------------------------------- */
 int fo_sparse_fa_run(const void* q, const void* k, const void* v, void* o, float* lse, int dtype,
                      const float* q_scale, const float* k_scale, int64_t q_stride_n,
@@ -127,9 +136,9 @@ int fo_sparse_fa_run(const void* q, const void* k, const void* v, void* o, float
                      int64_t o_stride_h, const int32_t* qo_indptr, const int32_t* kv_indptr,
                      const int32_t* q_blk_base, const int32_t* kv_blk_base,
                      const int32_t* row_req, const int32_t* row_qb, const int32_t* row_head,
-                     const int32_t* kv_row_ptr, const int32_t* kv_idx, int32_t* counts,
-                     int64_t max_rows, int32_t num_heads, int32_t head_dim, int32_t block_q,
-                     int32_t block_kv, float sm_scale, void* stream);
+                     const int32_t* kv_row_ptr, const int32_t* kv_idx, const int32_t* order,
+                     int32_t* sched, int64_t max_rows, int32_t num_heads, int32_t head_dim,
+                     int32_t block_q, int32_t block_kv, float sm_scale, void* stream);
 
 /* ---------------------------------------------------------------------------------------------
  * GEMM-Q: y[b, tile] = x[b] . w^T + bias for every (128-row, 128-column) tile whose symbol bit
