@@ -150,11 +150,15 @@ int fo_sparse_fa_run(const void* q, const void* k, const void* v, void* o, float
  * + (ix*128)/(N/num_qo_heads) of sparse_info + sparse_info_indptr[b] (gemm.cuh:50-58).
  * Requires N % 128 == 0 and K % 32 == 0 (csrc/gemm.cu:36); M may have a tail (the reference
  * demands M % 128 == 0).
+ * `workspace`: device scratch of at least fo_gemm_q_workspace_bytes(batch, m, n) bytes, 16-byte
+ * aligned; it receives the compacted list of flagged tile pairs that the GEMM kernel walks.
  * ------------------------------------------------------------------------------------------- */
+int64_t fo_gemm_q_workspace_bytes(int32_t batch, int32_t m, int32_t n);
 int fo_gemm_q(const void* x, const void* w, const void* bias, void* y, int dtype, int32_t batch,
               int32_t m, int32_t n, int32_t k, int32_t sparse_q_size, int32_t num_qo_heads,
               const uint8_t* sparse_info, const int32_t* sparse_info_indptr,
-              int32_t num_text_tokens, int is_full, void* stream);
+              int32_t num_text_tokens, int is_full, void* workspace, int64_t workspace_bytes,
+              void* stream);
 
 /* ---------------------------------------------------------------------------------------------
  * GEMM-O with reduction: y[b, row-tile, :] = init + sum over selected head slices of
