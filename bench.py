@@ -142,6 +142,25 @@ def bench_big_attention(dev, index, iters, warmup):
     ms = time_gpu(lambda: w.run(q, k, v, *args, out=out), iters, warmup)
     res["sparse_fa_bf16"] = entry(ms, flops=wl.attention_flops())
     res["sparse_fa_bf16"]["computed_blocks"] = wl.computed_blocks
+    if index == 4:
+        # fp8 e4m3 Q.K^T (per-(head, 128-token block) absmax scales), bf16 P.V
+        blocks = tuple(t.to(dev) for t in fo.token_blocks(wl.qo_indptr))
+        ms_q = time_gpu(lambda: fo.quant_fp8_block(q, wl.qo_indptr, blocks=blocks), iters, warmup)
+        res["quant_fp8"] = entry(ms_q, nbytes=3 * q.numel() + 4 * s.heads * s.n_blocks)
+        q8, qs = fo.quant_fp8_block(q, wl.qo_indptr, blocks=blocks)
+        k8, ks = fo.quant_fp8_block(k, wl.kv_indptr, blocks=blocks)
+        w8 = fo.BatchFlashOmniFAWithRaggedKVWrapper(ws)
+        w8.plan(wl.qo_indptr, wl.kv_indptr, s.heads, s.heads, 128, q_data_type=torch.float8_e4m3fn)
+        out8 = torch.zeros_like(q)
+        ms8 = time_gpu(lambda: w8.run(q8, k8, v, *args, out=out8, q_scale=qs, k_scale=ks), iters, warmup)
+        # QK^T half at the fp8 peak, PV half at the bf16 peak
+        res["sparse_fa_fp8qk"] = entry(ms8, flops=wl.attention_flops(), peak=2.0 / (1 / PEAK_FP8 + 1 / PEAK_BF16))
+        res["sparse_fa_fp8qk"]["frac_of_bf16_peak"] = round(res["sparse_fa_fp8qk"]["tflops"] / PEAK_BF16, 4)
+        # error of the fp8 output against the bf16 kernel's output on the same inputs
+        w.run(q, k, v, *args, out=out)
+        num = (out8.float() - out.float()).norm()
+        res["sparse_fa_fp8qk"]["rel_l2_vs_bf16_kernel"] = round(float(num / out.float().norm()), 4)
+        del q8, k8, out8
     del q, k, v, out
     torch.cuda.empty_cache()
     return res
@@ -168,11 +187,6 @@ def bench_big_gemms(dev, index, iters, warmup):
     ms = time_gpu(lambda: fo.flashomni_gemm_reduction(x, wq, s.heads, info, ip, 0, bias=cache,
                                                       is_for_cache=False), iters, warmup)
     res["gemm_o_final"] = entry(ms, flops=wl.gemm_o_flops(False))
-    # fp8 quantiser: 2 bytes read + 1 written per element (+ scales)
-    q = out.view(s.seq, s.heads, 128)
-    blocks = tuple(t.to(dev) for t in fo.token_blocks(wl.qo_indptr))
-    ms = time_gpu(lambda: fo.quant_fp8_block(q, wl.qo_indptr, blocks=blocks), iters, warmup)
-    res["quant_fp8"] = entry(ms, nbytes=3 * q.numel() + 4 * s.heads * s.n_blocks)
     del x, wq, out, cache
     torch.cuda.empty_cache()
     return res

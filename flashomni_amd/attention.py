@@ -420,7 +420,8 @@ class BatchFlashOmniFAWithRaggedKVWrapper:
             _lib.ptr(k_scale if fp8 else None),
             q.stride(0), q.stride(1), k_sn, k_sh, v_sn, v_sh, out.stride(0), out.stride(1),
             _lib.ptr(self._qo_indptr_buf), _lib.ptr(self._kv_indptr_buf), _lib.ptr(self._q_blk_base),
-            _lib.ptr(self._kv_blk_base), _lib.ptr(wl.row_req), _lib.ptr(wl.row_qb),
+            _lib.ptr(self._kv_blk_base), self._n_q_blk, self._n_kv_blk, _lib.ptr(wl.row_req),
+            _lib.ptr(wl.row_qb),
             _lib.ptr(wl.row_head), _lib.ptr(wl.kv_row_ptr), _lib.ptr(wl.kv_idx), _lib.ptr(wl.order),
             _lib.ptr(wl.sched), self._max_rows, q.size(1), q.size(2), self._sparse_block_size_for_q,
             self._sparse_block_size_for_kv, float(sm_scale), _lib.current_stream(self.device)))

@@ -36,6 +36,8 @@
 // include/flashomni/math.cuh:32, O = acc * rcp(d) with one round-to-nearest cast, a row with no kv
 // block writes zeros and lse = -5e4, lse = log2(d) + m*c.  (The row sum d is accumulated from the
 // fp32 p values; the reference sums the rounded ones.)
+#include <type_traits>
+
 #include "fo_common.h"
 
 namespace {
@@ -48,23 +50,30 @@ typedef __attribute__((ext_vector_type(4))) short s16x4;
 typedef __attribute__((ext_vector_type(16))) float f32x16;
 typedef __attribute__((ext_vector_type(4))) float f32x4;
 typedef __attribute__((ext_vector_type(4))) unsigned int u32x4;
+typedef __attribute__((ext_vector_type(8))) int i32x8;
+typedef __attribute__((ext_vector_type(4))) int i32x4;
 
 constexpr float kNegInf = -5e4f;  // finite "infinity" of the reference
 constexpr int kThreads = 512;
 constexpr int kGroupThreads = 256;
 constexpr int kBlockQ = 128, kBlockKV = 128, kHeadDim = 128;
 constexpr int kTileKV = 64;
-constexpr int kRowBytes = 256;  // one K or V row of 128 16-bit elements, unpadded (swizzled)
-constexpr int kKBytes = kTileKV * kRowBytes;
+constexpr int kRowBytes = 256;   // one K or V row of 128 16-bit elements, unpadded (swizzled)
+constexpr int kRowBytes8 = 128;  // one fp8 K row
 constexpr int kVBytes = kTileKV * kRowBytes;
-constexpr int kStageBytes = kKBytes + kVBytes;
-constexpr int kGroupBytes = 2 * kStageBytes;
-constexpr int kSmemBytes = 2 * kGroupBytes;
+// LDS geometry of one kv group: two stages of (K tile, V tile); K is 16-bit or fp8
+template <bool kFp8>
+struct Geom {
+  static constexpr int kKBytes = kTileKV * (kFp8 ? kRowBytes8 : kRowBytes);
+  static constexpr int kStageBytes = kKBytes + kVBytes;
+  static constexpr int kGroupBytes = 2 * kStageBytes;
+  static constexpr int kSmemBytes = 2 * kGroupBytes;
+};
 constexpr int kXcds = 8;
 constexpr float kLazyLog2 = 8.0f;  // the running max is raised only past a 2^8 overshoot
 // merge area (reuses the tile buffers): O^T of kv group 1, then its (m, d)
 constexpr int kMergeOBytes = 4 * 16 * 64 * 16;
-static_assert(kMergeOBytes + 4 * 64 * 8 <= kSmemBytes, "merge area must fit");
+static_assert(kMergeOBytes + 4 * 64 * 8 <= Geom<true>::kSmemBytes, "merge area must fit");
 
 struct FaParams {
   const void* q;
@@ -114,8 +123,10 @@ typedef __attribute__((address_space(3))) s16x4 lds_s16x4;
 typedef __attribute__((address_space(3))) void lds_void;
 typedef __attribute__((address_space(1))) const void glb_void;
 
-// chunk swizzle of LDS tile row r
+// chunk swizzle of a 256-byte LDS tile row r (16 chunks)
 __device__ __forceinline__ int swz(int r) { return ((r & 3) << 2) | ((r >> 2) & 3); }
+// chunk swizzle of a 128-byte LDS tile row r (8 chunks; two rows span the 64 banks)
+__device__ __forceinline__ int swz8(int r) { return (r >> 1) & 7; }
 
 // 64 lanes x 16 bytes, global -> LDS at lds_base + lane*16 (lds_base is wavefront-uniform)
 __device__ __forceinline__ void copy16_to_lds(const void* gsrc, uint8_t* lds_base) {
@@ -141,11 +152,18 @@ __device__ __forceinline__ int pop_row(const FaParams& p, int xcd) {
   return -1;
 }
 
-template <typename T>
+// T: element type of V, P and O (and of Q, K unless kFp8).  kFp8: Q and K are e4m3fn bytes with one
+// dequantisation scale per (head, 128-token block); S^T then comes from
+// v_mfma_scale_f32_32x32x64_f8f6f4 (64 d per instruction, unit block scale) and the two per-block
+// scales are folded into the softmax scale of the tile.
+template <typename T, bool kFp8>
 __global__ void __launch_bounds__(kThreads) sparse_fa_kernel(const FaParams p) {
   using TT = Types<T>;
   using x8 = typename TT::x8;
   using x4 = typename TT::x4;
+  using G = Geom<kFp8>;
+  using TQK = typename std::conditional<kFp8, uint8_t, T>::type;
+  constexpr int kStageBytes = G::kStageBytes, kKBytes = G::kKBytes, kGroupBytes = G::kGroupBytes;
   extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
   __shared__ int s_next_row;
 
@@ -153,8 +171,8 @@ __global__ void __launch_bounds__(kThreads) sparse_fa_kernel(const FaParams p) {
   const int qs = wv & 3, kg = wv >> 2;
   const int l32 = lane & 31, g = lane >> 5;
   const float c = p.sm_scale_log2;
-  const T* __restrict__ qp = static_cast<const T*>(p.q);
-  const T* __restrict__ kp = static_cast<const T*>(p.k);
+  const TQK* __restrict__ qp = static_cast<const TQK*>(p.q);
+  const TQK* __restrict__ kp = static_cast<const TQK*>(p.k);
   const T* __restrict__ vp = static_cast<const T*>(p.v);
   T* __restrict__ op = static_cast<T*>(p.o);
   uint8_t* const group_smem = smem + kg * kGroupBytes;
@@ -164,8 +182,14 @@ __global__ void __launch_bounds__(kThreads) sparse_fa_kernel(const FaParams p) {
   // fetch logical chunk (lane%16) ^ swz(row).  swz depends on row%16 = 4*qs + lane/16 only.
   const int cp_row = lane >> 4;
   const int cp_chunk = ((lane & 15) ^ swz(4 * qs + cp_row)) * 8;  // element offset inside the row
+  // fp8 K tile (128-byte rows): copy instruction n = 4*j + qs, j = 0..1, fills rows 8n..8n+7; the
+  // lane lands on row 8n + lane/8 at chunk position lane%8; swz8(row) = (4*(n%2) + lane/16) & 7
+  const int cp8_row = lane >> 3;
+  const int cp8_chunk = ((lane & 7) ^ ((4 * (qs & 1) + (lane >> 4)) & 7)) * 16;  // byte offset
   // K operand read: row mt*32 + l32, logical chunk 2*ks + g  ->  xor of a lane constant and ks<<5
-  const int k_rd_base = l32 * kRowBytes, k_rd_x = (g ^ swz(l32)) << 4;
+  // (fp8: logical chunks 4*slab + 2*g and +1 of a 128-byte row)
+  const int k_rd_base = l32 * (kFp8 ? kRowBytes8 : kRowBytes);
+  const int k_rd_x = kFp8 ? ((2 * g) ^ swz8(l32)) << 4 : (g ^ swz(l32)) << 4;
   // V^T transpose read: this lane supplies row j = (lane%16)/4 of a 4-row patch that starts at kv
   // row 16*kk + 4*g (+8 for the second read), 8 bytes at element column 32*dt + 16*q2 + 4*(lane%4)
   int v_rd_off[4][2];
@@ -220,39 +244,66 @@ __global__ void __launch_bounds__(kThreads) sparse_fa_kernel(const FaParams p) {
     const int my_tiles = (n_tiles - kg + 1) >> 1;  // tiles kg, kg+2, ...
 
     // Q operand: lane holds q row l32 of its q sub-tile, d = ks*16 + g*8 .. +7
-    x8 qreg[8];
-    {
-      const T* src = qp + q_tok * p.q_sn + static_cast<int64_t>(head) * p.q_sh + g * 8;
+    // (fp8: d = slab*64 + g*32 .. +31 for the two 64-wide slabs)
+    x8 qreg[kFp8 ? 1 : 8];
+    i32x8 qreg8[kFp8 ? 2 : 1];
+    if constexpr (kFp8) {
+      const uint8_t* src = qp + q_tok * p.q_sn + static_cast<int64_t>(head) * p.q_sh + g * 32;
+#pragma unroll
+      for (int sl = 0; sl < 2; ++sl) {
+        const i32x4 lo = *reinterpret_cast<const i32x4*>(src + sl * 64);
+        const i32x4 hi = *reinterpret_cast<const i32x4*>(src + sl * 64 + 16);
+        qreg8[sl] = i32x8{lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
+      }
+    } else {
+      const T* src = reinterpret_cast<const T*>(qp) + q_tok * p.q_sn + static_cast<int64_t>(head) * p.q_sh + g * 8;
 #pragma unroll
       for (int ks = 0; ks < 8; ++ks) qreg[ks] = *reinterpret_cast<const x8*>(src + ks * 16);
     }
+    // softmax scale in the log2 domain; with fp8 operands the per-block dequantisation scales of
+    // q (one per row of the list) and k (one per kv block) are folded in tile by tile
+    float cq = c;
+    if constexpr (kFp8) cq *= p.q_scale[static_cast<int64_t>(head) * p.n_q_blocks + p.q_blk_base[req] + qb];
+    const float* ksc = nullptr;
+    if constexpr (kFp8) ksc = p.k_scale + static_cast<int64_t>(head) * p.n_kv_blocks + p.kv_blk_base[req];
 
     f32x16 o_acc[4];
 #pragma unroll
     for (int dt = 0; dt < 4; ++dt)
 #pragma unroll
       for (int i = 0; i < 16; ++i) o_acc[dt][i] = 0.f;
-    float m_run = kNegInf, d_part = 0.f;
+    float m_run = kNegInf, d_part = 0.f;  // running max in the log2 domain (s * scale), partial sum
+    float cs_next = cq;
 
     // Issue the global->LDS copy of this kv group's tile `it` into LDS stage it&1.
-    const int64_t k_head = static_cast<int64_t>(head) * p.k_sh + cp_chunk;
+    const int64_t k_head = static_cast<int64_t>(head) * p.k_sh + (kFp8 ? cp8_chunk : cp_chunk);
     const int64_t v_head = static_cast<int64_t>(head) * p.v_sh + cp_chunk;
     auto copy_tile = [&](int it) {
       const int t = 2 * it + kg;
       const int blk = p.kv_idx[ptr0 + (t >> 1)];
       const int start = blk * kBlockKV + (t & 1) * kTileKV;
       const int valid = min(kTileKV, kv_len - start);
-      const T* kt = kp + static_cast<int64_t>(kv_begin + start) * p.k_sn + k_head;
+      const TQK* kt = kp + static_cast<int64_t>(kv_begin + start) * p.k_sn + k_head;
       const T* vt = vp + static_cast<int64_t>(kv_begin + start) * p.v_sn + v_head;
       uint8_t* kdst = group_smem + (it & 1) * kStageBytes;
       uint8_t* vdst = kdst + kKBytes;
+      if constexpr (kFp8) cs_next = cq * ksc[blk];
 #pragma unroll
       for (int j = 0; j < 4; ++j) {
         const int n = 4 * j + qs;
         int r = 4 * n + cp_row;
         r = r < valid ? r : valid - 1;  // ragged tail: re-read the last valid row, never overrun
-        copy16_to_lds(kt + static_cast<int64_t>(r) * p.k_sn, kdst + n * 1024);
+        if constexpr (!kFp8) copy16_to_lds(kt + static_cast<int64_t>(r) * p.k_sn, kdst + n * 1024);
         copy16_to_lds(vt + static_cast<int64_t>(r) * p.v_sn, vdst + n * 1024);
+      }
+      if constexpr (kFp8) {
+#pragma unroll
+        for (int j = 0; j < 2; ++j) {
+          const int n = 4 * j + qs;
+          int r = 8 * n + cp8_row;
+          r = r < valid ? r : valid - 1;
+          copy16_to_lds(kt + static_cast<int64_t>(r) * p.k_sn, kdst + n * 1024);
+        }
       }
       return valid;
     };
@@ -266,6 +317,7 @@ __global__ void __launch_bounds__(kThreads) sparse_fa_kernel(const FaParams p) {
       const uint8_t* vs_base = ks_base + kKBytes;
       const bool active = it < my_tiles;
       const int valid = valid_next;
+      const float cs = cs_next;  // softmax scale of this tile
       // this wavefront's copies of tile `it` have landed; after the barrier everyone's have, and
       // everyone has finished reading the other stage
       __builtin_amdgcn_s_waitcnt(0x0f70);  // vmcnt(0)
@@ -273,24 +325,44 @@ __global__ void __launch_bounds__(kThreads) sparse_fa_kernel(const FaParams p) {
       if (!active) continue;  // (only the last iteration of kv group 1; no barrier follows)
       if (it + 1 < my_tiles) valid_next = copy_tile(it + 1);
 
-      // ---- S^T = K . Q^T : two 32-key tiles x 32 q; all 16 operand reads are issued up front ----
-      x8 ka[8], kb[8];
-#pragma unroll
-      for (int ks = 0; ks < 8; ++ks)
-        ka[ks] = *reinterpret_cast<const x8*>(ks_base + k_rd_base + (k_rd_x ^ (ks << 5)));
-#pragma unroll
-      for (int ks = 0; ks < 8; ++ks)
-        kb[ks] = *reinterpret_cast<const x8*>(ks_base + 32 * kRowBytes + k_rd_base + (k_rd_x ^ (ks << 5)));
-      __builtin_amdgcn_sched_barrier(0);
+      // ---- S^T = K . Q^T : two 32-key tiles x 32 q; all operand reads are issued up front ----
       f32x16 s[2];
 #pragma unroll
       for (int mt = 0; mt < 2; ++mt)
 #pragma unroll
         for (int i = 0; i < 16; ++i) s[mt][i] = 0.f;
+      if constexpr (kFp8) {
+        i32x8 k8[2][2];  // [32-key tile][64-wide d slab]: 32 consecutive fp8 of row l32
 #pragma unroll
-      for (int ks = 0; ks < 8; ++ks) s[0] = TT::mfma(ka[ks], qreg[ks], s[0]);
+        for (int mt = 0; mt < 2; ++mt)
 #pragma unroll
-      for (int ks = 0; ks < 8; ++ks) s[1] = TT::mfma(kb[ks], qreg[ks], s[1]);
+          for (int sl = 0; sl < 2; ++sl) {
+            const uint8_t* rowp = ks_base + mt * 32 * kRowBytes8 + k_rd_base;
+            const i32x4 lo = *reinterpret_cast<const i32x4*>(rowp + (k_rd_x ^ (sl << 6)));
+            const i32x4 hi = *reinterpret_cast<const i32x4*>(rowp + ((k_rd_x ^ (sl << 6)) ^ 16));
+            k8[mt][sl] = i32x8{lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
+          }
+        __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+        for (int mt = 0; mt < 2; ++mt)
+#pragma unroll
+          for (int sl = 0; sl < 2; ++sl)
+            s[mt] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(k8[mt][sl], qreg8[sl], s[mt], 0, 0, 0,
+                                                                    0x7f7f7f7f, 0, 0x7f7f7f7f);
+      } else {
+        x8 ka[8], kb[8];
+#pragma unroll
+        for (int ks = 0; ks < 8; ++ks)
+          ka[ks] = *reinterpret_cast<const x8*>(ks_base + k_rd_base + (k_rd_x ^ (ks << 5)));
+#pragma unroll
+        for (int ks = 0; ks < 8; ++ks)
+          kb[ks] = *reinterpret_cast<const x8*>(ks_base + 32 * kRowBytes + k_rd_base + (k_rd_x ^ (ks << 5)));
+        __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+        for (int ks = 0; ks < 8; ++ks) s[0] = TT::mfma(ka[ks], qreg[ks], s[0]);
+#pragma unroll
+        for (int ks = 0; ks < 8; ++ks) s[1] = TT::mfma(kb[ks], qreg[ks], s[1]);
+      }
 
       // all V^T operands of the tile (4 slabs of 16 keys x 4 d tiles): in flight during the
       // softmax, in the registers the K operands just vacated
@@ -311,14 +383,14 @@ __global__ void __launch_bounds__(kThreads) sparse_fa_kernel(const FaParams p) {
       }
       __builtin_amdgcn_sched_barrier(0);
 
-      // ---- online softmax (per lane: one q column, 32 kv values) ----
+      // ---- online softmax (per lane: one q column, 32 kv values), log2 domain: x = s * cs ----
       if (valid < kTileKV) {
 #pragma unroll
         for (int mt = 0; mt < 2; ++mt)
 #pragma unroll
           for (int i = 0; i < 16; ++i) {
             const int kv = mt * 32 + (i >> 2) * 8 + g * 4 + (i & 3);
-            if (kv >= valid) s[mt][i] = kNegInf;
+            if (kv >= valid) s[mt][i] = -INFINITY;  // p = 0 whatever the scale
           }
       }
       float mx = s[0][0];
@@ -326,13 +398,13 @@ __global__ void __launch_bounds__(kThreads) sparse_fa_kernel(const FaParams p) {
       for (int mt = 0; mt < 2; ++mt)
 #pragma unroll
         for (int i = 0; i < 16; ++i) mx = fmaxf(mx, s[mt][i]);
-      mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
-      // The running max is only raised when a row's new max exceeds it by more than 2^kLazyLog2
+      mx = fmaxf(mx, __shfl_xor(mx, 32, 64)) * cs;
+      // The running max is only raised when a row's new max exceeds it by more than kLazyLog2
       // (p then stays <= 2^kLazyLog2, harmless in fp32 / bf16 / fp16): the rescale of O leaves the
       // steady-state path.
-      if (__builtin_expect(__any((mx - m_run) * c > kLazyLog2), 0)) {
+      if (__builtin_expect(__any(mx - m_run > kLazyLog2), 0)) {
         const float m_new = fmaxf(m_run, mx);
-        const float scale = __builtin_amdgcn_exp2f((m_run - m_new) * c);
+        const float scale = __builtin_amdgcn_exp2f(m_run - m_new);
         d_part *= scale;
 #pragma unroll
         for (int dt = 0; dt < 4; ++dt)
@@ -340,14 +412,13 @@ __global__ void __launch_bounds__(kThreads) sparse_fa_kernel(const FaParams p) {
           for (int i = 0; i < 16; ++i) o_acc[dt][i] *= scale;
         m_run = m_new;
       }
-      const float mc = m_run * c;
       x8 pb[4];
       float psum = 0.f;
 #pragma unroll
       for (int mt = 0; mt < 2; ++mt)
 #pragma unroll
         for (int i = 0; i < 16; ++i) {
-          const float e = __builtin_amdgcn_exp2f(__builtin_fmaf(s[mt][i], c, -mc));
+          const float e = __builtin_amdgcn_exp2f(__builtin_fmaf(s[mt][i], cs, -m_run));
           psum += e;
           pb[mt * 2 + (i >> 3)][i & 7] = static_cast<T>(e);
         }
@@ -382,8 +453,8 @@ __global__ void __launch_bounds__(kThreads) sparse_fa_kernel(const FaParams p) {
     if (kg == 0) {
       const float m1 = md[(qs * 64 + lane) * 2 + 0], d1 = md[(qs * 64 + lane) * 2 + 1];
       const float m = fmaxf(m_run, m1);
-      const float a0 = __builtin_amdgcn_exp2f((m_run - m) * c);
-      const float a1 = __builtin_amdgcn_exp2f((m1 - m) * c);
+      const float a0 = __builtin_amdgcn_exp2f(m_run - m);
+      const float a1 = __builtin_amdgcn_exp2f(m1 - m);
       const float d_lane = d_part * a0 + d1 * a1;
       const float d_tot = d_lane + __shfl_xor(d_lane, 32, 64);
       const float inv = __builtin_amdgcn_rcpf(d_tot);
@@ -402,7 +473,7 @@ __global__ void __launch_bounds__(kThreads) sparse_fa_kernel(const FaParams p) {
             *reinterpret_cast<x4*>(dst + dt * 32 + i4 * 8 + g * 4) = out;
           }
         if (p.lse && g == 0)
-          p.lse[q_tok * p.num_heads + head] = __builtin_amdgcn_logf(d_tot) + m * c;
+          p.lse[q_tok * p.num_heads + head] = __builtin_amdgcn_logf(d_tot) + m;
       }
     }
   }
@@ -418,11 +489,12 @@ __global__ void __launch_bounds__(kThreads) sparse_fa_kernel(const FaParams p) {
   }
 }
 
-template <typename T>
+template <typename T, bool kFp8>
 int launch(const FaParams& p, int64_t max_rows, hipStream_t stream) {
+  constexpr int kSmemBytes = Geom<kFp8>::kSmemBytes;
   static bool attr_set = false;
   if (!attr_set) {
-    FO_HIP_CALL(hipFuncSetAttribute(reinterpret_cast<const void*>(&sparse_fa_kernel<T>),
+    FO_HIP_CALL(hipFuncSetAttribute(reinterpret_cast<const void*>(&sparse_fa_kernel<T, kFp8>),
                                     hipFuncAttributeMaxDynamicSharedMemorySize, kSmemBytes));
     attr_set = true;
   }
@@ -430,7 +502,7 @@ int launch(const FaParams& p, int64_t max_rows, hipStream_t stream) {
   if (num_cu <= 0) return fo::fail(FO_ERR_HIP, "sparse_fa: no device");
   int64_t grid = num_cu;  // one persistent workgroup per CU (LDS bound)
   if (grid > max_rows) grid = max_rows;
-  sparse_fa_kernel<T><<<static_cast<unsigned>(grid), kThreads, kSmemBytes, stream>>>(p);
+  sparse_fa_kernel<T, kFp8><<<static_cast<unsigned>(grid), kThreads, kSmemBytes, stream>>>(p);
   FO_CHECK_LAUNCH();
   return FO_OK;
 }
@@ -443,7 +515,8 @@ extern "C" int fo_sparse_fa_run(const void* q, const void* k, const void* v, voi
                                 int64_t k_stride_h, int64_t v_stride_n, int64_t v_stride_h,
                                 int64_t o_stride_n, int64_t o_stride_h, const int32_t* qo_indptr,
                                 const int32_t* kv_indptr, const int32_t* q_blk_base,
-                                const int32_t* kv_blk_base, const int32_t* row_req,
+                                const int32_t* kv_blk_base, int32_t n_q_blocks,
+                                int32_t n_kv_blocks, const int32_t* row_req,
                                 const int32_t* row_qb, const int32_t* row_head,
                                 const int32_t* kv_row_ptr, const int32_t* kv_idx,
                                 const int32_t* order, int32_t* sched, int64_t max_rows,
@@ -463,8 +536,11 @@ extern "C" int fo_sparse_fa_run(const void* q, const void* k, const void* v, voi
   const int64_t strides[8] = {q_stride_n, q_stride_h, k_stride_n, k_stride_h,
                               v_stride_n, v_stride_h, o_stride_n, o_stride_h};
   for (int i = 0; i < 8; ++i)
-    FO_REQUIRE(strides[i] % 8 == 0 && strides[i] > 0,
-               "sparse_fa: strides must be positive multiples of 8 elements (128-bit accesses)");
+    FO_REQUIRE(strides[i] % (dtype == FO_FP8_E4M3 && i < 4 ? 16 : 8) == 0 && strides[i] > 0,
+               "sparse_fa: strides must be positive multiples of 16 bytes (128-bit accesses)");
+  if (dtype == FO_FP8_E4M3)
+    FO_REQUIRE(q_scale && k_scale && q_blk_base && kv_blk_base && n_q_blocks > 0 && n_kv_blocks > 0,
+               "sparse_fa: fp8 q/k need q_scale, k_scale, the block numbering and the scale row lengths");
   for (const void* ptr : {q, k, v, static_cast<const void*>(o)})
     FO_REQUIRE((reinterpret_cast<uintptr_t>(ptr) & 15) == 0,
                "sparse_fa: q/k/v/o must be 16-byte aligned");
@@ -478,10 +554,10 @@ extern "C" int fo_sparse_fa_run(const void* q, const void* k, const void* v, voi
   p.q_blk_base = q_blk_base; p.kv_blk_base = kv_blk_base;
   p.row_req = row_req; p.row_qb = row_qb; p.row_head = row_head;
   p.kv_row_ptr = kv_row_ptr; p.kv_idx = kv_idx; p.order = order; p.sched = sched;
-  p.num_heads = num_heads; p.n_q_blocks = 0; p.n_kv_blocks = 0;
+  p.num_heads = num_heads; p.n_q_blocks = n_q_blocks; p.n_kv_blocks = n_kv_blocks;
   p.sm_scale_log2 = sm_scale * 1.44269504088896340736f;
   hipStream_t s = static_cast<hipStream_t>(stream);
-  if (dtype == FO_BF16) return launch<__bf16>(p, max_rows, s);
-  if (dtype == FO_F16) return launch<_Float16>(p, max_rows, s);
-  return fo::fail(FO_ERR_INVALID, "sparse_fa: the fp8 path is not built yet");
+  if (dtype == FO_BF16) return launch<__bf16, false>(p, max_rows, s);
+  if (dtype == FO_F16) return launch<_Float16, false>(p, max_rows, s);
+  return launch<__bf16, true>(p, max_rows, s);
 }

@@ -119,8 +119,8 @@ int fo_decode_sparse(const uint8_t* sparse_info, const uint8_t* sparse_kv_info,
  * q [nnz_q,H,D], k,v [nnz_kv,H,D], o [nnz_q,H,D]; strides in elements (the innermost stride is
  * 1).  dtype FO_BF16 / FO_F16: q,k,v,o share it.  dtype FO_FP8_E4M3: q and k are e4m3fn bytes
  * with dequantisation scales q_scale[H][n_q_blocks], k_scale[H][n_kv_blocks] (fp32, blocks
- * numbered request by request); v and o are bf16.  (The fp8 form has no counterpart in the
- * reference.)
+ * numbered request by request: q_blk_base / kv_blk_base [batch+1] give each request's first
+ * block); v and o are bf16.  (The fp8 form has no counterpart in the reference.)
  * Rows of the list write every output row of their q-block; q-blocks not in the list are left
  * untouched; a listed row with no kv block writes zeros and lse = -5e4.  lse (optional, fp32
  * [nnz_q,H]) is base 2: log2(sum 2^(s*c - m*c)) + m*c, c = sm_scale*log2(e).
@@ -134,8 +134,8 @@ int fo_sparse_fa_run(const void* q, const void* k, const void* v, void* o, float
                      int64_t q_stride_h, int64_t k_stride_n, int64_t k_stride_h,
                      int64_t v_stride_n, int64_t v_stride_h, int64_t o_stride_n,
                      int64_t o_stride_h, const int32_t* qo_indptr, const int32_t* kv_indptr,
-                     const int32_t* q_blk_base, const int32_t* kv_blk_base,
-                     const int32_t* row_req, const int32_t* row_qb, const int32_t* row_head,
+                     const int32_t* q_blk_base, const int32_t* kv_blk_base, int32_t n_q_blocks,
+                     int32_t n_kv_blocks, const int32_t* row_req, const int32_t* row_qb, const int32_t* row_head,
                      const int32_t* kv_row_ptr, const int32_t* kv_idx, const int32_t* order,
                      int32_t* sched, int64_t max_rows, int32_t num_heads, int32_t head_dim,
                      int32_t block_q, int32_t block_kv, float sm_scale, void* stream);
