@@ -7,20 +7,22 @@
 //           where unselected head slices are never loaded
 //           (reference: gemm/w16a16/gemm_reduction.cuh:77-95, 126-160).
 //
-// Tiling.  The skip flags have a 128 x 128 granularity, but a 128 x 128 workgroup tile with 64 x 64
-// wavefront tiles needs one LDS operand read per MFMA, and LDS reads saturate before the matrix
-// cores do.  So a workgroup (4 wavefronts, one per SIMD) computes a *pair* of flagged units that
-// share one operand:
-//   GEMM-Q: two flagged token blocks of the same head column (shared: the W tile)  -> 256 x 128
-//   GEMM-O: two column blocks of the same token block (shared: the A tile)         -> 128 x 256
-// Each wavefront owns a 128 x 64 piece (8 MFMA tiles of 32 x 32, 128 accumulators): six operand
-// reads feed eight MFMAs.  A small kernel first compacts the GEMM-Q flags of every head column
-// into the pair list (order inside the list is by column; the output does not depend on it).
+// Tiling.  The skip flags have a 128 x 128 granularity ("unit"), but a CU can pull only ~50-60 B/clk
+// from L2 while its matrix cores eat a 128 x 128 x 64 step in ~1000 clocks, so small workgroup
+// tiles starve.  A workgroup (8 wavefronts, two per SIMD) therefore computes a *quad*: two token
+// blocks x two column blocks that share their operand tiles (four 128 x BK tiles feed four units).
+// Every unit is owned by two wavefronts (64 rows x 128 columns each, 128 accumulators); six LDS
+// operand reads feed eight MFMAs.  A list kernel packs the flagged units of every
+// (16-token-block window, column pair) cell into quads: rows flagged in both columns pair up into
+// full quads, rows flagged in one column pair up among themselves, leftovers are merged; a 4-bit
+// mask says which units of a quad exist (the others are computed on duplicated tiles and dropped).
+// GEMM-O runs the same kernel over unflagged quads and walks the union of the two token blocks'
+// selected heads; a token block that does not select a head gets that k step's X operand zeroed.
 //
-// Data path.  BK = 64.  Operand tiles go global -> LDS directly (global_load_lds_dwordx4) into a
-// 3-stage ring, two k steps ahead of the math, one barrier per k step.  A wavefront's copy lands
-// on 1 KB of consecutive LDS (8 rows of 128 B), so rows are XOR-swizzled instead of padded: row r
-// keeps logical 16-byte chunk c at position c ^ ((r >> 1) & 7), applied on the global side; the
+// Data path.  BK = 32.  Operand tiles go global -> LDS directly (global_load_lds_dwordx4) into a
+// 4-stage ring, three k steps ahead of the math, one barrier per k step.  A wavefront's copy lands
+// on 1 KB of consecutive LDS (16 rows of 64 B), so rows are XOR-swizzled instead of padded: row r
+// keeps logical 16-byte chunk c at position c ^ ((r >> 2) & 3), applied on the global side; the
 // 128-bit operand reads of 16 consecutive rows then cover all 64 banks.
 //
 // The product is formed transposed (A operand = W rows, B operand = X rows) so that in the 32 x 32
@@ -29,12 +31,11 @@
 // fp32 accumulation starts from the init value converted to fp32; one round-to-nearest cast at
 // the end.
 //
-// Work order.  Workgroups are persistent (one per CU).  The work is cut into windows of 16 token
-// blocks; inside a window XCD x (= blockIdx % 8) takes the head columns congruent to x mod 8
-// (GEMM-Q) / the x-th contiguous eighth of the (column pair, token block) entries (GEMM-O).  The
-// ~32 workgroups of an XCD therefore work at the same time on a 16-token-block x few-column patch, whose operand tiles they share through that XCD's L2, and
-// all XCDs sweep the token windows together, so the activations stream from HBM once while the
-// weights stay in the memory-side cache.
+// Work order.  Workgroups are persistent (one per CU).  The quad list is ordered by token window,
+// then column pair, then row pair, and XCD x (= blockIdx % 8) owns the x-th contiguous eighth of it.
+// The ~32 workgroups of an XCD therefore work at the same time on one token window and four
+// neighbouring column pairs (16 + 8 operand tiles for 32 quads), whose tiles they share through
+// that XCD's L2.
 #include "fo_common.h"
 
 namespace {
@@ -45,23 +46,25 @@ typedef __attribute__((ext_vector_type(8))) _Float16 f16x8;
 typedef __attribute__((ext_vector_type(4))) _Float16 f16x4;
 typedef __attribute__((ext_vector_type(16))) float f32x16;
 typedef __attribute__((ext_vector_type(4))) float f32x4;
+typedef __attribute__((ext_vector_type(4))) unsigned int u32x4;
 typedef __attribute__((address_space(3))) void lds_void;
 typedef __attribute__((address_space(1))) const void glb_void;
 
-constexpr int kThreads = 256;
+constexpr int kThreads = 512;
 constexpr int kTile = 128;  // unit edge = granularity of the skip flags
-constexpr int kBK = 64;
-constexpr int kRowBytes = kBK * 2;                 // one LDS row: 64 elements, 8 chunks of 16 B
-constexpr int kUnitBytes = kTile * kRowBytes;      // one 128-row operand tile: 16 KB
-constexpr int kStageBytes = 3 * kUnitBytes;        // shared tile + two paired tiles
-constexpr int kStages = 3;
-constexpr int kSmemBytes = kStages * kStageBytes;  // 144 KB
-constexpr int kCopiesPerWave = 3 * kUnitBytes / 1024 / 4;  // 12 copy instructions per stage
+constexpr int kBK = 32;
+constexpr int kRowBytes = kBK * 2;                 // one LDS row: 32 elements, 4 chunks of 16 B
+constexpr int kUnitBytes = kTile * kRowBytes;      // one 128-row operand tile: 8 KB
+constexpr int kStageBytes = 4 * kUnitBytes;        // X0, X1, W0, W1
+constexpr int kStages = 4;
+constexpr int kSmemBytes = kStages * kStageBytes;  // 128 KB
+constexpr int kCopiesPerWave = kStageBytes / 1024 / 8;  // 4 copy instructions per wavefront per stage
 constexpr int kMaxHeads = 256;
+constexpr int kMaxSteps = 2048;  // GEMM-O: k steps of one work item (K <= 65536)
 constexpr int kXcds = 8;
-constexpr int kPairThreads = 256;
-constexpr int kPairScanThreads = 1024;
-constexpr int kWindow = 16;  // token blocks per scheduling window
+constexpr int kListThreads = 1024;
+constexpr int kWindow = 16;   // token blocks per scheduling window
+constexpr int kQuadInts = 8;  // b, r0, r1, c0, c1, valid mask, pad, pad
 
 template <typename T>
 struct Types;
@@ -89,8 +92,8 @@ struct GemmParams {
   void* y;           // [B, M, N]
   const uint8_t* sparse_info;
   const int32_t* sparse_info_indptr;
-  const int32_t* pairs;  // GEMM-Q: int4 (b, ix, iy0, iy1) per pair, queue by queue
-  const int32_t* qoff;   // GEMM-Q: qoff[0..8] queue boundaries inside `pairs`
+  const int32_t* quads;  // kQuadInts per quad, queue by queue
+  const int32_t* qoff;   // qoff[0..8] queue boundaries inside `quads`
   int32_t batch, m, n, k;
   int32_t sparse_q_size, num_heads, head_dim, num_text_tokens;
   int32_t flag;       // GEMM-Q: is_full.  GEMM-O: is_for_cached
@@ -109,362 +112,407 @@ __device__ __forceinline__ bool flag_bit(const uint8_t* info, uint32_t bit) {
 }
 
 // ---------------------------------------------------------------------------------------------
-// GEMM-Q pair list.  A cell = (batch, window of 16 token blocks, head column); its flagged token
-// blocks are paired up (an odd one out is paired with -1).  Cells are laid out queue by queue
-// (queue x = columns congruent to x mod 8), window-major inside a queue; qoff[0..8] delimit the
-// queues.  One workgroup: every thread owns a contiguous range of cells in that order.
+// Quad list.  A cell = (batch, window of 16 token blocks, column pair); cells are ordered batch,
+// window, column pair.  One workgroup counts the quads of every cell (flagged-row masks of its two
+// columns), scans the counts, emits every cell's quads at its offset, and cuts the list into eight
+// contiguous, equally long queues.
 // ---------------------------------------------------------------------------------------------
-struct PairGeom {
-  int32_t batch, n_row_tiles, n_col_tiles, n_win, cols_per_q;
+struct ListGeom {
+  int32_t batch, n_row_tiles, n_col_tiles, n_win, n_cp;  // windows per batch, column pairs
 };
 
-__device__ __forceinline__ uint32_t cell_mask(const PairGeom& gm, int64_t key,
-                                              const uint8_t* __restrict__ sparse_info,
-                                              const int32_t* __restrict__ sparse_info_indptr,
-                                              int32_t sparse_q_size, int32_t num_heads,
-                                              int32_t head_dim, int32_t num_text_tokens, int is_full,
-                                              int* b_out, int* col_out, int* row0_out) {
-  // key = ((x * batch + b) * n_win + w) * cols_per_q + ci,  column = ci*8 + x
-  const int ci = static_cast<int>(key % gm.cols_per_q);
-  int64_t t = key / gm.cols_per_q;
-  const int w = static_cast<int>(t % gm.n_win);
-  t /= gm.n_win;
-  const int b = static_cast<int>(t % gm.batch);
-  const int x = static_cast<int>(t / gm.batch);
-  const int col = ci * kXcds + x;
+__device__ __forceinline__ void cell_masks(const ListGeom& gm, int cell, bool use_flags,
+                                           const uint8_t* __restrict__ sparse_info,
+                                           const int32_t* __restrict__ sparse_info_indptr,
+                                           int32_t sparse_q_size, int32_t num_heads, int32_t head_dim,
+                                           int32_t num_text_tokens, int* b_out, int* row0_out,
+                                           int* cp_out, uint32_t* m0, uint32_t* m1) {
+  const int cp = cell % gm.n_cp;
+  const int t = cell / gm.n_cp;
+  const int w = t % gm.n_win, b = t / gm.n_win;
   *b_out = b;
-  *col_out = col;
   *row0_out = w * kWindow;
-  if (col >= gm.n_col_tiles) return 0u;
+  *cp_out = cp;
   const int rows = min(kWindow, gm.n_row_tiles - w * kWindow);
-  if (is_full) return (1u << rows) - 1u;
-  const uint8_t* info = sparse_info + sparse_info_indptr[b];
-  uint32_t mask = 0;
-  for (int r = 0; r < rows; ++r) {
-    const uint32_t bit = static_cast<uint32_t>(num_text_tokens + (w * kWindow + r) * kTile) / sparse_q_size *
-                             num_heads + static_cast<uint32_t>(col * kTile) / head_dim;
-    mask |= static_cast<uint32_t>(flag_bit(info, bit)) << r;
+  const uint32_t all = (1u << rows) - 1u;
+  const bool has1 = 2 * cp + 1 < gm.n_col_tiles;
+  if (!use_flags) {
+    *m0 = all;
+    *m1 = has1 ? all : 0u;
+    return;
   }
-  return mask;
+  const uint8_t* info = sparse_info + sparse_info_indptr[b];
+  uint32_t a0 = 0, a1 = 0;
+  for (int r = 0; r < rows; ++r) {
+    const uint32_t base =
+        static_cast<uint32_t>(num_text_tokens + (w * kWindow + r) * kTile) / sparse_q_size * num_heads;
+    a0 |= static_cast<uint32_t>(flag_bit(info, base + static_cast<uint32_t>(2 * cp * kTile) / head_dim)) << r;
+    if (has1)
+      a1 |= static_cast<uint32_t>(
+                flag_bit(info, base + static_cast<uint32_t>((2 * cp + 1) * kTile) / head_dim)) << r;
+  }
+  *m0 = a0;
+  *m1 = a1;
 }
 
-__global__ void __launch_bounds__(kPairScanThreads) gemm_q_pairs_kernel(
-    const uint8_t* __restrict__ sparse_info, const int32_t* __restrict__ sparse_info_indptr,
-    PairGeom gm, int32_t sparse_q_size, int32_t num_heads, int32_t head_dim,
-    int32_t num_text_tokens, int is_full, int32_t* __restrict__ pairs, int32_t* __restrict__ qoff) {
-  __shared__ int32_t s_scan[kPairScanThreads];
-  const int tid = threadIdx.x;
-  const int64_t per_q = static_cast<int64_t>(gm.batch) * gm.n_win * gm.cols_per_q;
-  const int64_t n_keys = per_q * kXcds;
-  const int64_t chunk = (n_keys + kPairScanThreads - 1) / kPairScanThreads;
-  const int64_t lo = tid * chunk, hi = lo + chunk < n_keys ? lo + chunk : n_keys;
-  int b, col, row0;
-  int32_t mine = 0;
-  for (int64_t key = lo; key < hi; ++key)
-    mine += (__popc(cell_mask(gm, key, sparse_info, sparse_info_indptr, sparse_q_size, num_heads, head_dim,
-                              num_text_tokens, is_full, &b, &col, &row0)) + 1) >> 1;
-  s_scan[tid] = mine;
-  __syncthreads();
-  for (int off = 1; off < kPairScanThreads; off <<= 1) {
-    const int32_t v = tid >= off ? s_scan[tid - off] : 0;
-    __syncthreads();
-    s_scan[tid] += v;
-    __syncthreads();
+__device__ __forceinline__ int pop_lowest(uint32_t* m) {
+  const int r = __ffs(*m) - 1;
+  *m &= *m - 1;
+  return r;
+}
+
+// Packs a cell's flagged units into quads and calls f(r0, r1, valid) for each; r1 < 0 = no second
+// row.  valid bits: 1 = (r0,c0), 2 = (r0,c1), 4 = (r1,c0), 8 = (r1,c1).
+template <typename F>
+__device__ __forceinline__ void for_each_quad(uint32_t m0, uint32_t m1, F&& f) {
+  uint32_t both = m0 & m1, only0 = m0 & ~m1, only1 = m1 & ~m0;
+  while (__popc(both) >= 2) {
+    const int r0 = pop_lowest(&both), r1 = pop_lowest(&both);
+    f(r0, r1, 0xF);
   }
-  int32_t pos = s_scan[tid] - mine;
-  if (tid == kPairScanThreads - 1) qoff[kXcds] = s_scan[tid];
-  for (int64_t key = lo; key < hi; ++key) {
-    if (key % per_q == 0) qoff[key / per_q] = pos;  // a queue starts here
-    uint32_t mask = cell_mask(gm, key, sparse_info, sparse_info_indptr, sparse_q_size, num_heads, head_dim,
-                              num_text_tokens, is_full, &b, &col, &row0);
-    while (mask) {
-      const int r0 = __ffs(mask) - 1;
-      mask &= mask - 1;
-      int r1 = -1;
-      if (mask) {
-        r1 = __ffs(mask) - 1;
-        mask &= mask - 1;
-      }
-      int32_t* e = pairs + 4 * static_cast<int64_t>(pos++);
-      e[0] = b;
-      e[1] = col;
-      e[2] = row0 + r0;
-      e[3] = r1 < 0 ? -1 : row0 + r1;
+  while (__popc(only0) >= 2) {
+    const int r0 = pop_lowest(&only0), r1 = pop_lowest(&only0);
+    f(r0, r1, 0x5);
+  }
+  while (__popc(only1) >= 2) {
+    const int r0 = pop_lowest(&only1), r1 = pop_lowest(&only1);
+    f(r0, r1, 0xA);
+  }
+  // at most one row left in each class: merge them two by two
+  if (both) {
+    const int r0 = pop_lowest(&both);
+    if (only0) {
+      f(r0, pop_lowest(&only0), 0x3 | 0x4);
+    } else if (only1) {
+      f(r0, pop_lowest(&only1), 0x3 | 0x8);
+    } else {
+      f(r0, -1, 0x3);
     }
   }
-  // queues past the last key range (possible when n_keys < threads) start at the total
-  if (tid == 0 && n_keys == 0)
-    for (int x = 0; x < kXcds; ++x) qoff[x] = 0;
+  if (only0 && only1) {
+    const int r0 = pop_lowest(&only0);
+    f(r0, pop_lowest(&only1), 0x1 | 0x8);
+  } else if (only0) {
+    f(pop_lowest(&only0), -1, 0x1);
+  } else if (only1) {
+    f(pop_lowest(&only1), -1, 0x2);
+  }
+}
+
+struct ListArgs {
+  const uint8_t* sparse_info;
+  const int32_t* sparse_info_indptr;
+  int32_t use_flags;  // GEMM-Q without is_full: units come from the flags
+  int32_t sparse_q_size, num_heads, head_dim, num_text_tokens;
+};
+
+__global__ void __launch_bounds__(kListThreads) gemm_quads_kernel(ListArgs a, ListGeom gm,
+                                                                  int32_t* __restrict__ quads,
+                                                                  int32_t* __restrict__ qoff) {
+  __shared__ int32_t s_cnt[kListThreads];
+  const int tid = threadIdx.x;
+  const int n_cells = gm.batch * gm.n_win * gm.n_cp;
+  int b, row0, cp;
+  uint32_t m0, m1;
+  // every thread owns a contiguous run of cells: quad counts, then a block-wide scan
+  const int per = (n_cells + kListThreads - 1) / kListThreads;
+  const int lo = min(tid * per, n_cells), hi = min(lo + per, n_cells);
+  int32_t my_cnt = 0;
+  for (int cell = lo; cell < hi; ++cell) {
+    cell_masks(gm, cell, a.use_flags, a.sparse_info, a.sparse_info_indptr, a.sparse_q_size, a.num_heads,
+               a.head_dim, a.num_text_tokens, &b, &row0, &cp, &m0, &m1);
+    for_each_quad(m0, m1, [&](int, int, int) { ++my_cnt; });
+  }
+  s_cnt[tid] = my_cnt;
+  __syncthreads();
+  for (int d = 1; d < kListThreads; d <<= 1) {
+    const int32_t v = tid >= d ? s_cnt[tid - d] : 0;
+    __syncthreads();
+    s_cnt[tid] += v;
+    __syncthreads();
+  }
+  const int32_t total = s_cnt[kListThreads - 1];
+  if (tid <= kXcds) qoff[tid] = static_cast<int32_t>(static_cast<int64_t>(total) * tid / kXcds);
+  int32_t q = s_cnt[tid] - my_cnt;
+  for (int cell = lo; cell < hi; ++cell) {
+    cell_masks(gm, cell, a.use_flags, a.sparse_info, a.sparse_info_indptr, a.sparse_q_size, a.num_heads,
+               a.head_dim, a.num_text_tokens, &b, &row0, &cp, &m0, &m1);
+    for_each_quad(m0, m1, [&](int r0, int r1, int valid) {
+      int32_t* e = quads + kQuadInts * static_cast<int64_t>(q);
+      e[0] = b;
+      e[1] = row0 + r0;
+      e[2] = row0 + (r1 < 0 ? r0 : r1);
+      e[3] = (valid & 0x5) ? 2 * cp : 2 * cp + 1;
+      e[4] = (valid & 0xA) ? 2 * cp + 1 : 2 * cp;
+      e[5] = valid;
+      ++q;
+    });
+  }
 }
 
 // ---------------------------------------------------------------------------------------------
-// Main kernel.  kReduce = false: GEMM-Q (pair = two token blocks, shared = W tile).
-//               kReduce = true : GEMM-O (pair = two column blocks, shared = A tile).
+// Main kernel.  kReduce = false: GEMM-Q.  kReduce = true: GEMM-O.
 // ---------------------------------------------------------------------------------------------
 template <typename T, bool kReduce>
 __global__ void __launch_bounds__(kThreads) gemm_kernel(const GemmParams p) {
   using TT = Types<T>;
   using x8 = typename TT::x8;
   using x4 = typename TT::x4;
-  // accumulator tile of a wavefront, transposed product: NT n-tiles (W rows) x MT m-tiles (X rows)
-  constexpr int NT = kReduce ? 4 : 2;
-  constexpr int MT = kReduce ? 2 : 4;
+  constexpr int NT = 4, MT = 2;  // wavefront tile: 128 columns (W rows) x 64 token rows (X rows)
   extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
-  __shared__ int32_t s_heads[kMaxHeads];
+  __shared__ int32_t s_heads[kMaxHeads + 1];  // GEMM-O: head | (row0 selects) << 16 | (row1 selects) << 17
   __shared__ int32_t s_nsel;
+  // GEMM-O: per k step, k offset | (row0 selects) << 16 | (row1 selects) << 17; four entries past
+  // the end repeat the last step
+  __shared__ int32_t s_step[kReduce ? kMaxSteps + 4 : 1];
 
-  const int tid = threadIdx.x, lane = tid & 63, wv = tid >> 6;
+  const int tid = threadIdx.x, lane = tid & 63;
+  const int wv = __builtin_amdgcn_readfirstlane(tid >> 6);  // wavefront index, kept scalar
   const int l32 = lane & 31, g = lane >> 5;
-  const int wp = wv >> 1, wh = wv & 1;  // which unit of the pair / which half of the shared side
+  const int wr = wv >> 2, wc = (wv >> 1) & 1, wh = wv & 1;  // token block, column block, row half
 
   const T* __restrict__ xg = static_cast<const T*>(p.x);
   const T* __restrict__ wg = static_cast<const T*>(p.w);
 
-  // copy assignment: per stage 48 copy instructions (n = 0..47), 8 LDS rows each; wavefront wv
-  // issues n = 4*j + wv.  Instruction n fills rows 8*(n%16).. of tile n/16 (0 = shared, 1,2 = pair).
-  // Lane i lands on row 8*(n%16) + i/8 at chunk position i%8 and must fetch logical chunk
-  // (i%8) ^ ((row >> 1) & 7); (row >> 1) & 7 = (4*(n%2) + i/16) & 7 and n%2 = wv%2.
-  const int cp_row = lane >> 3;
-  const int cp_chunk = ((lane & 7) ^ ((4 * (wv & 1) + (lane >> 4)) & 7)) * 8;  // element offset
-  // operand reads: row r = tile row base + l32, logical chunk 2*ks + g -> position ^ ((r >> 1) & 7)
-  const int rd_x = (g ^ ((l32 >> 1) & 7)) << 4;  // xor-ed with ks << 5 at use; tile bases are
-                                                 // multiples of 32 rows, so they do not change it
+  // copy assignment: per stage 32 copy instructions, 16 LDS rows each; wavefront wv issues the
+  // rows 16*wv.. of each of the four tiles (0,1 = X of token block 0,1; 2,3 = W of column block
+  // 0,1).  Lane i lands on row 16*wv + i/4 at chunk position i%4 and must fetch logical chunk
+  // (i%4) ^ ((row >> 2) & 3) = (i%4) ^ ((i >> 4) & 3).
+  const int cp_row = 16 * wv + (lane >> 2);
+  const int cp_chunk = ((lane & 3) ^ ((lane >> 4) & 3)) * 8;  // element offset inside the k step
+  // operand reads: row = tile row base + l32 (bases are multiples of 32), logical chunk 2*ks + g
+  const int rd_swz = (l32 >> 2) & 3;
 
-  // persistent work loop: XCD x (= blockIdx % 8) walks queue x, one entry per workgroup per round
   const int xcd = blockIdx.x & (kXcds - 1), slot = blockIdx.x >> 3;
   const int per_xcd = gridDim.x >> 3;  // host launches a multiple of 8 workgroups
-  const int n_row_tiles = (p.m + kTile - 1) / kTile;
-  int q_lo, q_len;  // GEMM-Q: range of `pairs`; GEMM-O: q_len entries, decoded in closed form
-  // GEMM-O: a window holds rows x n_col_pairs entries in (column pair, token block) order and
-  // XCD x owns the x-th contiguous eighth of every window
-  const int n_col_pairs = (p.n / kTile + 1) / 2;
-  const int full_w = n_row_tiles / kWindow, rem_rows = n_row_tiles % kWindow;
-  const int chunk_full = kWindow * n_col_pairs / kXcds;  // 16 * P is a multiple of 8
-  const int last_lo = rem_rows * n_col_pairs * xcd / kXcds;
-  const int last_len = rem_rows * n_col_pairs * (xcd + 1) / kXcds - last_lo;
-  const int per_b = full_w * chunk_full + last_len;
-  if constexpr (kReduce) {
-    q_lo = 0;
-    q_len = p.batch * per_b;
-  } else {
-    q_lo = p.qoff[xcd];
-    q_len = p.qoff[xcd + 1] - q_lo;
-  }
+  const int q_lo = p.qoff[xcd], q_len = p.qoff[xcd + 1] - q_lo;
 
   for (int work = slot; work < q_len; work += per_xcd) {
-    // ---- decode the work item ----
-    int bz, iy[2], ix[2];  // unit u of the pair is output tile (iy[u], ix[u]); -1 = absent
-    if constexpr (kReduce) {
-      bz = work / per_b;
-      const int rem = work - bz * per_b;
-      int wdw, idx, rows;
-      if (rem < full_w * chunk_full) {
-        wdw = rem / chunk_full;
-        idx = xcd * chunk_full + (rem - wdw * chunk_full);
-        rows = kWindow;
-      } else {
-        wdw = full_w;
-        idx = last_lo + (rem - full_w * chunk_full);
-        rows = rem_rows;
-      }
-      const int jp = idx / rows, rr = idx - jp * rows;
-      iy[0] = iy[1] = wdw * kWindow + rr;
-      ix[0] = 2 * jp;
-      ix[1] = (2 * jp + 1) * kTile < p.n ? 2 * jp + 1 : -1;
-    } else {
-      const int32_t* e = p.pairs + 4 * static_cast<int64_t>(q_lo + work);
-      bz = e[0];
-      ix[0] = ix[1] = e[1];
-      iy[0] = e[2];
-      iy[1] = e[3];
-      if (iy[1] < 0) ix[1] = -1;
-    }
-    const bool has2 = ix[1] >= 0;
-    const bool my_valid = wp == 0 || has2;
+    const int32_t* e = p.quads + kQuadInts * static_cast<int64_t>(q_lo + work);
+    const int bz = e[0], valid = e[5];
+    const int r[2] = {e[1], e[2]}, c[2] = {e[3], e[4]};
+    const bool my_valid = (valid >> (wr * 2 + wc)) & 1;
 
     // ---- k-step list ----
     int n_iter;
+    __builtin_amdgcn_s_waitcnt(0x0f70);  // this wavefront's copies and stores of the previous work item
     __syncthreads();  // previous work item: LDS tiles and s_heads are free
     if constexpr (kReduce) {
       if (wv == 0) {
         const uint8_t* info = p.sparse_info + p.sparse_info_indptr[bz];
-        const uint32_t flag_base =
-            static_cast<uint32_t>(p.num_text_tokens + iy[0] * kTile) / p.sparse_q_size * p.num_heads;
+        const uint32_t base0 =
+            static_cast<uint32_t>(p.num_text_tokens + r[0] * kTile) / p.sparse_q_size * p.num_heads;
+        const uint32_t base1 =
+            static_cast<uint32_t>(p.num_text_tokens + r[1] * kTile) / p.sparse_q_size * p.num_heads;
+        const bool want1 = (valid & 0xC) != 0;
+        const bool pick = p.flag == 0;  // final pass picks bit 1, cache pass bit 0
         int count = 0;
         const int n_slices = p.k / p.head_dim;
         for (int h0 = 0; h0 < n_slices; h0 += 64) {
           const int h = h0 + lane;
-          bool sel = false;
+          bool s0 = false, s1 = false;
           if (h < n_slices) {
-            const bool one = flag_bit(info, flag_base + h);
-            sel = p.flag ? !one : one;
+            s0 = flag_bit(info, base0 + h) == pick;
+            s1 = want1 && (flag_bit(info, base1 + h) == pick);
           }
-          const unsigned long long mask = __ballot(sel);
-          if (sel) s_heads[count + __popcll(mask & ((1ull << lane) - 1ull))] = h;
+          const unsigned long long mask = __ballot(s0 || s1);
+          if (s0 || s1)
+            s_heads[count + __popcll(mask & ((1ull << lane) - 1ull))] = h | (s0 << 16) | (s1 << 17);
           count += __popcll(mask);
         }
         if (lane == 0) s_nsel = count;
       }
       __syncthreads();
-      n_iter = s_nsel * (p.head_dim / kBK);
-    } else {
-      n_iter = p.k / kBK;  // full k steps; a 32-wide K tail is finished after the loop
-    }
-    const int iters_per_head = kReduce ? p.head_dim / kBK : 1;
-    auto k_of = [&](int it) -> int {
-      if constexpr (kReduce) {
-        return s_heads[it / iters_per_head] * p.head_dim + (it % iters_per_head) * kBK;
-      } else {
-        return it * kBK;
+      const int iph = p.head_dim / kBK;
+      n_iter = s_nsel * iph;
+      if (n_iter > 0) {
+        for (int i = tid; i < n_iter + 4; i += kThreads) {
+          const int ii = i < n_iter ? i : n_iter - 1;
+          const int hv = s_heads[ii / iph];
+          s_step[i] = ((hv & 0xFFFF) * p.head_dim + (ii % iph) * kBK) | (hv & 0x30000);
+        }
       }
-    };
+      __syncthreads();
+    } else {
+      n_iter = p.k / kBK;
+    }
 
-    // ---- global row pointers of the three operand tiles (tile 0 = shared, 1/2 = the pair) ----
-    // GEMM-Q: shared = W rows of column ix, pair = X rows of token blocks iy[0], iy[1]
-    // GEMM-O: shared = X rows of token block iy, pair = W rows of column blocks ix[0], ix[1]
-    const T* tile_base[3];
-    int tile_rows[3];  // valid rows (clamp for the M tail)
+    // ---- global row pointers of the four operand tiles: X(r0), X(r1), W(c0), W(c1) ----
+    // this wavefront copies rows 16*wv.. of each; rows past M are clamped (their results are dropped)
+    const T* cp_src[4];
     {
       const T* xb = xg + static_cast<int64_t>(bz) * p.m * p.k;
-      if constexpr (kReduce) {
-        tile_base[0] = xb + static_cast<int64_t>(iy[0]) * kTile * p.k;
-        tile_rows[0] = min(kTile, p.m - iy[0] * kTile);
-        for (int u = 0; u < 2; ++u) {
-          const int c = has2 || u == 0 ? ix[u] : ix[0];
-          tile_base[1 + u] = wg + static_cast<int64_t>(c) * kTile * p.k;
-          tile_rows[1 + u] = kTile;
-        }
-      } else {
-        tile_base[0] = wg + static_cast<int64_t>(ix[0]) * kTile * p.k;
-        tile_rows[0] = kTile;
-        for (int u = 0; u < 2; ++u) {
-          const int r = has2 || u == 0 ? iy[u] : iy[0];
-          tile_base[1 + u] = xb + static_cast<int64_t>(r) * kTile * p.k;
-          tile_rows[1 + u] = min(kTile, p.m - r * kTile);
-        }
+#pragma unroll
+      for (int u = 0; u < 2; ++u) {
+        int xr = r[u] * kTile + cp_row;
+        xr = xr < p.m ? xr : p.m - 1;
+        cp_src[u] = xb + static_cast<int64_t>(xr) * p.k + cp_chunk;
+        cp_src[2 + u] = wg + static_cast<int64_t>(c[u] * kTile + cp_row) * p.k + cp_chunk;
       }
     }
-    auto copy_stage = [&](int it) {
-      const int k0 = k_of(it);
-      uint8_t* dst = smem + (it % kStages) * kStageBytes;
-#pragma unroll
-      for (int j = 0; j < kCopiesPerWave; ++j) {
-        const int n = 4 * j + wv;         // 0..47
-        const int tile = j >> 2;          // n / 16 (4*j + wv < 16 <=> j < 4)
-        int r = 8 * (n & 15) + cp_row;
-        r = r < tile_rows[tile] ? r : tile_rows[tile] - 1;
-        copy16_to_lds(tile_base[tile] + static_cast<int64_t>(r) * p.k + k0 + cp_chunk, dst + n * 1024);
+    // k offset of step it (steps past the end repeat the last one); GEMM-O: plus the select bits
+    auto step_entry = [&](int it) -> int {
+      if constexpr (kReduce) {
+        return s_step[it];
+      } else {
+        return (it < n_iter ? it : n_iter - 1) * kBK;
       }
+    };
+    auto copy_one = [&](int it, int entry, int j) {
+      uint8_t* dst = smem + (it % kStages) * kStageBytes + wv * 1024;
+      copy16_to_lds(cp_src[j] + (entry & 0xFFFF), dst + j * kUnitBytes);
+    };
+    auto copy_stage = [&](int it) {
+      const int entry = step_entry(it);
+#pragma unroll
+      for (int j = 0; j < kCopiesPerWave; ++j) copy_one(it, entry, j);
     };
 
     // ---- accumulators, initialised from bias / cached partial ----
     // acc[nt][mt][i]: n = n0 + nt*32 + (i/4)*8 + g*4 + i%4, m = m0 + mt*32 + l32
-    const int my_iy = kReduce ? iy[0] : iy[wp], my_ix = kReduce ? ix[wp] : ix[0];
-    const int m0 = (my_valid ? my_iy : 0) * kTile + (kReduce ? wh * 64 : 0);
-    const int n0 = (my_valid ? my_ix : 0) * kTile + (kReduce ? 0 : wh * 64);
+    // All init loads are issued before the first copies and converted after them; vector-memory
+    // loads return in order, so "tile 0 landed" below also covers them.
+    const int m0 = r[wr] * kTile + wh * 64;
+    const int n0 = c[wc] * kTile;
     const int64_t y_batch = static_cast<int64_t>(bz) * p.m * p.n;
-    f32x16 acc[NT][MT];
+    int64_t row_off[MT];
 #pragma unroll
-    for (int nt = 0; nt < NT; ++nt)
-#pragma unroll
-      for (int mt = 0; mt < MT; ++mt) {
-        const int mrow = m0 + mt * 32 + l32;
-        const int mrow_c = mrow < p.m ? mrow : p.m - 1;
-#pragma unroll
-        for (int i4 = 0; i4 < 4; ++i4) {
-          const int ncol = n0 + nt * 32 + i4 * 8 + g * 4;
-          f32x4 init = {0.f, 0.f, 0.f, 0.f};
-          if (p.bias_kind == FO_BIAS_VECTOR) {
-            const x4 bv = *reinterpret_cast<const x4*>(static_cast<const T*>(p.bias) + ncol);
-#pragma unroll
-            for (int j = 0; j < 4; ++j) init[j] = static_cast<float>(bv[j]);
-          } else if (p.bias_kind == FO_BIAS_MATRIX) {
-            const int64_t off = y_batch + static_cast<int64_t>(mrow_c) * p.n + ncol;
-            if (p.bias_f32) {
-              init = *reinterpret_cast<const f32x4*>(static_cast<const float*>(p.bias) + off);
-            } else {
-              const x4 bv = *reinterpret_cast<const x4*>(static_cast<const T*>(p.bias) + off);
-#pragma unroll
-              for (int j = 0; j < 4; ++j) init[j] = static_cast<float>(bv[j]);
-            }
-          }
-#pragma unroll
-          for (int j = 0; j < 4; ++j) acc[nt][mt][i4 * 4 + j] = init[j];
-        }
-      }
-
-    // LDS row bases of this wavefront's operands inside a stage
-    // A operand (W rows): GEMM-Q shared tile rows wh*64.., GEMM-O pair tile wp rows 0..
-    // B operand (X rows): GEMM-Q pair tile wp rows 0..,   GEMM-O shared tile rows wh*64..
-    const int a_base = (kReduce ? (1 + wp) * kUnitBytes : wh * 64 * kRowBytes) + l32 * kRowBytes;
-    const int b_base = (kReduce ? wh * 64 * kRowBytes : (1 + wp) * kUnitBytes) + l32 * kRowBytes;
-
-    // ---- main loop: copies run two k steps ahead ----
-    if (n_iter > 0) copy_stage(0);
-    if (n_iter > 1) copy_stage(1);
-    for (int it = 0; it < n_iter; ++it) {
-      // tile `it` of this wavefront has landed (the 12 copies of tile it+1 may still be in flight)
-      if (it + 1 < n_iter) {
-        __builtin_amdgcn_s_waitcnt(0x0f70 | (kCopiesPerWave & 15));  // vmcnt(12)
-      } else {
-        __builtin_amdgcn_s_waitcnt(0x0f70);  // vmcnt(0)
-      }
-      __syncthreads();  // everyone's copies of tile `it` landed; stage (it+2)%3 is no longer read
-      if (it + 2 < n_iter) copy_stage(it + 2);
-      // (a wavefront whose unit is absent computes on the duplicated tile and drops the result:
-      // no branch in the loop body)
-      const uint8_t* st = smem + (it % kStages) * kStageBytes;
-      // operand registers are double-buffered: the reads of k step ks+1 are issued before the
-      // MFMAs of k step ks (a single wavefront per SIMD has no other way to hide LDS latency)
-      x8 a[2][NT], b[2][MT];
-      auto load_ops = [&](int buf, int ks) {
-        const int sw = rd_x ^ (ks << 5);
-#pragma unroll
-        for (int nt = 0; nt < NT; ++nt)
-          a[buf][nt] = *reinterpret_cast<const x8*>(st + a_base + nt * 32 * kRowBytes + sw);
-#pragma unroll
-        for (int mt = 0; mt < MT; ++mt)
-          b[buf][mt] = *reinterpret_cast<const x8*>(st + b_base + mt * 32 * kRowBytes + sw);
-      };
-      load_ops(0, 0);
+    for (int mt = 0; mt < MT; ++mt) {
+      const int mrow = m0 + mt * 32 + l32;
+      row_off[mt] = y_batch + static_cast<int64_t>(mrow < p.m ? mrow : p.m - 1) * p.n + n0 + g * 4;
+    }
+    auto first_copies = [&]() {
       __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
-      for (int ks = 0; ks < kBK / 16; ++ks) {
-        if (ks + 1 < kBK / 16) load_ops((ks + 1) & 1, ks + 1);
-        __builtin_amdgcn_sched_barrier(0);
+      for (int s = 0; s < kStages - 1; ++s)
+        if (n_iter > 0) copy_stage(s);
+      __builtin_amdgcn_sched_barrier(0);
+    };
+    f32x16 acc[NT][MT];
+    // the previous work item's stores are complete: from here on vmcnt counts loads only
+    __builtin_amdgcn_s_waitcnt(0x0f70);
+    if (p.bias_kind == FO_BIAS_VECTOR) {
+      x4 bv[NT][4];
 #pragma unroll
-        for (int nt = 0; nt < NT; ++nt)
+      for (int nt = 0; nt < NT; ++nt)
 #pragma unroll
-          for (int mt = 0; mt < MT; ++mt)
-            acc[nt][mt] = TT::mfma(a[ks & 1][nt], b[ks & 1][mt], acc[nt][mt]);
-        __builtin_amdgcn_sched_barrier(0);
-      }
+        for (int i4 = 0; i4 < 4; ++i4)
+          bv[nt][i4] = *reinterpret_cast<const x4*>(static_cast<const T*>(p.bias) + n0 + g * 4 + nt * 32 + i4 * 8);
+      first_copies();
+#pragma unroll
+      for (int nt = 0; nt < NT; ++nt)
+#pragma unroll
+        for (int mt = 0; mt < MT; ++mt)
+#pragma unroll
+          for (int i = 0; i < 16; ++i) acc[nt][mt][i] = static_cast<float>(bv[nt][i >> 2][i & 3]);
+    } else if (p.bias_kind == FO_BIAS_MATRIX && p.bias_f32) {
+      f32x4 bm[NT][MT][4];
+#pragma unroll
+      for (int nt = 0; nt < NT; ++nt)
+#pragma unroll
+        for (int mt = 0; mt < MT; ++mt)
+#pragma unroll
+          for (int i4 = 0; i4 < 4; ++i4)
+            bm[nt][mt][i4] = *reinterpret_cast<const f32x4*>(static_cast<const float*>(p.bias) + row_off[mt] + nt * 32 + i4 * 8);
+      first_copies();
+#pragma unroll
+      for (int nt = 0; nt < NT; ++nt)
+#pragma unroll
+        for (int mt = 0; mt < MT; ++mt)
+#pragma unroll
+          for (int i = 0; i < 16; ++i) acc[nt][mt][i] = bm[nt][mt][i >> 2][i & 3];
+    } else if (p.bias_kind == FO_BIAS_MATRIX) {
+      x4 bm[NT][MT][4];
+#pragma unroll
+      for (int nt = 0; nt < NT; ++nt)
+#pragma unroll
+        for (int mt = 0; mt < MT; ++mt)
+#pragma unroll
+          for (int i4 = 0; i4 < 4; ++i4)
+            bm[nt][mt][i4] = *reinterpret_cast<const x4*>(static_cast<const T*>(p.bias) + row_off[mt] + nt * 32 + i4 * 8);
+      first_copies();
+#pragma unroll
+      for (int nt = 0; nt < NT; ++nt)
+#pragma unroll
+        for (int mt = 0; mt < MT; ++mt)
+#pragma unroll
+          for (int i = 0; i < 16; ++i) acc[nt][mt][i] = static_cast<float>(bm[nt][mt][i >> 2][i & 3]);
+    } else {
+      first_copies();
+#pragma unroll
+      for (int nt = 0; nt < NT; ++nt)
+#pragma unroll
+        for (int mt = 0; mt < MT; ++mt)
+#pragma unroll
+          for (int i = 0; i < 16; ++i) acc[nt][mt][i] = 0.f;
     }
 
-    // ---- 32-wide K tail (K % 64 == 32, GEMM-Q only): operands straight from global memory ----
-    if (!kReduce && (p.k % kBK) != 0) {
-      const int k0 = (p.k / kBK) * kBK;
-      const int a_row0 = wh * 64, b_row0 = 0;  // rows inside the shared W tile / this unit's X tile
-      const T* wsrc = tile_base[0];
-      const T* xsrc = tile_base[1 + wp];
-      const int xrows = tile_rows[1 + wp];
-#pragma unroll
-      for (int ks = 0; ks < 2; ++ks) {
-        x8 a[NT], b[MT];
-#pragma unroll
-        for (int nt = 0; nt < NT; ++nt)
-          a[nt] = *reinterpret_cast<const x8*>(wsrc + static_cast<int64_t>(a_row0 + nt * 32 + l32) * p.k +
-                                               k0 + ks * 16 + g * 8);
+    // LDS byte offsets of this wavefront's operand rows inside a stage
+    const int a_base = (2 + wc) * kUnitBytes + l32 * kRowBytes;        // W rows nt*32 + l32
+    const int b_base = wr * kUnitBytes + (wh * 64 + l32) * kRowBytes;  // X rows wh*64 + mt*32 + l32
+
+    // ---- main loop ----
+    // Copies run up to three k steps ahead.  Operand reads run half a k step ahead of the MFMAs
+    // that use them (two register sets), so a wavefront's LDS reads overlap its own math:
+    //   MFMAs(it, first half) with reads(it, second half) in their shadow | tile it+1 landed, barrier,
+    //   copy(it+3) | MFMAs(it, second half) with reads(it+1, first half) in their shadow
+    x8 a[2][NT], b[2][MT];
+    // one operand read of half-step (it, ks): j = 0..3 W rows, j = 4..5 X rows
+    // one operand read of half-step (it, ks): j = 0..3 W rows, j = 4..5 X rows
+    auto read_one = [&](int it, int ks, int j) {
+      const uint8_t* st = smem + (it % kStages) * kStageBytes;
+      const int sw = ((2 * ks + g) ^ rd_swz) << 4;
+      if (j < NT) {
+        a[ks][j] = *reinterpret_cast<const x8*>(st + a_base + j * 32 * kRowBytes + sw);
+      } else {
+        b[ks][j - NT] = *reinterpret_cast<const x8*>(st + b_base + (j - NT) * 32 * kRowBytes + sw);
+      }
+    };
+    // the eight MFMAs of half-step ks; in their shadow the six operand reads of half-step (rit, rks)
+    // and, if cit >= 0, this wavefront's four copies of tile cit.  GEMM-O: a token block that does
+    // not select this step's head contributes nothing: its X operand is zeroed (keep = 0).  (Skipping
+    // the MFMAs instead puts them under a branch, and the register allocator then copies and spills
+    // accumulators in the loop.)
+    auto math_and_read = [&](int ks, unsigned keep, int rit, int rks, int cit, int centry) {
+      if constexpr (kReduce) {
 #pragma unroll
         for (int mt = 0; mt < MT; ++mt) {
-          int r = b_row0 + mt * 32 + l32;
-          r = r < xrows ? r : xrows - 1;
-          b[mt] = *reinterpret_cast<const x8*>(xsrc + static_cast<int64_t>(r) * p.k + k0 + ks * 16 + g * 8);
+          u32x4 v = __builtin_bit_cast(u32x4, b[ks][mt]);
+          v &= keep;
+          b[ks][mt] = __builtin_bit_cast(x8, v);
         }
+      }
 #pragma unroll
-        for (int nt = 0; nt < NT; ++nt)
+      for (int i = 0; i < NT * MT; ++i) {
+        const int nt = i / MT, mt = i % MT;
+        acc[nt][mt] = TT::mfma(a[ks][nt], b[ks][mt], acc[nt][mt]);
+        if (cit >= 0 && i < kCopiesPerWave) copy_one(cit, centry, i);
+        if (i < NT + MT) read_one(rit, rks, i);
+        __builtin_amdgcn_sched_barrier(0);
+      }
+    };
+    auto keep_of = [&](int entry) -> unsigned {
+      return kReduce ? (((entry >> (16 + wr)) & 1) ? 0xFFFFFFFFu : 0u) : 0xFFFFFFFFu;
+    };
+    // Copies past the last k step repeat the last one (into a stage nobody reads any more), so the
+    // loop body and its vmcnt arithmetic are the same for every step.
+    if (n_iter > 0) {
+      __builtin_amdgcn_s_waitcnt(0x0f70 | (2 * kCopiesPerWave));  // tile 0 landed, 1 and 2 in flight
+      __builtin_amdgcn_s_barrier();
 #pragma unroll
-          for (int mt = 0; mt < MT; ++mt) acc[nt][mt] = TT::mfma(a[nt], b[mt], acc[nt][mt]);
+      for (int j = 0; j < NT + MT; ++j) read_one(0, 0, j);
+      unsigned keep = keep_of(step_entry(0));
+      for (int it = 0; it < n_iter; ++it) {
+        // table entries of the tile to copy and of the next tile, read ahead of their use
+        const int centry = step_entry(it + 3);
+        const unsigned keep_next = keep_of(step_entry(it + 1));
+        math_and_read(0, keep, it, 1, -1, 0);
+        __builtin_amdgcn_s_waitcnt(0x0f70 | kCopiesPerWave);  // tile it+1 landed (it+2 may be in flight)
+        __builtin_amdgcn_s_barrier();  // ... for every wavefront; nobody reads stage (it-1)%4 any more
+        // copies of tile it+3 and reads of tile it+1 in the shadow of the second half's MFMAs
+        // (the reads of the last step fetch a stale stage; never used)
+        math_and_read(1, keep, it + 1, 0, it + 3, centry);
+        keep = keep_next;
       }
     }
 
@@ -472,43 +520,80 @@ __global__ void __launch_bounds__(kThreads) gemm_kernel(const GemmParams p) {
     if (my_valid) {
 #pragma unroll
       for (int mt = 0; mt < MT; ++mt) {
-        const int mrow = m0 + mt * 32 + l32;
-        if (mrow >= p.m) continue;
+        if (m0 + mt * 32 + l32 >= p.m) continue;
+        if (p.y_f32) {
+          float* yrow = static_cast<float*>(p.y) + row_off[mt];
 #pragma unroll
-        for (int nt = 0; nt < NT; ++nt)
+          for (int nt = 0; nt < NT; ++nt)
 #pragma unroll
-          for (int i4 = 0; i4 < 4; ++i4) {
-            const int ncol = n0 + nt * 32 + i4 * 8 + g * 4;
-            const int64_t off = y_batch + static_cast<int64_t>(mrow) * p.n + ncol;
-            if (p.y_f32) {
+            for (int i4 = 0; i4 < 4; ++i4) {
               f32x4 out;
 #pragma unroll
               for (int j = 0; j < 4; ++j) out[j] = acc[nt][mt][i4 * 4 + j];
-              *reinterpret_cast<f32x4*>(static_cast<float*>(p.y) + off) = out;
-            } else {
+              *reinterpret_cast<f32x4*>(yrow + nt * 32 + i4 * 8) = out;
+            }
+        } else {
+          T* yrow = static_cast<T*>(p.y) + row_off[mt];
+#pragma unroll
+          for (int nt = 0; nt < NT; ++nt)
+#pragma unroll
+            for (int i4 = 0; i4 < 4; ++i4) {
               x4 out;
 #pragma unroll
               for (int j = 0; j < 4; ++j) out[j] = static_cast<T>(acc[nt][mt][i4 * 4 + j]);
-              *reinterpret_cast<x4*>(static_cast<T*>(p.y) + off) = out;
+              *reinterpret_cast<x4*>(yrow + nt * 32 + i4 * 8) = out;
             }
-          }
+        }
       }
     }
   }
 }
 
+ListGeom make_geom(int32_t batch, int32_t m, int32_t n) {
+  ListGeom gm;
+  gm.batch = batch;
+  gm.n_row_tiles = (m + kTile - 1) / kTile;
+  gm.n_col_tiles = n / kTile;
+  gm.n_win = (gm.n_row_tiles + kWindow - 1) / kWindow;
+  gm.n_cp = (gm.n_col_tiles + 1) / 2;
+  return gm;
+}
+
+int64_t workspace_ints(const ListGeom& gm, int64_t* max_quads_out) {
+  const int64_t n_wt = static_cast<int64_t>(gm.batch) * gm.n_win, n_cells = n_wt * gm.n_cp;
+  const int64_t max_quads = n_cells * kWindow;  // a cell of 16 rows x 2 columns yields at most 16 quads
+  if (max_quads_out) *max_quads_out = max_quads;
+  return 16 + kQuadInts * max_quads;
+}
+
 template <typename T, bool kReduce>
-int launch(const GemmParams& p, int64_t max_work, hipStream_t stream) {
+int launch(GemmParams& p, const ListGeom& gm, bool use_flags, void* workspace, hipStream_t stream) {
   static bool attr_set = false;
   if (!attr_set) {
     FO_HIP_CALL(hipFuncSetAttribute(reinterpret_cast<const void*>(&gemm_kernel<T, kReduce>),
                                     hipFuncAttributeMaxDynamicSharedMemorySize, kSmemBytes));
     attr_set = true;
   }
+  int64_t max_quads = 0;
+  workspace_ints(gm, &max_quads);
+  int32_t* qoff = static_cast<int32_t*>(workspace);
+  int32_t* quads = qoff + 16;
+  ListArgs la;
+  la.sparse_info = p.sparse_info;
+  la.sparse_info_indptr = p.sparse_info_indptr;
+  la.use_flags = use_flags ? 1 : 0;
+  la.sparse_q_size = p.sparse_q_size;
+  la.num_heads = p.num_heads;
+  la.head_dim = p.head_dim;
+  la.num_text_tokens = p.num_text_tokens;
+  gemm_quads_kernel<<<1, kListThreads, 0, stream>>>(la, gm, quads, qoff);
+  FO_CHECK_LAUNCH();
+  p.quads = quads;
+  p.qoff = qoff;
   int num_cu = fo_num_cu();
   if (num_cu <= 0) return fo::fail(FO_ERR_HIP, "gemm: no device");
   int64_t grid = (num_cu + kXcds - 1) / kXcds * kXcds;  // one persistent workgroup per CU
-  const int64_t cap = (max_work + kXcds - 1) / kXcds * kXcds;
+  const int64_t cap = (max_quads + kXcds - 1) / kXcds * kXcds;
   if (grid > cap) grid = cap;
   if (grid < kXcds) grid = kXcds;
   gemm_kernel<T, kReduce><<<static_cast<unsigned>(grid), kThreads, kSmemBytes, stream>>>(p);
@@ -517,7 +602,8 @@ int launch(const GemmParams& p, int64_t max_work, hipStream_t stream) {
 }
 
 int check_common(const void* x, const void* w, void* y, int dtype, int32_t batch, int32_t m,
-                 int32_t n, int32_t k, int32_t sparse_q_size, int32_t num_qo_heads) {
+                 int32_t n, int32_t k, int32_t sparse_q_size, int32_t num_qo_heads,
+                 void* workspace, int64_t workspace_bytes) {
   FO_REQUIRE(dtype == FO_BF16 || dtype == FO_F16, "gemm: only bf16 / fp16 operands are supported");
   FO_REQUIRE(batch > 0 && m > 0 && n > 0 && k > 0, "gemm: bad shape");
   FO_REQUIRE(n % 128 == 0 && k % 32 == 0, "only support N %% 128 == 0, K %% 32 == 0 (got N=%d K=%d)",
@@ -528,18 +614,20 @@ int check_common(const void* x, const void* w, void* y, int dtype, int32_t batch
   FO_REQUIRE(((reinterpret_cast<uintptr_t>(x) | reinterpret_cast<uintptr_t>(w) |
                reinterpret_cast<uintptr_t>(y)) & 15) == 0,
              "gemm: x, w, y must be 16-byte aligned");
-  FO_REQUIRE(static_cast<int64_t>(batch) * ((m + kTile - 1) / kTile) * (n / kTile) < (int64_t(1) << 30),
-             "gemm: too many tiles");
+  const ListGeom gm = make_geom(batch, m, n);
+  FO_REQUIRE(static_cast<int64_t>(batch) * gm.n_win * gm.n_cp < (int64_t(1) << 24), "gemm: too many tiles");
+  const int64_t need = 4 * workspace_ints(gm, nullptr);
+  if (!workspace || workspace_bytes < need || (reinterpret_cast<uintptr_t>(workspace) & 15))
+    return fo::fail(FO_ERR_WORKSPACE, "gemm: workspace of %lld bytes (16-byte aligned) required, got %lld",
+                    static_cast<long long>(need), static_cast<long long>(workspace_bytes));
   return FO_OK;
 }
 
 }  // namespace
 
-extern "C" int64_t fo_gemm_q_workspace_bytes(int32_t batch, int32_t m, int32_t n) {
+extern "C" int64_t fo_gemm_workspace_bytes(int32_t batch, int32_t m, int32_t n) {
   if (batch <= 0 || m <= 0 || n <= 0) return 0;
-  const int64_t n_row_tiles = (m + kTile - 1) / kTile, n_win = (n_row_tiles + kWindow - 1) / kWindow;
-  const int64_t max_pairs = static_cast<int64_t>(batch) * (n / kTile) * n_win * (kWindow / 2);
-  return 64 + 16 * max_pairs;
+  return 4 * workspace_ints(make_geom(batch, m, n), nullptr);
 }
 
 extern "C" int fo_gemm_q(const void* x, const void* w, const void* bias, void* y, int dtype,
@@ -547,53 +635,43 @@ extern "C" int fo_gemm_q(const void* x, const void* w, const void* bias, void* y
                          int32_t num_qo_heads, const uint8_t* sparse_info,
                          const int32_t* sparse_info_indptr, int32_t num_text_tokens, int is_full,
                          void* workspace, int64_t workspace_bytes, void* stream) {
-  if (int rc = check_common(x, w, y, dtype, batch, m, n, k, sparse_q_size, num_qo_heads)) return rc;
+  if (int rc = check_common(x, w, y, dtype, batch, m, n, k, sparse_q_size, num_qo_heads, workspace,
+                            workspace_bytes))
+    return rc;
   FO_REQUIRE(is_full || (sparse_info && sparse_info_indptr),
              "gemm: sparse_info and sparse_info_indptr are required unless is_full");
   FO_REQUIRE(num_text_tokens >= 0, "gemm: negative num_text_tokens");
   FO_REQUIRE(!bias || (reinterpret_cast<uintptr_t>(bias) & 7) == 0, "gemm: bias must be 8-byte aligned");
-  const int64_t need = fo_gemm_q_workspace_bytes(batch, m, n);
-  if (!workspace || workspace_bytes < need || (reinterpret_cast<uintptr_t>(workspace) & 15))
-    return fo::fail(FO_ERR_WORKSPACE, "gemm: workspace of %lld bytes (16-byte aligned) required, got %lld",
-                    static_cast<long long>(need), static_cast<long long>(workspace_bytes));
-  hipStream_t s = static_cast<hipStream_t>(stream);
-  int32_t* qoff = static_cast<int32_t*>(workspace);
-  int32_t* pairs = qoff + 16;
-  PairGeom gm;
-  gm.batch = batch;
-  gm.n_row_tiles = (m + kTile - 1) / kTile;
-  gm.n_col_tiles = n / kTile;
-  gm.n_win = (gm.n_row_tiles + kWindow - 1) / kWindow;
-  gm.cols_per_q = (gm.n_col_tiles + kXcds - 1) / kXcds;
-  gemm_q_pairs_kernel<<<1, kPairScanThreads, 0, s>>>(is_full ? nullptr : sparse_info, sparse_info_indptr, gm,
-                                                     sparse_q_size, num_qo_heads, n / num_qo_heads,
-                                                     num_text_tokens, is_full ? 1 : 0, pairs, qoff);
-  FO_CHECK_LAUNCH();
   GemmParams p{};
   p.x = x; p.w = w; p.bias = bias; p.y = y;
   p.sparse_info = is_full ? nullptr : sparse_info;
   p.sparse_info_indptr = sparse_info_indptr;
-  p.pairs = pairs; p.qoff = qoff;
   p.batch = batch; p.m = m; p.n = n; p.k = k;
   p.sparse_q_size = sparse_q_size; p.num_heads = num_qo_heads; p.head_dim = n / num_qo_heads;
   p.num_text_tokens = num_text_tokens;
   p.flag = is_full ? 1 : 0;
   p.bias_kind = bias ? FO_BIAS_VECTOR : FO_BIAS_NONE;
-  const int64_t max_pairs = static_cast<int64_t>(batch) * gm.n_col_tiles * gm.n_win * (kWindow / 2);
-  return dtype == FO_BF16 ? launch<__bf16, false>(p, max_pairs, s) : launch<_Float16, false>(p, max_pairs, s);
+  const ListGeom gm = make_geom(batch, m, n);
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  return dtype == FO_BF16 ? launch<__bf16, false>(p, gm, !is_full, workspace, s)
+                          : launch<_Float16, false>(p, gm, !is_full, workspace, s);
 }
 
 extern "C" int fo_gemm_o(const void* x, const void* w, const void* bias, void* y, int dtype,
                          int bias_kind, int bias_dtype, int y_dtype, int32_t batch, int32_t m,
                          int32_t n, int32_t k, int32_t sparse_q_size, int32_t num_qo_heads,
                          const uint8_t* sparse_info, const int32_t* sparse_info_indptr,
-                         int32_t num_text_tokens, int is_for_cached, void* stream) {
-  if (int rc = check_common(x, w, y, dtype, batch, m, n, k, sparse_q_size, num_qo_heads)) return rc;
+                         int32_t num_text_tokens, int is_for_cached, void* workspace,
+                         int64_t workspace_bytes, void* stream) {
+  if (int rc = check_common(x, w, y, dtype, batch, m, n, k, sparse_q_size, num_qo_heads, workspace,
+                            workspace_bytes))
+    return rc;
   FO_REQUIRE(sparse_info && sparse_info_indptr, "gemm_reduction: sparse_info is required");
   FO_REQUIRE(num_text_tokens >= 0, "gemm: negative num_text_tokens");
   const int head_dim = n / num_qo_heads;
-  FO_REQUIRE(head_dim % kBK == 0 && k % head_dim == 0 && k / head_dim <= kMaxHeads,
-             "gemm_reduction: head slice width %d must be a multiple of 64 and divide K=%d", head_dim, k);
+  FO_REQUIRE(head_dim % kBK == 0 && k % head_dim == 0 && k / head_dim <= kMaxHeads && k / kBK <= kMaxSteps,
+             "gemm_reduction: head slice width %d must be a multiple of 32 and divide K=%d <= 65536",
+             head_dim, k);
   FO_REQUIRE(bias_kind == FO_BIAS_NONE || bias_kind == FO_BIAS_VECTOR || bias_kind == FO_BIAS_MATRIX,
              "gemm_reduction: bad bias kind");
   FO_REQUIRE(bias_kind == FO_BIAS_NONE || bias, "gemm_reduction: bias pointer is null");
@@ -614,7 +692,8 @@ extern "C" int fo_gemm_o(const void* x, const void* w, const void* bias, void* y
   p.bias_kind = bias_kind;
   p.bias_f32 = bias_dtype == FO_F32;
   p.y_f32 = y_dtype == FO_F32;
+  const ListGeom gm = make_geom(batch, m, n);
   hipStream_t s = static_cast<hipStream_t>(stream);
-  const int64_t work = static_cast<int64_t>(batch) * ((m + kTile - 1) / kTile) * ((n / kTile + 1) / 2);
-  return dtype == FO_BF16 ? launch<__bf16, true>(p, work, s) : launch<_Float16, true>(p, work, s);
+  return dtype == FO_BF16 ? launch<__bf16, true>(p, gm, false, workspace, s)
+                          : launch<_Float16, true>(p, gm, false, workspace, s);
 }

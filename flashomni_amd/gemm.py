@@ -59,8 +59,8 @@ def flashomni_gemm(
     if not is_full and info is None:
         raise RuntimeError("flashomni_gemm: sparse_info is required unless is_full=True")
     L = _lib.lib()
-    ws_bytes = L.fo_gemm_q_workspace_bytes(A.shape[0], A.shape[1], B.shape[0])
-    workspace = torch.empty(ws_bytes, dtype=torch.uint8, device=A.device)  # pair list scratch
+    ws_bytes = L.fo_gemm_workspace_bytes(A.shape[0], A.shape[1], B.shape[0])
+    workspace = torch.empty(ws_bytes, dtype=torch.uint8, device=A.device)  # tile-list scratch
     _lib.check(L.fo_gemm_q(
         _lib.ptr(A), _lib.ptr(B), _lib.ptr(bias), _lib.ptr(out), _lib.dtype_code(A.dtype),
         A.shape[0], A.shape[1], B.shape[0], A.shape[2], sparse_q_size, num_qo_heads,
@@ -114,9 +114,12 @@ def flashomni_gemm_reduction(
             bias_code = _lib.dtype_code(bias.dtype)
         bias = bias.contiguous()
     info, indptr = _symbols(sparse_info, sparse_info_indptr, A.device)
-    _lib.check(_lib.lib().fo_gemm_o(
+    L = _lib.lib()
+    ws_bytes = L.fo_gemm_workspace_bytes(Bsz, M, N)
+    workspace = torch.empty(ws_bytes, dtype=torch.uint8, device=A.device)  # tile-list scratch
+    _lib.check(L.fo_gemm_o(
         _lib.ptr(A), _lib.ptr(B), _lib.ptr(bias), _lib.ptr(out), _lib.dtype_code(A.dtype), kind,
         bias_code, _lib.dtype_code(out_dtype), Bsz, M, N, A.shape[2], sparse_q_size, num_qo_heads,
         _lib.ptr(info), _lib.ptr(indptr), num_text_tokens, int(bool(is_for_cache)),
-        _lib.current_stream(A.device)))
+        _lib.ptr(workspace), ws_bytes, _lib.current_stream(A.device)))
     return out

@@ -150,10 +150,10 @@ int fo_sparse_fa_run(const void* q, const void* k, const void* v, void* o, float
  * + (ix*128)/(N/num_qo_heads) of sparse_info + sparse_info_indptr[b] (gemm.cuh:50-58).
  * Requires N % 128 == 0 and K % 32 == 0 (csrc/gemm.cu:36); M may have a tail (the reference
  * demands M % 128 == 0).
- * `workspace`: device scratch of at least fo_gemm_q_workspace_bytes(batch, m, n) bytes, 16-byte
- * aligned; it receives the compacted list of flagged tile pairs that the GEMM kernel walks.
+ * `workspace`: device scratch of at least fo_gemm_workspace_bytes(batch, m, n) bytes, 16-byte
+ * aligned; it receives the list of tile quads that the GEMM kernel walks.
  * ------------------------------------------------------------------------------------------- */
-int64_t fo_gemm_q_workspace_bytes(int32_t batch, int32_t m, int32_t n);
+int64_t fo_gemm_workspace_bytes(int32_t batch, int32_t m, int32_t n);
 int fo_gemm_q(const void* x, const void* w, const void* bias, void* y, int dtype, int32_t batch,
               int32_t m, int32_t n, int32_t k, int32_t sparse_q_size, int32_t num_qo_heads,
               const uint8_t* sparse_info, const int32_t* sparse_info_indptr,
@@ -170,12 +170,13 @@ int fo_gemm_q(const void* x, const void* w, const void* bias, void* y, int dtype
  *           slice selection).
  * bias_dtype: the activation dtype (as in the reference) or FO_F32 for the matrix form;
  * y_dtype: the activation dtype or FO_F32 (so a cached partial can stay in fp32).
+ * hd must be a multiple of 32.  `workspace` as for fo_gemm_q.
  * ------------------------------------------------------------------------------------------- */
 int fo_gemm_o(const void* x, const void* w, const void* bias, void* y, int dtype, int bias_kind,
               int bias_dtype, int y_dtype, int32_t batch, int32_t m, int32_t n, int32_t k,
               int32_t sparse_q_size, int32_t num_qo_heads, const uint8_t* sparse_info,
               const int32_t* sparse_info_indptr, int32_t num_text_tokens, int is_for_cached,
-              void* stream);
+              void* workspace, int64_t workspace_bytes, void* stream);
 
 /* ---------------------------------------------------------------------------------------------
  * fp8 e4m3fn quantiser with one absmax scale per (head, 128-token block).
