@@ -52,6 +52,7 @@ typedef __attribute__((ext_vector_type(4))) float f32x4;
 typedef __attribute__((ext_vector_type(4))) unsigned int u32x4;
 typedef __attribute__((ext_vector_type(8))) int i32x8;
 typedef __attribute__((ext_vector_type(4))) int i32x4;
+typedef __attribute__((ext_vector_type(2))) unsigned int u32x2;
 
 constexpr float kNegInf = -5e4f;  // finite "infinity" of the reference
 constexpr int kThreads = 512;
@@ -70,6 +71,7 @@ struct Geom {
   static constexpr int kSmemBytes = 2 * kGroupBytes;
 };
 constexpr int kXcds = 8;
+constexpr int kMaxRowBlocks = 4096;  // kv blocks of one row held in LDS (512 Ki tokens per request)
 constexpr float kLazyLog2 = 8.0f;  // the running max is raised only past a 2^8 overshoot
 // merge area (reuses the tile buffers): O^T of kv group 1, then its (m, d)
 constexpr int kMergeOBytes = 4 * 16 * 64 * 16;
@@ -109,6 +111,14 @@ struct Types<__bf16> {
   static __device__ __forceinline__ f32x16 mfma(x8 a, x8 b, f32x16 c) {
     return __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, b, c, 0, 0, 0);
   }
+  // acc + sum of the eight elements of v (v_dot2c_f32_bf16 against ones)
+  static __device__ __forceinline__ float add_elems(x8 v, float acc) {
+    typedef __attribute__((ext_vector_type(2))) __bf16 x2;
+    const x2 ones = {static_cast<__bf16>(1.0f), static_cast<__bf16>(1.0f)};
+#pragma unroll
+    for (int i = 0; i < 4; ++i) acc = __builtin_amdgcn_fdot2_f32_bf16(x2{v[2 * i], v[2 * i + 1]}, ones, acc, false);
+    return acc;
+  }
 };
 template <>
 struct Types<_Float16> {
@@ -116,6 +126,13 @@ struct Types<_Float16> {
   using x4 = f16x4;
   static __device__ __forceinline__ f32x16 mfma(x8 a, x8 b, f32x16 c) {
     return __builtin_amdgcn_mfma_f32_32x32x16_f16(a, b, c, 0, 0, 0);
+  }
+  static __device__ __forceinline__ float add_elems(x8 v, float acc) {
+    typedef __attribute__((ext_vector_type(2))) _Float16 x2;
+    const x2 ones = {static_cast<_Float16>(1.0f), static_cast<_Float16>(1.0f)};
+#pragma unroll
+    for (int i = 0; i < 4; ++i) acc = __builtin_amdgcn_fdot2(x2{v[2 * i], v[2 * i + 1]}, ones, acc, false);
+    return acc;
   }
 };
 
@@ -128,9 +145,18 @@ __device__ __forceinline__ int swz(int r) { return ((r & 3) << 2) | ((r >> 2) & 
 // chunk swizzle of a 128-byte LDS tile row r (8 chunks; two rows span the 64 banks)
 __device__ __forceinline__ int swz8(int r) { return (r >> 1) & 7; }
 
-// 64 lanes x 16 bytes, global -> LDS at lds_base + lane*16 (lds_base is wavefront-uniform)
-__device__ __forceinline__ void copy16_to_lds(const void* gsrc, uint8_t* lds_base) {
-  __builtin_amdgcn_global_load_lds((glb_void*)gsrc, (lds_void*)lds_base, 16, 0, 0);
+// 64 lanes x 16 bytes, global -> LDS: lane i fetches 16 bytes at sbase + voff and lands at LDS byte
+// address lds_addr + 16*i.  sbase and lds_addr are wavefront-uniform (scalar registers), so a copy
+// costs no vector-ALU work.  Issued as inline assembly on purpose: the compiler then does not
+// track the copy, and does not put a vmcnt(0) in front of later LDS reads of the *other* stage that
+// it cannot tell apart from the copy's destination (that wait would expose the whole copy latency
+// every tile).  All waits on these copies are the explicit s_waitcnt vmcnt(0) + barrier at the
+// head of a tile's MFMA block.
+__device__ __forceinline__ void copy16_to_lds(const void* sbase, uint32_t voff, uint32_t lds_addr) {
+  asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2"
+               :
+               : "s"(lds_addr), "v"(voff), "s"(sbase)
+               : "memory", "m0");
 }
 
 // Four 16-bit values from a 4-row x 16-column LDS patch, transposed across a 16-lane group:
@@ -138,6 +164,13 @@ __device__ __forceinline__ void copy16_to_lds(const void* gsrc, uint8_t* lds_bas
 // column i of rows 0..3.
 __device__ __forceinline__ s16x4 lds_read_tr16(const uint8_t* p) {
   return __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4*)(p));
+}
+
+// max of x over lane and lane^32 (v_permlane32_swap: no LDS round trip)
+__device__ __forceinline__ float max_across_halves(float x) {
+  const unsigned u = __builtin_bit_cast(unsigned, x);
+  const u32x2 r = __builtin_amdgcn_permlane32_swap(u, u, false, false);
+  return fmaxf(__builtin_bit_cast(float, r[0]), __builtin_bit_cast(float, r[1]));
 }
 
 // Pop the next row for this workgroup: own XCD queue first, then the neighbours'.
@@ -166,8 +199,10 @@ __global__ void __launch_bounds__(kThreads) sparse_fa_kernel(const FaParams p) {
   constexpr int kStageBytes = G::kStageBytes, kKBytes = G::kKBytes, kGroupBytes = G::kGroupBytes;
   extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
   __shared__ int s_next_row;
+  __shared__ int32_t s_blk[kMaxRowBlocks];  // kv block list of the current row
 
-  const int tid = threadIdx.x, lane = tid & 63, wv = tid >> 6;
+  const int tid = threadIdx.x, lane = tid & 63;
+  const int wv = __builtin_amdgcn_readfirstlane(tid >> 6);  // wavefront index, kept scalar
   const int qs = wv & 3, kg = wv >> 2;
   const int l32 = lane & 31, g = lane >> 5;
   const float c = p.sm_scale_log2;
@@ -209,7 +244,7 @@ __global__ void __launch_bounds__(kThreads) sparse_fa_kernel(const FaParams p) {
     __syncthreads();  // everyone is done with s_next_row and with the previous row's LDS data
     if (tid == 0) s_next_row = pop_row(p, blockIdx.x & (kXcds - 1));
     __syncthreads();
-    const int w = s_next_row;
+    const int w = __builtin_amdgcn_readfirstlane(s_next_row);  // uniform: row data goes through scalar loads
     if (w < 0) break;
 
     const int req = p.row_req[w], qb = p.row_qb[w], head = p.row_head[w];
@@ -217,7 +252,8 @@ __global__ void __launch_bounds__(kThreads) sparse_fa_kernel(const FaParams p) {
     const int q_rows = min(kBlockQ, p.qo_indptr[req + 1] - q_begin);
     const int kv_begin = p.kv_indptr[req];
     const int kv_len = p.kv_indptr[req + 1] - kv_begin;
-    const int ptr0 = p.kv_row_ptr[w], nb = p.kv_row_ptr[w + 1] - ptr0;
+    // (a row longer than the LDS list is cut; the host side refuses such requests at plan time)
+    const int ptr0 = p.kv_row_ptr[w], nb = min(p.kv_row_ptr[w + 1] - ptr0, kMaxRowBlocks);
 
     const int my_row = qs * 32 + l32;  // q row of this lane inside the block
     const bool row_ok = my_row < q_rows;
@@ -235,12 +271,13 @@ __global__ void __launch_bounds__(kThreads) sparse_fa_kernel(const FaParams p) {
       continue;
     }
 
+    // the row's kv block list goes to LDS: the main loop then has no global loads besides the
+    // tile copies, whose completion it tracks by counting (s_waitcnt vmcnt)
+    for (int i = tid; i < nb; i += kThreads) s_blk[i] = p.kv_idx[ptr0 + i];
+    __syncthreads();
     // number of 64-key tiles; only the last listed block can be the request's ragged tail
     int n_tiles = 2 * nb;
-    {
-      const int last_blk = p.kv_idx[ptr0 + nb - 1];
-      if (kv_len - last_blk * kBlockKV <= kTileKV) n_tiles -= 1;
-    }
+    if (kv_len - s_blk[nb - 1] * kBlockKV <= kTileKV) n_tiles -= 1;
     const int my_tiles = (n_tiles - kg + 1) >> 1;  // tiles kg, kg+2, ...
 
     // Q operand: lane holds q row l32 of its q sub-tile, d = ks*16 + g*8 .. +7
@@ -258,7 +295,12 @@ __global__ void __launch_bounds__(kThreads) sparse_fa_kernel(const FaParams p) {
     } else {
       const T* src = reinterpret_cast<const T*>(qp) + q_tok * p.q_sn + static_cast<int64_t>(head) * p.q_sh + g * 8;
 #pragma unroll
-      for (int ks = 0; ks < 8; ++ks) qreg[ks] = *reinterpret_cast<const x8*>(src + ks * 16);
+      for (int ks = 0; ks < 8; ++ks) {
+        // the softmax scale (log2 domain) is folded into Q, so S^T needs no multiply afterwards
+        const x8 raw = *reinterpret_cast<const x8*>(src + ks * 16);
+#pragma unroll
+        for (int e = 0; e < 8; ++e) qreg[ks][e] = static_cast<T>(static_cast<float>(raw[e]) * c);
+      }
     }
     // softmax scale in the log2 domain; with fp8 operands the per-block dequantisation scales of
     // q (one per row of the list) and k (one per kv block) are folded in tile by tile
@@ -272,66 +314,142 @@ __global__ void __launch_bounds__(kThreads) sparse_fa_kernel(const FaParams p) {
     for (int dt = 0; dt < 4; ++dt)
 #pragma unroll
       for (int i = 0; i < 16; ++i) o_acc[dt][i] = 0.f;
-    float m_run = kNegInf, d_part = 0.f;  // running max in the log2 domain (s * scale), partial sum
-    float cs_next = cq;
+    // Running reference point m_run of the softmax (log2 domain), partial sum d_part.  S^T is formed
+    // relative to m_run: the MFMA accumulator starts at -m_run (c_init), so p = exp2(S^T) directly.
+    // m_run is set to the tile's exact row max on the first tile and afterwards only raised when a
+    // row's new max exceeds it by more than kLazyLog2 (p then stays <= 2^kLazyLog2, harmless in
+    // fp32 / bf16 / fp16): the rescale of O leaves the steady-state path.
+    float m_run = 0.f, d_part = 0.f;
+    f32x16 c_init;
+#pragma unroll
+    for (int i = 0; i < 16; ++i) c_init[i] = 0.f;
 
-    // Issue the global->LDS copy of this kv group's tile `it` into LDS stage it&1.
-    const int64_t k_head = static_cast<int64_t>(head) * p.k_sh + (kFp8 ? cp8_chunk : cp_chunk);
-    const int64_t v_head = static_cast<int64_t>(head) * p.v_sh + cp_chunk;
-    auto copy_tile = [&](int it) {
-      const int t = 2 * it + kg;
-      const int blk = p.kv_idx[ptr0 + (t >> 1)];
-      const int start = blk * kBlockKV + (t & 1) * kTileKV;
+    // Tile copies.  The address of a copy is a wavefront-uniform tile base plus a per-lane byte
+    // offset that does not change from tile to tile (row inside the tile, swizzled chunk); only a
+    // request's ragged last tile clamps rows.  Tile j of this kv group = 64 keys of block j of the
+    // row's list; it lives in LDS stage j & 1.  K and V of a tile are copied at different times,
+    // each as early as its half of the stage is free:
+    //   K of tile j+2 at the start of the VALU block of tile j   (K of tile j was consumed by S(j))
+    //   V of tile j+1 during the MFMA block of tile j            (V of tile j-1 is in registers)
+    // so a K copy has about two block periods to land and a V copy more than one.
+    const TQK* k_head = kp + static_cast<int64_t>(kv_begin) * p.k_sn + static_cast<int64_t>(head) * p.k_sh;
+    const T* v_head = vp + static_cast<int64_t>(kv_begin) * p.v_sn + static_cast<int64_t>(head) * p.v_sh;
+    // lane offsets of copy instruction 0; instruction n adds a uniform 16 (fp8 K: 32) rows
+    const uint32_t v_voff = static_cast<uint32_t>((4 * qs + cp_row) * p.v_sn + cp_chunk) * sizeof(T);
+    const uint32_t k_voff = kFp8 ? static_cast<uint32_t>((8 * qs + cp8_row) * p.k_sn + cp8_chunk)
+                                 : static_cast<uint32_t>((4 * qs + cp_row) * p.k_sn + cp_chunk) * sizeof(T);
+    const int64_t k_jstep = (kFp8 ? 32 : 16) * p.k_sn * static_cast<int64_t>(sizeof(TQK));
+    const int64_t v_jstep = 16 * p.v_sn * static_cast<int64_t>(sizeof(T));
+    const uint32_t lds_group = static_cast<uint32_t>(reinterpret_cast<uintptr_t>((lds_void*)group_smem));
+    constexpr int kKCopies = kFp8 ? 2 : 4, kVCopies = 4;  // copy instructions per wavefront and tile
+    auto tile_start = [&](int j) { return s_blk[j] * kBlockKV + kg * kTileKV; };
+    auto tile_valid = [&](int j) { return min(kTileKV, kv_len - tile_start(j)); };
+    // all K copies of tile j at once
+    auto copy_k = [&](int j) {
+      const int start = __builtin_amdgcn_readfirstlane(tile_start(j));
       const int valid = min(kTileKV, kv_len - start);
-      const TQK* kt = kp + static_cast<int64_t>(kv_begin + start) * p.k_sn + k_head;
-      const T* vt = vp + static_cast<int64_t>(kv_begin + start) * p.v_sn + v_head;
-      uint8_t* kdst = group_smem + (it & 1) * kStageBytes;
-      uint8_t* vdst = kdst + kKBytes;
-      if constexpr (kFp8) cs_next = cq * ksc[blk];
+      const uint8_t* kt = reinterpret_cast<const uint8_t*>(k_head + static_cast<int64_t>(start) * p.k_sn);
+      const uint32_t kdst = lds_group + (j & 1) * kStageBytes + qs * 1024;
+      if (__builtin_expect(valid == kTileKV, 1)) {
 #pragma unroll
-      for (int j = 0; j < 4; ++j) {
-        const int n = 4 * j + qs;
-        int r = 4 * n + cp_row;
-        r = r < valid ? r : valid - 1;  // ragged tail: re-read the last valid row, never overrun
-        if constexpr (!kFp8) copy16_to_lds(kt + static_cast<int64_t>(r) * p.k_sn, kdst + n * 1024);
-        copy16_to_lds(vt + static_cast<int64_t>(r) * p.v_sn, vdst + n * 1024);
-      }
-      if constexpr (kFp8) {
+        for (int n = 0; n < kKCopies; ++n) copy16_to_lds(kt + n * k_jstep, k_voff, kdst + n * 4096);
+      } else {
+        // ragged tail: re-read the last valid row, never overrun
 #pragma unroll
-        for (int j = 0; j < 2; ++j) {
-          const int n = 4 * j + qs;
-          int r = 8 * n + cp8_row;
+        for (int n = 0; n < kKCopies; ++n) {
+          int r = (kFp8 ? 8 : 4) * (4 * n + qs) + (kFp8 ? cp8_row : cp_row);
           r = r < valid ? r : valid - 1;
-          copy16_to_lds(kt + static_cast<int64_t>(r) * p.k_sn, kdst + n * 1024);
+          const uint32_t off = kFp8 ? static_cast<uint32_t>(r * p.k_sn + cp8_chunk)
+                                    : static_cast<uint32_t>((r * p.k_sn + cp_chunk) * sizeof(T));
+          copy16_to_lds(kt, off, kdst + n * 4096);
         }
       }
-      return valid;
+    };
+    // V copies of tile j: prepared once, then issued one instruction at a time between MFMAs (a
+    // wavefront that issues its share in one burst sits in the issue stage while the CU's address
+    // unit, 64 B/clk, works through the burst of all eight wavefronts)
+    const uint8_t* cp_v = nullptr;
+    uint32_t cp_vdst = 0;
+    bool cp_pending = false;
+    auto copy_v_prepare = [&](int j) {
+      const int start = __builtin_amdgcn_readfirstlane(tile_start(j));
+      const int valid = min(kTileKV, kv_len - start);
+      cp_v = reinterpret_cast<const uint8_t*>(v_head + static_cast<int64_t>(start) * p.v_sn);
+      cp_vdst = lds_group + (j & 1) * kStageBytes + kKBytes + qs * 1024;
+      cp_pending = valid == kTileKV;
+      if (__builtin_expect(!cp_pending, 0)) {
+#pragma unroll
+        for (int n = 0; n < kVCopies; ++n) {
+          int r = 4 * (4 * n + qs) + cp_row;
+          r = r < valid ? r : valid - 1;
+          copy16_to_lds(cp_v, static_cast<uint32_t>((r * p.v_sn + cp_chunk) * sizeof(T)), cp_vdst + n * 4096);
+        }
+      }
+    };
+    auto copy_v_issue = [&](int n) {
+      if (cp_pending) copy16_to_lds(cp_v + n * v_jstep, v_voff, cp_vdst + n * 4096);
+    };
+    // wait until at most n of this wavefront's copy instructions are outstanding (they complete in
+    // issue order, so "the copies issued after X" outstanding means X has landed)
+    auto wait_copies = [&](int n) {
+      if (n >= 8) {
+        __builtin_amdgcn_s_waitcnt(0x0f70 | 8);
+      } else if (n >= 6) {
+        __builtin_amdgcn_s_waitcnt(0x0f70 | 6);
+      } else if (n >= 4) {
+        __builtin_amdgcn_s_waitcnt(0x0f70 | 4);
+      } else {
+        __builtin_amdgcn_s_waitcnt(0x0f70);
+      }
     };
 
-    const int n_iter = (n_tiles + 1) >> 1;
-    int valid_next = kTileKV;
-    if (my_tiles > 0) valid_next = copy_tile(0);
-
-    for (int it = 0; it < n_iter; ++it) {
-      const uint8_t* ks_base = group_smem + (it & 1) * kStageBytes;
-      const uint8_t* vs_base = ks_base + kKBytes;
-      const bool active = it < my_tiles;
-      const int valid = valid_next;
-      const float cs = cs_next;  // softmax scale of this tile
-      // this wavefront's copies of tile `it` have landed; after the barrier everyone's have, and
-      // everyone has finished reading the other stage
-      __builtin_amdgcn_s_waitcnt(0x0f70);  // vmcnt(0)
-      __syncthreads();
-      if (!active) continue;  // (only the last iteration of kv group 1; no barrier follows)
-      if (it + 1 < my_tiles) valid_next = copy_tile(it + 1);
-
-      // ---- S^T = K . Q^T : two 32-key tiles x 32 q; all operand reads are issued up front ----
-      f32x16 s[2];
+    // ---- main loop: two-phase ("ping-pong") schedule ----
+    // A wavefront alternates between an MFMA block (P.V of the previous tile, then K.Q^T of the
+    // next) and a VALU block (online softmax).  The two kv groups share the SIMDs (wavefront w and
+    // w+4 sit on SIMD w%4) and run half a period apart: every block starts at a workgroup barrier
+    // and kv group 1 takes one extra barrier up front, so while one group's wavefronts feed the
+    // matrix cores the other group's run their softmax on the vector ALUs.
+    //   barrier calls: group 0 makes 2*T0 + 1, group 1 makes 1 + 2*T1 + 1 (T = tiles of the group);
+    //   both pad to the larger count before the merge.
+    const int calls_mine = kg == 0 ? 2 * ((n_tiles + 1) >> 1) + 1 : 2 * (n_tiles >> 1) + 2;
+    const int calls_all = max(2 * ((n_tiles + 1) >> 1) + 1, 2 * (n_tiles >> 1) + 2);
+    // copy order of a wavefront: K0, V0, K1 | V1 (MFMA block 0) | K2 (VALU block 0) | V2 | K3 | ...
+    if (my_tiles > 0) {
+      copy_k(0);
+      copy_v_prepare(0);
 #pragma unroll
-      for (int mt = 0; mt < 2; ++mt)
+      for (int n = 0; n < kVCopies; ++n) copy_v_issue(n);
+      cp_pending = false;
+      if (my_tiles > 1) copy_k(1);
+    }
+    if (kg == 1) __builtin_amdgcn_s_barrier();
+
+    f32x16 s[2];
+    x8 vop[4][4], pb[4];
+
+    // K operand reads of stage `it & 1`, d slices ks0..ks0+3 of both 32-key halves (16-bit K):
+    // kop[h][ks - ks0] = rows h*32 + l32, d = ks*16 + g*8 .. +7
+    auto read_k = [&](int it, int ks0, x8 (&kop)[2][4]) {
+      const uint8_t* ks_base = group_smem + (it & 1) * kStageBytes + k_rd_base;
 #pragma unroll
-        for (int i = 0; i < 16; ++i) s[mt][i] = 0.f;
+      for (int j = 0; j < 4; ++j)
+#pragma unroll
+        for (int h = 0; h < 2; ++h)
+          kop[h][j] = *reinterpret_cast<const x8*>(ks_base + h * 32 * kRowBytes + (k_rd_x ^ ((ks0 + j) << 5)));
+    };
+    // four d slices of S^T for both 32-key halves; the two accumulator chains alternate so that no
+    // MFMA waits for the one issued just before it
+    auto s_math = [&](int ks0, const x8 (&kop)[2][4], int j0) {  // d slices ks0+j0, ks0+j0+1
+#pragma unroll
+      for (int j = j0; j < j0 + 2; ++j)
+#pragma unroll
+        for (int h = 0; h < 2; ++h)
+          s[h] = TT::mfma(kop[h][j], qreg[ks0 + j], (ks0 + j) == 0 ? c_init : s[h]);
+    };
+    // fp8: S^T straight from LDS (four reads, four MFMAs)
+    auto s_fp8 = [&](int it) {
       if constexpr (kFp8) {
+        const uint8_t* ks_base = group_smem + (it & 1) * kStageBytes;
         i32x8 k8[2][2];  // [32-key tile][64-wide d slab]: 32 consecutive fp8 of row l32
 #pragma unroll
         for (int mt = 0; mt < 2; ++mt)
@@ -344,29 +462,35 @@ __global__ void __launch_bounds__(kThreads) sparse_fa_kernel(const FaParams p) {
           }
         __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
-        for (int mt = 0; mt < 2; ++mt)
+        for (int mt = 0; mt < 2; ++mt) {
+#pragma unroll
+          for (int i = 0; i < 16; ++i) s[mt][i] = 0.f;
 #pragma unroll
           for (int sl = 0; sl < 2; ++sl)
             s[mt] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(k8[mt][sl], qreg8[sl], s[mt], 0, 0, 0,
                                                                     0x7f7f7f7f, 0, 0x7f7f7f7f);
-      } else {
-        x8 ka[8], kb[8];
-#pragma unroll
-        for (int ks = 0; ks < 8; ++ks)
-          ka[ks] = *reinterpret_cast<const x8*>(ks_base + k_rd_base + (k_rd_x ^ (ks << 5)));
-#pragma unroll
-        for (int ks = 0; ks < 8; ++ks)
-          kb[ks] = *reinterpret_cast<const x8*>(ks_base + 32 * kRowBytes + k_rd_base + (k_rd_x ^ (ks << 5)));
-        __builtin_amdgcn_sched_barrier(0);
-#pragma unroll
-        for (int ks = 0; ks < 8; ++ks) s[0] = TT::mfma(ka[ks], qreg[ks], s[0]);
-#pragma unroll
-        for (int ks = 0; ks < 8; ++ks) s[1] = TT::mfma(kb[ks], qreg[ks], s[1]);
+        }
       }
-
-      // all V^T operands of the tile (4 slabs of 16 keys x 4 d tiles): in flight during the
-      // softmax, in the registers the K operands just vacated
-      x8 vop[4][4];
+    };
+    // O^T += V^T . P^T for 16-key slabs kk0, kk0+1
+    auto pv_math = [&](int kk) {
+#pragma unroll
+      for (int dt = 0; dt < 4; ++dt) o_acc[dt] = TT::mfma(vop[kk][dt], pb[kk], o_acc[dt]);
+    };
+    // VALU block of tile `it`: all V^T operands of the tile (4 slabs of 16 keys x 4 d tiles) are
+    // requested first and land during the softmax
+    auto valu_block = [&](int it, bool first) {
+      // V of tile `it` has landed once only the copies issued after it (K and V of tile it+1) are
+      // outstanding; after the barrier that holds for the whole kv group, and the group is done
+      // reading K of this stage, which tile it+2 may now overwrite
+      __builtin_amdgcn_s_setprio(0);
+      wait_copies(it + 1 < my_tiles ? kKCopies + kVCopies : 0);
+      __builtin_amdgcn_s_barrier();
+      if (it + 2 < my_tiles) copy_k(it + 2);
+      const int valid = tile_valid(it);
+      float cs = cq;
+      if constexpr (kFp8) cs = cq * ksc[s_blk[it]];
+      const uint8_t* vs_base = group_smem + (it & 1) * kStageBytes + kKBytes;
 #pragma unroll
       for (int kk = 0; kk < 4; ++kk) {
         const uint8_t* base = vs_base + kk * 16 * kRowBytes;
@@ -382,15 +506,21 @@ __global__ void __launch_bounds__(kThreads) sparse_fa_kernel(const FaParams p) {
         }
       }
       __builtin_amdgcn_sched_barrier(0);
-
-      // ---- online softmax (per lane: one q column, 32 kv values), log2 domain: x = s * cs ----
+      // online softmax (per lane: one q column, 32 kv values), log2 domain.  s holds x - m_run
+      // (fp8: raw dot products, scaled and shifted here because the scale changes per kv block)
+      if constexpr (kFp8) {
+#pragma unroll
+        for (int mt = 0; mt < 2; ++mt)
+#pragma unroll
+          for (int i = 0; i < 16; ++i) s[mt][i] = __builtin_fmaf(s[mt][i], cs, -m_run);
+      }
       if (valid < kTileKV) {
 #pragma unroll
         for (int mt = 0; mt < 2; ++mt)
 #pragma unroll
           for (int i = 0; i < 16; ++i) {
             const int kv = mt * 32 + (i >> 2) * 8 + g * 4 + (i & 3);
-            if (kv >= valid) s[mt][i] = -INFINITY;  // p = 0 whatever the scale
+            if (kv >= valid) s[mt][i] = -INFINITY;  // p = 0
           }
       }
       float mx = s[0][0];
@@ -398,39 +528,132 @@ __global__ void __launch_bounds__(kThreads) sparse_fa_kernel(const FaParams p) {
       for (int mt = 0; mt < 2; ++mt)
 #pragma unroll
         for (int i = 0; i < 16; ++i) mx = fmaxf(mx, s[mt][i]);
-      mx = fmaxf(mx, __shfl_xor(mx, 32, 64)) * cs;
-      // The running max is only raised when a row's new max exceeds it by more than kLazyLog2
-      // (p then stays <= 2^kLazyLog2, harmless in fp32 / bf16 / fp16): the rescale of O leaves the
-      // steady-state path.
-      if (__builtin_expect(__any(mx - m_run > kLazyLog2), 0)) {
-        const float m_new = fmaxf(m_run, mx);
-        const float scale = __builtin_amdgcn_exp2f(m_run - m_new);
-        d_part *= scale;
+      mx = max_across_halves(mx);  // row max relative to m_run
+      if (first || __builtin_expect(__any(mx > kLazyLog2), 0)) {
+        const float delta = first ? mx : fmaxf(mx, 0.f);
+        if (!first) {
+          const float scale = __builtin_amdgcn_exp2f(-delta);
+          d_part *= scale;
 #pragma unroll
-        for (int dt = 0; dt < 4; ++dt)
+          for (int dt = 0; dt < 4; ++dt)
 #pragma unroll
-          for (int i = 0; i < 16; ++i) o_acc[dt][i] *= scale;
-        m_run = m_new;
+            for (int i = 0; i < 16; ++i) o_acc[dt][i] *= scale;
+        }
+        m_run += delta;
+#pragma unroll
+        for (int mt = 0; mt < 2; ++mt)
+#pragma unroll
+          for (int i = 0; i < 16; ++i) s[mt][i] -= delta;
+#pragma unroll
+        for (int i = 0; i < 16; ++i) c_init[i] = -m_run;
       }
-      x8 pb[4];
-      float psum = 0.f;
 #pragma unroll
       for (int mt = 0; mt < 2; ++mt)
 #pragma unroll
-        for (int i = 0; i < 16; ++i) {
-          const float e = __builtin_amdgcn_exp2f(__builtin_fmaf(s[mt][i], cs, -m_run));
-          psum += e;
-          pb[mt * 2 + (i >> 3)][i & 7] = static_cast<T>(e);
-        }
+        for (int i = 0; i < 16; ++i)
+          pb[mt * 2 + (i >> 3)][i & 7] = static_cast<T>(__builtin_amdgcn_exp2f(s[mt][i]));
+      // the row sum is taken over the rounded p, as the reference does
+      float psum = 0.f;
+#pragma unroll
+      for (int j = 0; j < 4; ++j) psum = TT::add_elems(pb[j], psum);
       d_part += psum;
       __builtin_amdgcn_sched_barrier(0);
+    };
+    // start of an MFMA block: K of tile `it` has landed once only the copies issued after it (V of
+    // this tile, K of the next) are outstanding, and this wavefront's V^T reads of the previous tile
+    // have returned; after the barrier both hold for the whole kv group, so the V half of the other
+    // stage may be overwritten
+    auto open_mfma_block = [&](int it) {
+      wait_copies(kVCopies + (it + 1 < my_tiles ? kKCopies : 0));
+      __builtin_amdgcn_s_waitcnt(0xc07f);  // lgkmcnt(0)
+      __builtin_amdgcn_s_barrier();
+      __builtin_amdgcn_s_setprio(3);  // the MFMA block outranks the other kv group's softmax at issue
+      cp_pending = false;
+      if (it + 1 < my_tiles) copy_v_prepare(it + 1);
+    };
+    // four MFMAs are followed by one copy instruction of the next tile
+    auto after4 = [&](int n) {
+      if (n < kVCopies) copy_v_issue(n);
+      __builtin_amdgcn_sched_barrier(0);
+    };
 
-      // ---- O^T += V^T . P^T : four 16-key slabs x four 32-wide d tiles ----
+    if (my_tiles > 0) {
+      // first tile: nothing to multiply by V yet
+      open_mfma_block(0);
+      if constexpr (kFp8) {
+        s_fp8(0);
 #pragma unroll
-      for (int kk = 0; kk < 4; ++kk)
+        for (int n = 0; n < 8; ++n) after4(n);
+      } else {
+        x8 k_lo[2][4], k_hi[2][4];
+        read_k(0, 0, k_lo);
+        read_k(0, 4, k_hi);
+        __builtin_amdgcn_sched_barrier(0);
+        s_math(0, k_lo, 0);
+        after4(0);
+        after4(1);
+        s_math(0, k_lo, 2);
+        after4(2);
+        after4(3);
+        s_math(4, k_hi, 0);
+        after4(4);
+        after4(5);
+        s_math(4, k_hi, 2);
+        after4(6);
+        after4(7);
+      }
+      valu_block(0, true);
+      for (int it = 1; it < my_tiles; ++it) {
+        open_mfma_block(it);
+        if constexpr (kFp8) {
+          pv_math(0);
+          after4(0);
+          pv_math(1);
+          after4(1);
+          pv_math(2);
+          after4(2);
+          pv_math(3);
+          after4(3);
+          s_fp8(it);
+        } else {
+          // K operands are fetched under the MFMAs, half of them at a time, into the registers that
+          // the V^T operands free
+          x8 k_lo[2][4], k_hi[2][4];
+          pv_math(0);
+          after4(0);
+          pv_math(1);
+          after4(1);
+          read_k(it, 0, k_lo);
+          __builtin_amdgcn_sched_barrier(0);
+          pv_math(2);
+          after4(2);
+          pv_math(3);
+          after4(3);
+          read_k(it, 4, k_hi);
+          __builtin_amdgcn_sched_barrier(0);
+          s_math(0, k_lo, 0);
+          after4(4);
+          s_math(0, k_lo, 2);
+          after4(5);
+          s_math(4, k_hi, 0);
+          after4(6);
+          s_math(4, k_hi, 2);
+          after4(7);
+        }
+        valu_block(it, false);
+      }
+      // last MFMA block: P.V of the last tile
+      __builtin_amdgcn_s_waitcnt(0xc07f);  // lgkmcnt(0)
+      __builtin_amdgcn_s_barrier();
+      __builtin_amdgcn_s_setprio(3);
 #pragma unroll
-        for (int dt = 0; dt < 4; ++dt) o_acc[dt] = TT::mfma(vop[kk][dt], pb[kk], o_acc[dt]);
+      for (int kk = 0; kk < 4; ++kk) pv_math(kk);
+      __builtin_amdgcn_s_setprio(0);
+    } else {
+      __builtin_amdgcn_s_barrier();
     }
+    for (int i = calls_mine; i < calls_all; ++i) __builtin_amdgcn_s_barrier();
+    if (my_tiles == 0) m_run = kNegInf;  // nothing seen: weight 0 in the merge
 
     // ---- merge the two kv groups through LDS, then write the row ----
     __syncthreads();  // all tile reads done: the tile buffers can be reused
@@ -538,6 +761,8 @@ extern "C" int fo_sparse_fa_run(const void* q, const void* k, const void* v, voi
   for (int i = 0; i < 8; ++i)
     FO_REQUIRE(strides[i] % (dtype == FO_FP8_E4M3 && i < 4 ? 16 : 8) == 0 && strides[i] > 0,
                "sparse_fa: strides must be positive multiples of 16 bytes (128-bit accesses)");
+  FO_REQUIRE(k_stride_n < (int64_t(1) << 23) && v_stride_n < (int64_t(1) << 23),
+             "sparse_fa: k/v token strides must be below 2^23 elements (32-bit tile offsets)");
   if (dtype == FO_FP8_E4M3)
     FO_REQUIRE(q_scale && k_scale && q_blk_base && kv_blk_base && n_q_blocks > 0 && n_kv_blocks > 0,
                "sparse_fa: fp8 q/k need q_scale, k_scale, the block numbering and the scale row lengths");
