@@ -212,6 +212,9 @@ class BatchFlashOmniFAWithRaggedKVWrapper:
         qo_indptr_host = qo_indptr.to("cpu", torch.int32).contiguous()
         kv_indptr_host = kv_indptr.to("cpu", torch.int32).contiguous()
         total_num_rows = int(qo_indptr_host[-1])
+        # the attention kernel stages one row's kv block list in LDS (4096 entries)
+        if kv_indptr_host.numel() > 1 and int((kv_indptr_host[1:] - kv_indptr_host[:-1]).max()) > 4096 * 128:
+            raise NotImplementedError("requests longer than 524288 kv tokens are not supported")
 
         if self.is_cuda_graph_enabled:
             if self._max_total_num_rows is None:
