@@ -198,7 +198,7 @@ __global__ void __launch_bounds__(kThreads) sparse_fa_kernel(const FaParams p) {
   using TQK = typename std::conditional<kFp8, uint8_t, T>::type;
   constexpr int kStageBytes = G::kStageBytes, kKBytes = G::kKBytes, kGroupBytes = G::kGroupBytes;
   extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
-  __shared__ int s_next_row;
+  __shared__ int s_next_row[2];  // this row / the next one
   __shared__ int32_t s_blk[kMaxRowBlocks];  // kv block list of the current row
 
   const int tid = threadIdx.x, lane = tid & 63;
@@ -240,11 +240,12 @@ __global__ void __launch_bounds__(kThreads) sparse_fa_kernel(const FaParams p) {
       }
   }
 
-  for (;;) {
-    __syncthreads();  // everyone is done with s_next_row and with the previous row's LDS data
-    if (tid == 0) s_next_row = pop_row(p, blockIdx.x & (kXcds - 1));
-    __syncthreads();
-    const int w = __builtin_amdgcn_readfirstlane(s_next_row);  // uniform: row data goes through scalar loads
+  // The next row is popped by kv group 1 while kv group 0 combines and stores the current one
+  // (group 1 has nothing else to do then), so the queue atomics are off the critical path.
+  if (tid == 0) s_next_row[0] = pop_row(p, blockIdx.x & (kXcds - 1));
+  for (int row_it = 0;; ++row_it) {
+    __syncthreads();  // s_next_row is published; everyone is done with the previous row's LDS data
+    const int w = __builtin_amdgcn_readfirstlane(s_next_row[row_it & 1]);  // uniform: scalar loads below
     if (w < 0) break;
 
     const int req = p.row_req[w], qb = p.row_qb[w], head = p.row_head[w];
@@ -268,20 +269,13 @@ __global__ void __launch_bounds__(kThreads) sparse_fa_kernel(const FaParams p) {
         for (int j = 0; j < 8; ++j) reinterpret_cast<u32x4*>(dst)[j] = z;
         if (p.lse && g == 0) p.lse[q_tok * p.num_heads + head] = kNegInf;
       }
+      if (tid == kGroupThreads) s_next_row[(row_it + 1) & 1] = pop_row(p, blockIdx.x & (kXcds - 1));
       continue;
     }
 
-    // the row's kv block list goes to LDS: the main loop then has no global loads besides the
-    // tile copies, whose completion it tracks by counting (s_waitcnt vmcnt)
-    for (int i = tid; i < nb; i += kThreads) s_blk[i] = p.kv_idx[ptr0 + i];
-    __syncthreads();
-    // number of 64-key tiles; only the last listed block can be the request's ragged tail
-    int n_tiles = 2 * nb;
-    if (kv_len - s_blk[nb - 1] * kBlockKV <= kTileKV) n_tiles -= 1;
-    const int my_tiles = (n_tiles - kg + 1) >> 1;  // tiles kg, kg+2, ...
-
-    // Q operand: lane holds q row l32 of its q sub-tile, d = ks*16 + g*8 .. +7
-    // (fp8: d = slab*64 + g*32 .. +31 for the two 64-wide slabs)
+    // Q operand, requested first so that its latency overlaps the staging below: lane holds q row
+    // l32 of its q sub-tile, d = ks*16 + g*8 .. +7 (fp8: d = slab*64 + g*32 .. +31 for the two
+    // 64-wide slabs)
     x8 qreg[kFp8 ? 1 : 8];
     i32x8 qreg8[kFp8 ? 2 : 1];
     if constexpr (kFp8) {
@@ -295,12 +289,23 @@ __global__ void __launch_bounds__(kThreads) sparse_fa_kernel(const FaParams p) {
     } else {
       const T* src = reinterpret_cast<const T*>(qp) + q_tok * p.q_sn + static_cast<int64_t>(head) * p.q_sh + g * 8;
 #pragma unroll
-      for (int ks = 0; ks < 8; ++ks) {
-        // the softmax scale (log2 domain) is folded into Q, so S^T needs no multiply afterwards
-        const x8 raw = *reinterpret_cast<const x8*>(src + ks * 16);
+      for (int ks = 0; ks < 8; ++ks) qreg[ks] = *reinterpret_cast<const x8*>(src + ks * 16);
+    }
+    // the row's kv block list goes to LDS: the main loop then has no global loads besides the
+    // tile copies, whose completion it tracks by counting (s_waitcnt vmcnt)
+    for (int i = tid; i < nb; i += kThreads) s_blk[i] = p.kv_idx[ptr0 + i];
+    __syncthreads();
+    // number of 64-key tiles; only the last listed block can be the request's ragged tail
+    int n_tiles = 2 * nb;
+    if (kv_len - s_blk[nb - 1] * kBlockKV <= kTileKV) n_tiles -= 1;
+    const int my_tiles = (n_tiles - kg + 1) >> 1;  // tiles kg, kg+2, ...
+
+    // (bf16/fp16) the softmax scale (log2 domain) is folded into Q, so S^T needs no multiply
+    if constexpr (!kFp8) {
 #pragma unroll
-        for (int e = 0; e < 8; ++e) qreg[ks][e] = static_cast<T>(static_cast<float>(raw[e]) * c);
-      }
+      for (int ks = 0; ks < 8; ++ks)
+#pragma unroll
+        for (int e = 0; e < 8; ++e) qreg[ks][e] = static_cast<T>(static_cast<float>(qreg[ks][e]) * c);
     }
     // softmax scale in the log2 domain; with fp8 operands the per-block dequantisation scales of
     // q (one per row of the list) and k (one per kv block) are folded in tile by tile
@@ -673,6 +678,7 @@ __global__ void __launch_bounds__(kThreads) sparse_fa_kernel(const FaParams p) {
       md[(qs * 64 + lane) * 2 + 1] = d_part;
     }
     __syncthreads();
+    if (tid == kGroupThreads) s_next_row[(row_it + 1) & 1] = pop_row(p, blockIdx.x & (kXcds - 1));
     if (kg == 0) {
       const float m1 = md[(qs * 64 + lane) * 2 + 0], d1 = md[(qs * 64 + lane) * 2 + 1];
       const float m = fmaxf(m_run, m1);
