@@ -240,8 +240,9 @@ def cpu_baseline(layer):
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
-    ap.add_argument("--steps", type=int, default=50)
-    ap.add_argument("--warmup", type=int, default=10)
+    ap.add_argument("--steps", type=int, default=200)
+    ap.add_argument("--warmup", type=int, default=300,
+                    help="untimed steps; the clocks of an idle device need ~100 ms of load to settle")
     ap.add_argument("--configs", default="0,1,2,3,4")
     ap.add_argument("--no-cpu", action="store_true")
     ap.add_argument("--copy-calibration", action="store_true",

@@ -67,7 +67,7 @@ class DecodedWorkList:
         self.counts = torch.zeros(4, dtype=torch.int32, device=device)
         self.order = torch.empty(n, dtype=torch.int32, device=device)
         self.sched = torch.zeros(32, dtype=torch.int32, device=device)
-        self.scratch = torch.empty(2 * n + num_heads, dtype=torch.int32, device=device)
+        self.scratch = torch.empty(2 * n + 8192, dtype=torch.int32, device=device)
 
     def sizes(self) -> Tuple[int, int]:
         c = self.counts.cpu()

@@ -9,9 +9,12 @@
 // Besides the canonical list the decoder emits an execution order for the attention kernel:
 // `order` lists row positions grouped by head, heads dealt to the 8 XCDs round-robin (head % 8), so
 // that the workgroups of one XCD (which share an L2) walk the rows of the same few heads and find
-// that head's K/V in their L2.  sched[0..8] delimit the 8 per-XCD queues inside `order`,
-// sched[16..23] are the queue cursors and sched[24] a completion counter (all cleared here).
-// The order inside a head is not deterministic (atomic cursors); results do not depend on it.
+// that head's K/V in their L2.  Inside a head the rows go longest first (up to 32 length classes relative
+// to the longest row of the launch), which evens out the workgroups' finishing times when there are
+// only a few rows per CU.  sched[0..8] delimit the 8 per-XCD queues inside `order`, sched[16..23]
+// are the queue cursors, sched[24] a completion counter (all cleared here) and sched[25] the
+// longest row's kv count.  The order inside a length class is not deterministic (atomic cursors);
+// results do not depend on it.
 // Integer work, bounded by HBM traffic and launch latency; bit-exact by construction.
 //
 // Symbol semantics (reference: include/flashomni/attention/prefill.cuh:1284-1294, 1380-1403,
@@ -26,6 +29,17 @@ constexpr int kCountThreads = 256;  // 4 candidates per workgroup
 constexpr int kScanThreads = 1024;
 constexpr int kMaxHeads = 1024;
 constexpr int kXcds = 8;
+constexpr int kHistSlots = 8192;  // (head, length class) counters of the order layout
+
+// number of length classes for num_heads heads (32 up to 256 heads)
+__host__ __device__ __forceinline__ int len_classes(int32_t num_heads) {
+  const int k = kHistSlots / num_heads;
+  return k > 32 ? 32 : k;
+}
+// length class of a row with n kv blocks when the longest row has max_n: 0 = longest
+__device__ __forceinline__ int len_class(int32_t n, int32_t max_n, int n_classes) {
+  return static_cast<int>(static_cast<int64_t>(max_n - n) * n_classes / (max_n + 1));
+}
 
 struct Candidate {
   int32_t req, qb, head, nkv;
@@ -105,19 +119,26 @@ __global__ void __launch_bounds__(kScanThreads) decode_scan_kernel(
     int32_t* __restrict__ head_cursor, int32_t* __restrict__ sched) {
   __shared__ int32_t s_rows[kScanThreads];
   __shared__ int32_t s_kv[kScanThreads];
-  __shared__ int32_t s_hist[kMaxHeads];
+  __shared__ int32_t s_hist[kHistSlots];
+  __shared__ int32_t s_max;
   const int tid = threadIdx.x;
-  for (int h = tid; h < num_heads; h += kScanThreads) s_hist[h] = 0;
+  const int n_classes = len_classes(num_heads);
+  for (int h = tid; h < num_heads * n_classes; h += kScanThreads) s_hist[h] = 0;
+  if (tid == 0) s_max = 0;
   __syncthreads();
   const int64_t chunk = (n_cand + kScanThreads - 1) / kScanThreads;
   const int64_t lo = tid * chunk, hi = (lo + chunk < n_cand) ? lo + chunk : n_cand;
-  int32_t rows = 0, kv = 0;
+  int32_t rows = 0, kv = 0, mx = 0;
   for (int64_t c = lo; c < hi; ++c) {
-    const int32_t a = act[c];
-    rows += a;
+    rows += act[c];
     kv += cnt[c];
-    if (a) atomicAdd(&s_hist[c % num_heads], 1);
+    mx = max(mx, cnt[c]);
   }
+  atomicMax(&s_max, mx);
+  __syncthreads();
+  const int32_t max_n = s_max;
+  for (int64_t c = lo; c < hi; ++c)
+    if (act[c]) atomicAdd(&s_hist[(c % num_heads) * n_classes + len_class(cnt[c], max_n, n_classes)], 1);
   s_rows[tid] = rows;
   s_kv[tid] = kv;
   __syncthreads();
@@ -154,13 +175,15 @@ __global__ void __launch_bounds__(kScanThreads) decode_scan_kernel(
     int32_t pos = 0;
     for (int x = 0; x < kXcds; ++x) {
       sched[x] = pos;
-      for (int h = x; h < num_heads; h += kXcds) {
-        head_cursor[h] = pos;
-        pos += s_hist[h];
-      }
+      for (int h = x; h < num_heads; h += kXcds)
+        for (int k = 0; k < n_classes; ++k) {
+          head_cursor[h * n_classes + k] = pos;
+          pos += s_hist[h * n_classes + k];
+        }
     }
     sched[kXcds] = pos;
     for (int i = kXcds + 1; i < 32; ++i) sched[i] = 0;
+    sched[25] = max_n;
   }
 }
 
@@ -173,7 +196,8 @@ __global__ void __launch_bounds__(kCountThreads) decode_fill_kernel(
     const int32_t* __restrict__ kv_pos, int32_t* __restrict__ row_req,
     int32_t* __restrict__ row_qb, int32_t* __restrict__ row_head,
     int32_t* __restrict__ kv_row_ptr, int32_t* __restrict__ kv_idx,
-    int32_t* __restrict__ head_cursor, int32_t* __restrict__ order) {
+    int32_t* __restrict__ head_cursor, int32_t* __restrict__ order,
+    const int32_t* __restrict__ counts, const int32_t* __restrict__ sched) {
   const int lane = threadIdx.x % kWave;
   const int64_t c = static_cast<int64_t>(blockIdx.x) * (kCountThreads / kWave) + threadIdx.x / kWave;
   if (c >= n_cand) return;
@@ -187,7 +211,9 @@ __global__ void __launch_bounds__(kCountThreads) decode_fill_kernel(
     row_qb[pos] = cd.qb;
     row_head[pos] = cd.head;
     kv_row_ptr[pos] = out;
-    order[atomicAdd(&head_cursor[cd.head], 1)] = pos;
+    const int32_t listed = (c + 1 < n_cand ? kv_pos[c + 1] : counts[1]) - out;  // kv blocks of this row
+    const int n_classes = len_classes(num_heads);
+    order[atomicAdd(&head_cursor[cd.head * n_classes + len_class(listed, sched[25], n_classes)], 1)] = pos;
   }
   if (cd.nkv <= 0) return;
   if (is_full) {
@@ -257,7 +283,7 @@ extern "C" int fo_decode_sparse(const uint8_t* sparse_info, const uint8_t* spars
     decode_fill_kernel<<<grid, kCountThreads, 0, s>>>(
         sparse_info, sparse_kv_info, sparse_info_indptr, sparse_kv_info_indptr, blk_req, blk_qb,
         kv_indptr, n_cand, num_heads, block_kv, is_full, act, cnt, row_req, row_qb, row_head,
-        kv_row_ptr, kv_idx, head_cursor, order);
+        kv_row_ptr, kv_idx, head_cursor, order, counts, sched);
     FO_CHECK_LAUNCH();
   }
   return FO_OK;

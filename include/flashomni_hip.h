@@ -88,13 +88,14 @@ int fo_prefill_plan(void* float_ws, size_t float_ws_bytes, void* int_ws_dev, voi
  *   kv_row_ptr [n_rows+1], kv_idx [nnz]  kept kv blocks of each row, ascending
  *   counts[0] = n_rows, counts[1] = nnz, counts[2..3] = 0
  *   order [n_rows]   execution order for the attention kernel: canonical row positions grouped by
- *                    head, heads dealt round-robin to 8 queues (head % 8, one queue per XCD); the
- *                    order inside one head is unspecified
+ *                    head, heads dealt round-robin to 8 queues (head % 8, one queue per XCD);
+ *                    inside one head longer rows first (up to 32 length classes), otherwise unspecified
  *   sched [32]       sched[0..8] = queue boundaries inside `order`, sched[16..23] = queue cursors
- *                    and sched[24] = completion counter, both cleared to 0
+ *                    and sched[24] = completion counter, both cleared to 0; sched[25] = kv count of
+ *                    the longest row
  * is_full != 0 ignores the symbol tensors (which may be NULL) and lists everything
  * (csrc/batch_sparseFA.cu:123-128).
- * `scratch` needs 2*n_blk*H + H int32.
+ * `scratch` needs 2*n_blk*H + 8192 int32.
  * ------------------------------------------------------------------------------------------- */
 int fo_sparse_block_table(const int32_t* qo_indptr_host, uint32_t batch_size, uint32_t block_q,
                           int32_t* blk_req_host, int32_t* blk_qb_host, int64_t capacity,
