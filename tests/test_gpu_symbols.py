@@ -108,3 +108,37 @@ def test_decoder_full_size_configs(dev, index):
     for g, e in zip(got, exp):
         np.testing.assert_array_equal(g, e)
     assert len(got[0]) == wl.active_rows and len(got[4]) == wl.computed_blocks
+
+
+@pytest.mark.parametrize("case", CASES[:3])
+def test_decoder_execution_order(dev, case):
+    """`order` / `sched`: a permutation of the rows, cut into 8 queues by head % 8, heads back to
+    back inside a queue, and inside a head no row is followed by one of a longer length class."""
+    import flashomni_amd as fo
+    ql, kl, heads, pa, pk = case
+    m = make_ragged_masks(ql, kl, heads, pa, pk, seed=7)
+    ws = torch.empty(128 << 20, dtype=torch.uint8, device=dev)
+    w = fo.BatchFlashOmniFAWithRaggedKVWrapper(ws)
+    w.plan(torch.from_numpy(m["qo_indptr"]), torch.from_numpy(m["kv_indptr"]), heads, heads, 128,
+           q_data_type=torch.bfloat16)
+    t = lambda a: torch.from_numpy(a).to(dev)
+    wl = w.decode(t(m["packed_info"]), t(m["packed_keep"]), t(m["info_indptr"]), t(m["keep_indptr"]))
+    n_rows, _ = wl.sizes()
+    order = wl.order[:n_rows].cpu().numpy()
+    sched = wl.sched.cpu().numpy()
+    row_head = wl.row_head[:n_rows].cpu().numpy()
+    ptr = wl.kv_row_ptr[:n_rows + 1].cpu().numpy()
+    lens = ptr[1:] - ptr[:-1]
+    assert sorted(order.tolist()) == list(range(n_rows))
+    assert sched[0] == 0 and sched[8] == n_rows and (sched[16:25] == 0).all()
+    max_n = int(lens.max()) if n_rows else 0
+    assert sched[25] == max_n
+    n_classes = min(32, 8192 // heads)
+    for x in range(8):
+        seg = order[sched[x]:sched[x + 1]]
+        h = row_head[seg]
+        assert (h % 8 == x).all()
+        assert (np.diff(h) >= 0).all()          # heads back to back, ascending
+        cls = (max_n - lens[seg]).astype(np.int64) * n_classes // (max_n + 1)
+        same_head = np.diff(h) == 0
+        assert (np.diff(cls)[same_head] >= 0).all()   # longest class first inside a head
