@@ -92,8 +92,10 @@ struct GemmParams {
   void* y;           // [B, M, N]
   const uint8_t* sparse_info;
   const int32_t* sparse_info_indptr;
-  const int32_t* quads;  // kQuadInts per quad, queue by queue
+  const int32_t* quads;  // kQuadInts per quad, queue by queue; null: every unit is computed and the
+                         // quads are enumerated arithmetically (GEMM-O, GEMM-Q with is_full)
   const int32_t* qoff;   // qoff[0..8] queue boundaries inside `quads`
+  int32_t n_row_tiles, n_col_tiles, n_cp;  // geometry for the arithmetic enumeration
   int32_t batch, m, n, k;
   int32_t sparse_q_size, num_heads, head_dim, num_text_tokens;
   int32_t flag;       // GEMM-Q: is_full.  GEMM-O: is_for_cached
@@ -285,12 +287,57 @@ __global__ void __launch_bounds__(kThreads) gemm_kernel(const GemmParams p) {
 
   const int xcd = blockIdx.x & (kXcds - 1), slot = blockIdx.x >> 3;
   const int per_xcd = gridDim.x >> 3;  // host launches a multiple of 8 workgroups
-  const int q_lo = p.qoff[xcd], q_len = p.qoff[xcd + 1] - q_lo;
+  // dense enumeration (same order as the list kernel's): per batch, windows of 16 token blocks
+  // (8 row pairs; the last window may be shorter), column pairs inside a window, row pairs inside
+  // a column pair
+  const int full_w = p.n_row_tiles / kWindow, last_rows = p.n_row_tiles % kWindow;
+  const int last_q = (last_rows + 1) / 2;
+  const int quads_per_batch = (full_w * (kWindow / 2) + last_q) * p.n_cp;
+  int q_lo, q_len;
+  if (p.quads) {
+    q_lo = p.qoff[xcd];
+    q_len = p.qoff[xcd + 1] - q_lo;
+  } else {
+    const int64_t total = static_cast<int64_t>(quads_per_batch) * p.batch;
+    q_lo = static_cast<int>(total * xcd / kXcds);
+    q_len = static_cast<int>(total * (xcd + 1) / kXcds) - q_lo;
+  }
 
   for (int work = slot; work < q_len; work += per_xcd) {
-    const int32_t* e = p.quads + kQuadInts * static_cast<int64_t>(q_lo + work);
-    const int bz = e[0], valid = e[5];
-    const int r[2] = {e[1], e[2]}, c[2] = {e[3], e[4]};
+    int bz, valid, r[2], c[2];
+    if (p.quads) {
+      const int32_t* e = p.quads + kQuadInts * static_cast<int64_t>(q_lo + work);
+      bz = e[0];
+      r[0] = e[1];
+      r[1] = e[2];
+      c[0] = e[3];
+      c[1] = e[4];
+      valid = e[5];
+    } else {
+      const int q = q_lo + work;
+      bz = q / quads_per_batch;
+      int rem = q - bz * quads_per_batch;
+      int w, cp, i, rows;
+      if (rem < full_w * p.n_cp * (kWindow / 2)) {
+        const int cell = rem / (kWindow / 2);
+        i = rem - cell * (kWindow / 2);
+        w = cell / p.n_cp;
+        cp = cell - w * p.n_cp;
+        rows = kWindow;
+      } else {
+        rem -= full_w * p.n_cp * (kWindow / 2);
+        cp = rem / last_q;
+        i = rem - cp * last_q;
+        w = full_w;
+        rows = last_rows;
+      }
+      const bool has_r1 = 2 * i + 1 < rows, has_c1 = 2 * cp + 1 < p.n_col_tiles;
+      r[0] = w * kWindow + 2 * i;
+      r[1] = has_r1 ? r[0] + 1 : r[0];
+      c[0] = 2 * cp;
+      c[1] = has_c1 ? c[0] + 1 : c[0];
+      valid = 0x1 | (has_c1 ? 0x2 : 0) | (has_r1 ? 0x4 : 0) | (has_r1 && has_c1 ? 0x8 : 0);
+    }
     const bool my_valid = (valid >> (wr * 2 + wc)) & 1;
 
     // ---- k-step list ----
@@ -576,6 +623,23 @@ int launch(GemmParams& p, const ListGeom& gm, bool use_flags, void* workspace, h
   }
   int64_t max_quads = 0;
   workspace_ints(gm, &max_quads);
+  p.n_row_tiles = gm.n_row_tiles;
+  p.n_col_tiles = gm.n_col_tiles;
+  p.n_cp = gm.n_cp;
+  int num_cu = fo_num_cu();
+  if (num_cu <= 0) return fo::fail(FO_ERR_HIP, "gemm: no device");
+  int64_t grid = (num_cu + kXcds - 1) / kXcds * kXcds;  // one persistent workgroup per CU
+  const int64_t cap = (max_quads + kXcds - 1) / kXcds * kXcds;
+  if (grid > cap) grid = cap;
+  if (grid < kXcds) grid = kXcds;
+  if (!use_flags) {
+    // every unit is computed: no list, the kernel enumerates the quads itself
+    p.quads = nullptr;
+    p.qoff = nullptr;
+    gemm_kernel<T, kReduce><<<static_cast<unsigned>(grid), kThreads, kSmemBytes, stream>>>(p);
+    FO_CHECK_LAUNCH();
+    return FO_OK;
+  }
   int32_t* qoff = static_cast<int32_t*>(workspace);
   int32_t* quads = qoff + 16;
   ListArgs la;
@@ -590,12 +654,6 @@ int launch(GemmParams& p, const ListGeom& gm, bool use_flags, void* workspace, h
   FO_CHECK_LAUNCH();
   p.quads = quads;
   p.qoff = qoff;
-  int num_cu = fo_num_cu();
-  if (num_cu <= 0) return fo::fail(FO_ERR_HIP, "gemm: no device");
-  int64_t grid = (num_cu + kXcds - 1) / kXcds * kXcds;  // one persistent workgroup per CU
-  const int64_t cap = (max_quads + kXcds - 1) / kXcds * kXcds;
-  if (grid > cap) grid = cap;
-  if (grid < kXcds) grid = kXcds;
   gemm_kernel<T, kReduce><<<static_cast<unsigned>(grid), kThreads, kSmemBytes, stream>>>(p);
   FO_CHECK_LAUNCH();
   return FO_OK;
@@ -603,7 +661,7 @@ int launch(GemmParams& p, const ListGeom& gm, bool use_flags, void* workspace, h
 
 int check_common(const void* x, const void* w, void* y, int dtype, int32_t batch, int32_t m,
                  int32_t n, int32_t k, int32_t sparse_q_size, int32_t num_qo_heads,
-                 void* workspace, int64_t workspace_bytes) {
+                 void* workspace, int64_t workspace_bytes, bool needs_list) {
   FO_REQUIRE(dtype == FO_BF16 || dtype == FO_F16, "gemm: only bf16 / fp16 operands are supported");
   FO_REQUIRE(batch > 0 && m > 0 && n > 0 && k > 0, "gemm: bad shape");
   FO_REQUIRE(n % 128 == 0 && k % 32 == 0, "only support N %% 128 == 0, K %% 32 == 0 (got N=%d K=%d)",
@@ -617,6 +675,7 @@ int check_common(const void* x, const void* w, void* y, int dtype, int32_t batch
   const ListGeom gm = make_geom(batch, m, n);
   FO_REQUIRE(static_cast<int64_t>(batch) * gm.n_win * gm.n_cp < (int64_t(1) << 24), "gemm: too many tiles");
   const int64_t need = 4 * workspace_ints(gm, nullptr);
+  if (!needs_list) return FO_OK;  // the workspace only holds the tile list
   if (!workspace || workspace_bytes < need || (reinterpret_cast<uintptr_t>(workspace) & 15))
     return fo::fail(FO_ERR_WORKSPACE, "gemm: workspace of %lld bytes (16-byte aligned) required, got %lld",
                     static_cast<long long>(need), static_cast<long long>(workspace_bytes));
@@ -636,7 +695,7 @@ extern "C" int fo_gemm_q(const void* x, const void* w, const void* bias, void* y
                          const int32_t* sparse_info_indptr, int32_t num_text_tokens, int is_full,
                          void* workspace, int64_t workspace_bytes, void* stream) {
   if (int rc = check_common(x, w, y, dtype, batch, m, n, k, sparse_q_size, num_qo_heads, workspace,
-                            workspace_bytes))
+                            workspace_bytes, !is_full))
     return rc;
   FO_REQUIRE(is_full || (sparse_info && sparse_info_indptr),
              "gemm: sparse_info and sparse_info_indptr are required unless is_full");
@@ -664,7 +723,7 @@ extern "C" int fo_gemm_o(const void* x, const void* w, const void* bias, void* y
                          int32_t num_text_tokens, int is_for_cached, void* workspace,
                          int64_t workspace_bytes, void* stream) {
   if (int rc = check_common(x, w, y, dtype, batch, m, n, k, sparse_q_size, num_qo_heads, workspace,
-                            workspace_bytes))
+                            workspace_bytes, false))
     return rc;
   FO_REQUIRE(sparse_info && sparse_info_indptr, "gemm_reduction: sparse_info is required");
   FO_REQUIRE(num_text_tokens >= 0, "gemm: negative num_text_tokens");

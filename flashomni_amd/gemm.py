@@ -115,8 +115,7 @@ def flashomni_gemm_reduction(
         bias = bias.contiguous()
     info, indptr = _symbols(sparse_info, sparse_info_indptr, A.device)
     L = _lib.lib()
-    ws_bytes = L.fo_gemm_workspace_bytes(Bsz, M, N)
-    workspace = torch.empty(ws_bytes, dtype=torch.uint8, device=A.device)  # tile-list scratch
+    workspace, ws_bytes = None, 0  # the reduction visits every token block: no tile list
     _lib.check(L.fo_gemm_o(
         _lib.ptr(A), _lib.ptr(B), _lib.ptr(bias), _lib.ptr(out), _lib.dtype_code(A.dtype), kind,
         bias_code, _lib.dtype_code(out_dtype), Bsz, M, N, A.shape[2], sparse_q_size, num_qo_heads,

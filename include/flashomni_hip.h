@@ -171,7 +171,8 @@ int fo_gemm_q(const void* x, const void* w, const void* bias, void* y, int dtype
  *           slice selection).
  * bias_dtype: the activation dtype (as in the reference) or FO_F32 for the matrix form;
  * y_dtype: the activation dtype or FO_F32 (so a cached partial can stay in fp32).
- * hd must be a multiple of 32.  `workspace` as for fo_gemm_q.
+ * hd must be a multiple of 32.  `workspace` is not used (every token block is visited, the tile
+ * order is computed arithmetically) and may be NULL; fo_gemm_q with is_full != 0 likewise.
  * ------------------------------------------------------------------------------------------- */
 int fo_gemm_o(const void* x, const void* w, const void* bias, void* y, int dtype, int bias_kind,
               int bias_dtype, int y_dtype, int32_t batch, int32_t m, int32_t n, int32_t k,
