@@ -376,11 +376,17 @@ __global__ void __launch_bounds__(kThreads) sparse_fa_kernel(const FaParams p) {
     const uint8_t* cp_v = nullptr;
     uint32_t cp_vdst = 0;
     bool cp_pending = false;
-    auto copy_v_prepare = [&](int j) {
+    int cp_valid = kTileKV;
+    // scalar part (any time: it touches no LDS stage)
+    auto copy_v_address = [&](int j) {
       const int start = __builtin_amdgcn_readfirstlane(tile_start(j));
-      const int valid = min(kTileKV, kv_len - start);
+      cp_valid = min(kTileKV, kv_len - start);
       cp_v = reinterpret_cast<const uint8_t*>(v_head + static_cast<int64_t>(start) * p.v_sn);
       cp_vdst = lds_group + (j & 1) * kStageBytes + kKBytes + qs * 1024;
+    };
+    // once the target stage is free: arm the one-by-one issue, or issue a ragged tile at once
+    auto copy_v_prepare = [&]() {
+      const int valid = cp_valid;
       cp_pending = valid == kTileKV;
       if (__builtin_expect(!cp_pending, 0)) {
 #pragma unroll
@@ -421,11 +427,15 @@ __global__ void __launch_bounds__(kThreads) sparse_fa_kernel(const FaParams p) {
     // copy order of a wavefront: K0, V0, K1 | V1 (MFMA block 0) | K2 (VALU block 0) | V2 | K3 | ...
     if (my_tiles > 0) {
       copy_k(0);
-      copy_v_prepare(0);
+      copy_v_address(0);
+      copy_v_prepare();
 #pragma unroll
       for (int n = 0; n < kVCopies; ++n) copy_v_issue(n);
       cp_pending = false;
-      if (my_tiles > 1) copy_k(1);
+      if (my_tiles > 1) {
+        copy_k(1);
+        copy_v_address(1);
+      }
     }
     if (kg == 1) __builtin_amdgcn_s_barrier();
 
@@ -562,6 +572,7 @@ __global__ void __launch_bounds__(kThreads) sparse_fa_kernel(const FaParams p) {
 #pragma unroll
       for (int j = 0; j < 4; ++j) psum = TT::add_elems(pb[j], psum);
       d_part += psum;
+      if (it + 2 < my_tiles) copy_v_address(it + 2);  // for the V copies of the next MFMA block
       __builtin_amdgcn_sched_barrier(0);
     };
     // start of an MFMA block: K of tile `it` has landed once only the copies issued after it (V of
@@ -574,7 +585,7 @@ __global__ void __launch_bounds__(kThreads) sparse_fa_kernel(const FaParams p) {
       __builtin_amdgcn_s_barrier();
       __builtin_amdgcn_s_setprio(3);  // the MFMA block outranks the other kv group's softmax at issue
       cp_pending = false;
-      if (it + 1 < my_tiles) copy_v_prepare(it + 1);
+      if (it + 1 < my_tiles) copy_v_prepare();  // addresses were worked out in the last softmax block
     };
     // four MFMAs are followed by one copy instruction of the next tile
     auto after4 = [&](int n) {
