@@ -170,20 +170,55 @@ __global__ void __launch_bounds__(kScanThreads) decode_scan_kernel(
     counts[3] = 0;
     kv_row_ptr[n_rows] = nnz;
   }
-  // execution order layout: queue x holds heads x, x+8, x+16, ... back to back
-  if (tid == 0) {
-    int32_t pos = 0;
-    for (int x = 0; x < kXcds; ++x) {
-      sched[x] = pos;
-      for (int h = x; h < num_heads; h += kXcds)
-        for (int k = 0; k < n_classes; ++k) {
-          head_cursor[h * n_classes + k] = pos;
-          pos += s_hist[h * n_classes + k];
-        }
+  // execution order layout: queue x holds heads x, x+8, x+16, ... back to back, each head's length
+  // classes in order.  Exclusive prefix sum of the histogram taken in that order: every thread owns
+  // a run of consecutive entries, wavefront scan by lane shifts, then the sixteen wavefront totals.
+  __syncthreads();  // s_rows / s_kv are free again
+  {
+    const int n_ent = num_heads * n_classes;
+    const int per = (n_ent + kScanThreads - 1) / kScanThreads;
+    const int e_lo = min(tid * per, n_ent), e_hi = min(e_lo + per, n_ent);
+    // entry j of the order -> slot of the histogram: j / n_classes is the head's rank in queue order
+    auto slot_of = [&](int j, int* queue) {
+      const int rank = j / n_classes, k = j - rank * n_classes;
+      int x = 0, base = 0;
+      for (; x < kXcds; ++x) {
+        const int c = num_heads > x ? (num_heads - x + kXcds - 1) / kXcds : 0;  // heads of queue x
+        if (rank < base + c) break;
+        base += c;
+      }
+      *queue = x;
+      return (x + kXcds * (rank - base)) * n_classes + k;
+    };
+    int32_t mine = 0;
+    int qx;
+    for (int j = e_lo; j < e_hi; ++j) mine += s_hist[slot_of(j, &qx)];
+    const int lane = tid & 63, wave = tid >> 6;
+    int32_t incl = mine;
+#pragma unroll
+    for (int d = 1; d < 64; d <<= 1) {
+      const int32_t up = __shfl_up(incl, d, 64);
+      if (lane >= d) incl += up;
     }
-    sched[kXcds] = pos;
-    for (int i = kXcds + 1; i < 32; ++i) sched[i] = 0;
-    sched[25] = max_n;
+    if (lane == 63) s_rows[wave] = incl;
+    __syncthreads();
+    int32_t pos = incl - mine;
+    for (int w = 0; w < wave; ++w) pos += s_rows[w];
+    for (int j = e_lo; j < e_hi; ++j) {
+      const int slot = slot_of(j, &qx);
+      head_cursor[slot] = pos;
+      if (j % n_classes == 0 && slot / n_classes == qx) sched[qx] = pos;  // first head of queue qx
+      pos += s_hist[slot];
+    }
+    if (tid == 0) {
+      int32_t total = 0;
+      for (int w = 0; w < kScanThreads / 64; ++w) total += s_rows[w];
+      // queues without heads (fewer than 8 heads) are empty and sit at the end
+      for (int x = num_heads; x < kXcds; ++x) sched[x] = total;
+      sched[kXcds] = total;
+      for (int i = kXcds + 1; i < 32; ++i) sched[i] = 0;
+      sched[25] = max_n;
+    }
   }
 }
 

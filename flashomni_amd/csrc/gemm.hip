@@ -211,7 +211,7 @@ struct ListArgs {
 __global__ void __launch_bounds__(kListThreads) gemm_quads_kernel(ListArgs a, ListGeom gm,
                                                                   int32_t* __restrict__ quads,
                                                                   int32_t* __restrict__ qoff) {
-  __shared__ int32_t s_cnt[kListThreads];
+  __shared__ int32_t s_cnt[kListThreads / 64];
   const int tid = threadIdx.x;
   const int n_cells = gm.batch * gm.n_win * gm.n_cp;
   int b, row0, cp;
@@ -225,20 +225,31 @@ __global__ void __launch_bounds__(kListThreads) gemm_quads_kernel(ListArgs a, Li
                a.head_dim, a.num_text_tokens, &b, &row0, &cp, &m0, &m1);
     for_each_quad(m0, m1, [&](int, int, int) { ++my_cnt; });
   }
-  s_cnt[tid] = my_cnt;
-  __syncthreads();
-  for (int d = 1; d < kListThreads; d <<= 1) {
-    const int32_t v = tid >= d ? s_cnt[tid - d] : 0;
-    __syncthreads();
-    s_cnt[tid] += v;
-    __syncthreads();
+  // inclusive scan of the per-thread counts: inside a wavefront by lane shifts, then over the
+  // sixteen wavefront totals
+  const int lane = tid & 63, wave = tid >> 6;
+  int32_t incl = my_cnt;
+#pragma unroll
+  for (int d = 1; d < 64; d <<= 1) {
+    const int32_t up = __shfl_up(incl, d, 64);
+    if (lane >= d) incl += up;
   }
-  const int32_t total = s_cnt[kListThreads - 1];
+  if (lane == 63) s_cnt[wave] = incl;
+  __syncthreads();
+  int32_t wave_base = 0, total = 0;
+#pragma unroll
+  for (int w = 0; w < kListThreads / 64; ++w) {
+    const int32_t t = s_cnt[w];
+    if (w < wave) wave_base += t;
+    total += t;
+  }
+  const int32_t my_incl = wave_base + incl;
   if (tid <= kXcds) qoff[tid] = static_cast<int32_t>(static_cast<int64_t>(total) * tid / kXcds);
-  int32_t q = s_cnt[tid] - my_cnt;
+  int32_t q = my_incl - my_cnt;
   for (int cell = lo; cell < hi; ++cell) {
-    cell_masks(gm, cell, a.use_flags, a.sparse_info, a.sparse_info_indptr, a.sparse_q_size, a.num_heads,
-               a.head_dim, a.num_text_tokens, &b, &row0, &cp, &m0, &m1);
+    if (per > 1)  // with one cell per thread the masks of the counting pass are still at hand
+      cell_masks(gm, cell, a.use_flags, a.sparse_info, a.sparse_info_indptr, a.sparse_q_size, a.num_heads,
+                 a.head_dim, a.num_text_tokens, &b, &row0, &cp, &m0, &m1);
     for_each_quad(m0, m1, [&](int r0, int r1, int valid) {
       int32_t* e = quads + kQuadInts * static_cast<int64_t>(q);
       e[0] = b;
