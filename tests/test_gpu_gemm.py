@@ -164,3 +164,31 @@ def test_flux_gemm_o_full_config(dev):
     assert max_abs(cache.cpu(), exp_cache) <= 1e-3
     dense = F.linear(a.float(), w.float(), b.float())
     assert max_abs(final, dense) <= MAX_ABS and rel_l2(final, dense) <= REL_L2
+
+
+@pytest.mark.parametrize("shape", [(2, 2500, 384, 256), (1, 4224, 640, 128), (3, 130, 128, 64)])
+def test_dense_tile_enumeration_geometries(dev, shape):
+    """Every unit computed (is_full GEMM-Q, GEMM-O): the kernel enumerates its tiles arithmetically.
+    More than one 16-block window, a short last window, an odd number of column tiles, a token
+    tail and several batches; every output element must be written and right."""
+    import flashomni_amd as fo
+    batch, m, n, k = shape
+    heads = n // 128
+    x, w, b = _operands(batch, m, n, k, torch.bfloat16, seed=m + k)
+    out0 = sentinel_like((batch, m, n), torch.bfloat16)
+    out = out0.clone().to(dev)
+    fo.flashomni_gemm(x.to(dev), w.to(dev), heads, bias=b.to(dev), out=out, is_full=True)
+    exp = F.linear(x.float(), w.float(), b.float())
+    assert max_abs(out.cpu(), exp) <= MAX_ABS and rel_l2(out.cpu(), exp) <= REL_L2
+    # GEMM-O over the same geometry (K = N there: heads slice the contraction)
+    nqb = (m + 127) // 128
+    info, packed, indptr = _flags(batch, nqb, heads, 0.5, seed=n)
+    a = torch.randn(batch, m, n, generator=torch.Generator().manual_seed(3)).to(torch.bfloat16)
+    wo = (torch.randn(n, n, generator=torch.Generator().manual_seed(4)) * 0.05).to(torch.bfloat16)
+    pk, ip = torch.from_numpy(packed).to(dev), torch.from_numpy(indptr).to(dev)
+    cache = fo.flashomni_gemm_reduction(a.to(dev), wo.to(dev), heads, pk, ip, 0, bias=None,
+                                        is_for_cache=True, out_dtype=torch.float32)
+    final = fo.flashomni_gemm_reduction(a.to(dev), wo.to(dev), heads, pk, ip, 0, bias=cache,
+                                        is_for_cache=False)
+    exp = torch.matmul(a.float(), wo.float().t())       # cache + final = the full product
+    assert max_abs(final.cpu(), exp) <= 4e-2 and rel_l2(final.cpu(), exp) <= REL_L2
