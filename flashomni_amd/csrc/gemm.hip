@@ -16,8 +16,9 @@
 // (16-token-block window, column pair) cell into quads: rows flagged in both columns pair up into
 // full quads, rows flagged in one column pair up among themselves, leftovers are merged; a 4-bit
 // mask says which units of a quad exist (the others are computed on duplicated tiles and dropped).
-// GEMM-O runs the same kernel over unflagged quads and walks the union of the two token blocks'
-// selected heads; a token block that does not select a head gets that k step's X operand zeroed.
+// GEMM-O (and GEMM-Q with is_full) computes every unit: no list then, the kernel derives its quads
+// from the shape.  GEMM-O walks the union of the two token blocks' selected heads; a token block
+// that does not select a head gets that k step's X operand zeroed.
 //
 // Data path.  BK = 32.  Operand tiles go global -> LDS directly (global_load_lds_dwordx4) into a
 // 4-stage ring, three k steps ahead of the math, one barrier per k step.  A wavefront's copy lands

@@ -3,11 +3,11 @@
 // One workgroup = 8 wavefronts (512 lanes, two per SIMD) owns one work-list row = one (request,
 // 128-row q-block, head).  Wavefront w serves q rows 32*(w%4)..+31 and kv group w/4: the row's
 // 64-key tiles are dealt alternately to the two kv groups, each group keeps its own running
-// (max, sum, O) state and the two states are merged through LDS when the row ends.  Two wavefronts
-// per SIMD let one wavefront's softmax (VALU) run under the other's matrix products (MFMA);
-// splitting a row over two kv groups halves its latency, which is what bounds the tail when there
-// are only a few rows per CU.  LDS operand reads are issued in batches ahead of the MFMAs that
-// consume them (one wavefront can start a 128-bit LDS read only every ~32 cycles).
+// (max, sum, O) state and the two states are merged through LDS when the row ends.  Splitting a
+// row over two kv groups halves its latency, which is what bounds the tail when there are only a
+// few rows per CU, and gives every SIMD two wavefronts that are kept in opposite phases: one
+// feeds the matrix cores (P.V of its previous tile, K.Q^T of its next) while the other runs its
+// softmax on the vector ALUs (see the main loop).
 // Only the kv blocks listed for the row are ever loaded; q-blocks that are not in the list are
 // never visited, so their output bytes stay untouched.
 //
@@ -18,8 +18,9 @@
 // With v_mfma_f32_32x32x16 every lane holds one q column of S^T / O^T, so the online-softmax row
 // statistics are per-lane scalars plus one exchange with lane^32.
 //
-// K/V tiles go global -> LDS directly (global_load_lds_dwordx4: no staging registers, the copy of
-// the next tile runs under the current tile's math), two LDS stages per kv group, one barrier per
+// K/V tiles go global -> LDS directly (global_load_lds_dwordx4: no staging registers), two LDS
+// stages per kv group; K and V of a tile are copied separately, each as soon as its half of a stage
+// is free, and their completion is tracked by counting (s_waitcnt vmcnt); two barriers per
 // tile.  A wavefront's 64 lanes land on 1 KB of consecutive LDS, so instead of padding the tile
 // rows (256 B = 16 chunks of 16 B) are XOR-swizzled: row r keeps logical chunk c at position
 // c ^ f(r), f(r) = ((r & 3) << 2) | ((r >> 2) & 3), applied on the global side of the copy.  That
@@ -32,10 +33,11 @@
 //
 // Numerics follow the reference kernel (include/flashomni/attention/prefill.cuh:759-962): base-2
 // softmax p = exp2(s*c - m*c) with c = sm_scale*log2(e), P rounded to the activation type before
-// P.V, masked logits and the initial running max are the finite -5e4 of
-// include/flashomni/math.cuh:32, O = acc * rcp(d) with one round-to-nearest cast, a row with no kv
-// block writes zeros and lse = -5e4, lse = log2(d) + m*c.  (The row sum d is accumulated from the
-// fp32 p values; the reference sums the rounded ones.)
+// P.V, row sum d over the rounded p, O = acc * rcp(d) with one round-to-nearest cast, a row with no
+// kv block writes zeros and lse = -5e4 (the finite "infinity" of include/flashomni/math.cuh:32),
+// lse = log2(d) + m*c.  Two liberties inside the stated tolerances: for 16-bit inputs c is
+// multiplied into Q once per row (one extra rounding of q), and the reference point m is the exact
+// row max of the first tile and afterwards raised only when exceeded by more than 2^8.
 #include <type_traits>
 
 #include "fo_common.h"
