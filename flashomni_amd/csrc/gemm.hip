@@ -283,7 +283,12 @@ __global__ void __launch_bounds__(kThreads) gemm_kernel(const GemmParams p) {
   const int tid = threadIdx.x, lane = tid & 63;
   const int wv = __builtin_amdgcn_readfirstlane(tid >> 6);  // wavefront index, kept scalar
   const int l32 = lane & 31, g = lane >> 5;
-  const int wr = wv >> 2, wc = (wv >> 1) & 1, wh = wv & 1;  // token block, column block, row half
+  // wavefront -> (unit, row half).  Wavefronts w and w+4 share SIMD w%4; SIMD s hosts half 0 of unit s
+  // and half 1 of unit 3-s (unit = 2*token block + column block), so a quad with only one row or
+  // only one column of units still puts one working wavefront on every SIMD.
+  const int wh = wv >> 2;
+  const int unit = wh ? 3 - (wv & 3) : (wv & 3);
+  const int wr = unit >> 1, wc = unit & 1;  // token block, column block
 
   const T* __restrict__ xg = static_cast<const T*>(p.x);
   const T* __restrict__ wg = static_cast<const T*>(p.w);
@@ -426,6 +431,25 @@ __global__ void __launch_bounds__(kThreads) gemm_kernel(const GemmParams p) {
 #pragma unroll
       for (int j = 0; j < kCopiesPerWave; ++j) copy_one(it, entry, j);
     };
+
+    if (!my_valid) {
+      // This wavefront's unit does not exist in this quad (unflagged, or past the matrix edge): it
+      // only does its share of the copies and keeps the barrier and vmcnt sequence of the others,
+      // leaving its SIMD's matrix core to the other wavefront.
+      __builtin_amdgcn_s_waitcnt(0x0f70);
+      if (n_iter > 0) {
+#pragma unroll
+        for (int s = 0; s < kStages - 1; ++s) copy_stage(s);
+        __builtin_amdgcn_s_waitcnt(0x0f70 | (2 * kCopiesPerWave));
+        __builtin_amdgcn_s_barrier();
+        for (int it = 0; it < n_iter; ++it) {
+          __builtin_amdgcn_s_waitcnt(0x0f70 | kCopiesPerWave);
+          __builtin_amdgcn_s_barrier();
+          copy_stage(it + 3);
+        }
+      }
+      continue;
+    }
 
     // ---- accumulators, initialised from bias / cached partial ----
     // acc[nt][mt][i]: n = n0 + nt*32 + (i/4)*8 + g*4 + i%4, m = m0 + mt*32 + l32
@@ -576,7 +600,7 @@ __global__ void __launch_bounds__(kThreads) gemm_kernel(const GemmParams p) {
     }
 
     // ---- epilogue ----
-    if (my_valid) {
+    {
 #pragma unroll
       for (int mt = 0; mt < MT; ++mt) {
         if (m0 + mt * 32 + l32 >= p.m) continue;
