@@ -221,3 +221,39 @@ def test_fp8_attention_needs_scales(dev):
     v = torch.zeros(128, 1, 128, device=dev, dtype=torch.bfloat16)
     with pytest.raises(ValueError, match="q_scale and k_scale"):
         w.run(q8, q8, v, is_full=True)
+
+
+@pytest.mark.parametrize("sign", [1.0, -1.0])
+def test_logits_that_move_the_running_max(dev, sign):
+    """Keys whose logits grow along the sequence (the running reference point has to be raised many
+    times), and the mirrored case where every logit is far below zero (the first tile has to
+    re-centre downwards): both against the fp32 oracle, output and base-2 lse."""
+    import flashomni_amd as fo
+    heads, nq, nk = 2, 256, 2048 + 37
+    m = make_ragged_masks([nq], [nk], heads, 1.0, 0.7, seed=21)
+    g = torch.Generator().manual_seed(21)
+    q = torch.randn(nq, heads, 128, generator=g)
+    k = torch.randn(nk, heads, 128, generator=g) * 0.3
+    # a component along q's mean direction that grows with the key position: the logits drift by
+    # about 24 in the log2 domain over the sequence
+    drift = torch.linspace(1.0, 2.0, nk).view(nk, 1, 1) * sign
+    k = k + drift * torch.ones(1, heads, 128) * 1.5
+    q = q + 1.0
+    v = torch.randn(nk, heads, 128, generator=g)
+    q, k, v = (x.to(torch.bfloat16) for x in (q, k, v))
+    t = lambda a: torch.from_numpy(a).to(dev)
+    w = fo.BatchFlashOmniFAWithRaggedKVWrapper(torch.empty(128 << 20, dtype=torch.uint8, device=dev))
+    w.plan(t(m["qo_indptr"]), t(m["kv_indptr"]), heads, heads, 128, q_data_type=torch.bfloat16)
+    out, lse = w.run(q.to(dev), k.to(dev), v.to(dev), t(m["packed_info"]), t(m["packed_keep"]),
+                     t(m["info_indptr"]), t(m["keep_indptr"]), return_lse=True)
+    exp_lse = torch.full((nq, heads), float("nan"))
+    exp = oracle.sparse_attention(q, k, v, m["packed_info"], m["packed_keep"], m["info_indptr"],
+                                  m["keep_indptr"], m["qo_indptr"], m["kv_indptr"],
+                                  out=torch.zeros(nq, heads, 128, dtype=torch.bfloat16), lse=exp_lse)
+    x = torch.einsum("qhd,khd->hqk", q.float(), k.float()) * (128 ** -0.5) * 1.4426950408889634
+    assert float(x.max() - x.min()) > 16.0          # the case really leaves the lazy window of 2^8
+    assert sign > 0 or float(x.max()) < -8.0        # mirrored case: every logit far below zero
+    assert max_abs(out.cpu(), exp) <= MAX_ABS and rel_l2(out.cpu(), exp) <= REL_L2
+    # |logits| reach ~50 here: the one extra bf16 rounding of q (scale folded into Q) shows as a
+    # relative error of the lse
+    assert float(((lse.cpu() - exp_lse).abs() / (1.0 + exp_lse.abs())).max()) < 2e-3
