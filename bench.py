@@ -326,13 +326,28 @@ def main():
         xb = (torch.rand(n, device=dev) < 0.5)
         pk["n=%d" % n] = entry(time_gpu(lambda: layer.fo.packbits(xb, "little"), K, W), nbytes=n + n // 8)
     kernels["packbits"] = pk
+    # symbol producer (pooled scores -> packed symbols) at the block grids of configs 0, 3 and 4
+    from flashomni_amd.workloads import SHAPES
+    sp = {}
+    for idx in (0, 3, 4):
+        if idx not in configs:
+            continue
+        sh = SHAPES[idx]
+        gen = torch.Generator(device=dev).manual_seed(2000 + idx)
+        pooled = torch.randn(1, sh.heads, sh.n_blocks, sh.n_blocks, generator=gen, device=dev) * 2.0
+        thr = torch.full((sh.heads,), 0.3, device=dev)
+        it, wm = (K, W) if idx == 0 else (max(3, min(K, 20)), 3)
+        ms = time_gpu(lambda: layer.fo.sparse_symbols_from_scores(pooled, 4, 0.2, thr), it, wm)
+        sp[sh.name] = entry(ms, nbytes=pooled.numel() * 4 + pooled.numel() // 8)
+        sp[sh.name]["rows"] = sh.heads * sh.n_blocks
+        del pooled
+    kernels["symbols_from_scores"] = sp
     for name, d in kernels.items():
         log("[bench]", name, json.dumps(d))
 
     big_iters, big_warm = max(3, min(K, 10)), 2
     for idx in (3, 4):
         if idx in configs:
-            from flashomni_amd.workloads import SHAPES
             log("[bench] config %d attention (bf16)" % idx)
             res = bench_big_attention(dev, idx, big_iters, big_warm)
             if idx == 4:

@@ -34,6 +34,7 @@ SIGNATURES = {
                   c_int),
     "fo_quant_fp8_block": ([c_vp, c_int, c_i64, c_i64, c_vp, c_vp, c_vp, c_vp, c_i32, c_i32, c_i32,
                             c_vp], c_int),
+    "fo_symbols_from_scores": ([c_vp, c_int] + [c_i32] * 6 + [c_vp] * 7, c_int),
 }
 
 FO_BF16, FO_F16, FO_FP8_E4M3, FO_F32 = 0, 1, 2, 3

@@ -10,7 +10,7 @@ import sys
 CSRC = os.path.join(os.path.dirname(os.path.abspath(__file__)), "csrc")
 LIB_PATH = os.path.join(CSRC, "libflashomni_hip.so")
 SOURCES = ["fo_error.cpp", "planner.cpp", "packbits.hip", "decode.hip", "sparse_fa.hip", "gemm.hip",
-           "quant_fp8.hip"]
+           "quant_fp8.hip", "symbols.hip"]
 # -packed-fp32-ops off: the compiler must not form packed fp32 VALU instructions on this target
 FLAGS = ["--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-x", "hip",
          "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",

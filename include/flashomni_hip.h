@@ -191,6 +191,31 @@ int fo_quant_fp8_block(const void* x, int dtype, int64_t x_stride_n, int64_t x_s
                        uint8_t* x8, float* scale, const int32_t* blk_tok0, const int32_t* blk_len,
                        int32_t n_blk, int32_t num_heads, int32_t head_dim, void* stream);
 
+/* ---------------------------------------------------------------------------------------------
+ * Symbol producer: pooled attention scores -> packed sparse_info / sparse_kv_info.
+ * replaces: the torch sort / cumsum / searchsorted steps of benchmark/test_attn_score.py:96-105,
+ *           :117-127, the Triton fill kernels :5-91, and the transposition + segment_packbits that
+ *           turn the maps into run() arguments (benchmark/utils.py:83-84,
+ *           benchmark/test_flashomni_attention.py:254-257).
+ * scores [batch, H, NQ, NK] contiguous (FO_F32, FO_BF16 or FO_F16), finite.
+ * q symbols: the scores of the first n_text_q q blocks towards key blocks n_text_kv.. are summed
+ *   over heads and those q blocks and soft-maxed; the key blocks of lowest score whose cumulative
+ *   probability stays <= q_threshold[request] are cached: q block n_text_q + j gets symbol 0 for
+ *   every head.  kv symbols: each row (head, q block >= n_text_q) is soft-maxed over all NK key
+ *   blocks and those of lowest score whose cumulative probability stays <= kv_threshold[head] get
+ *   symbol 0; text q rows keep every key block.  Equal scores are taken in index order; cumulative
+ *   probabilities are exact sums of probabilities rounded to 2^-30.
+ * Outputs (device): sparse_info batch*ceil(NQ*H/8) bytes, sparse_kv_info batch*ceil(NQ*H*NK/8)
+ *   bytes, little-endian bits at q_block*H+head resp. (q_block*H+head)*NK+kv_block inside each
+ *   request's byte-aligned segment; the two indptr arrays (int32 [batch+1], byte offsets) are
+ *   written too.  Every output byte is written: no clearing needed.  NQ, NK <= 4096.
+ * ------------------------------------------------------------------------------------------- */
+int fo_symbols_from_scores(const void* scores, int dtype, int32_t batch, int32_t num_heads,
+                           int32_t n_q_blocks, int32_t n_kv_blocks, int32_t n_text_q,
+                           int32_t n_text_kv, const float* q_threshold, const float* kv_threshold,
+                           uint8_t* sparse_info, int32_t* sparse_info_indptr,
+                           uint8_t* sparse_kv_info, int32_t* sparse_kv_info_indptr, void* stream);
+
 #ifdef __cplusplus
 }
 #endif

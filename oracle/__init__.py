@@ -20,6 +20,12 @@ Pinning status (what each restatement is checked against, see tests/):
   quantizer and up-casts fp8 to fp16 before its MMA): parity unpinned against
   the reference; pinned only by closed forms (scale = absmax/448, torch's own
   float8_e4m3fn cast) and by the fp32 dense masked reference at rel-L2 3e-2.
+* symbol producer (producer.py) -- the reference holds no vectors for it (its script
+  prints); pinned by hand-worked rows with exactly representable probabilities, by a
+  remove-the-smallest brute force, by the script's own consistency checks
+  (benchmark/test_attn_score.py:155-160) and by mass invariants.  The order of equal
+  scores and rows whose cumulative mass meets the threshold within fp32 rounding are
+  left open by the reference (torch.sort / torch.cumsum): parity unpinned there.
 """
 from .symbols import (  # noqa: F401
     get_bit, packbits, segment_packbits, sparse_info_indptr_bits,
@@ -29,3 +35,4 @@ from .planner import prefill_plan  # noqa: F401
 from .attention import sparse_attention  # noqa: F401
 from .gemm import gemm_q, gemm_o  # noqa: F401
 from .quant import quant_fp8_block, dequant_fp8_block  # noqa: F401
+from . import producer  # noqa: F401
