@@ -11,9 +11,9 @@
 // steps of bisection over the key space find the largest key bound whose mass below fits.  Equal
 // scores at the cut are taken in index order, as a stable sort would.
 //
-// One pass over the scores (4 B per entry read, 1/8 B written); eight consecutive rows of a request
-// make one workgroup, so every workgroup owns whole output bytes and nothing needs atomics or a
-// cleared output.
+// One launch, one pass over the scores (4 B per entry read, 1/8 B written); eight consecutive rows
+// of a request make one workgroup, so every workgroup owns whole output bytes and nothing needs
+// atomics or a cleared output.
 #include "fo_common.h"
 
 #include <hip/hip_bf16.h>
@@ -151,21 +151,73 @@ __device__ __forceinline__ uint8_t gather8(uint64_t flags) {
 }
 
 // ---- q symbols: one workgroup per request --------------------------------------------------------
+// The H * n_text_q contributing rows are split into `parts` interleaved subsets; a wavefront sums
+// one subset over one 64-column chunk (coalesced 256 B loads, eight in flight), and the partial sums
+// are added in subset order, so the result does not depend on which wavefront did what.
+// LDS (carved from the launch's dynamic block): partial sums [parts][width], sums [width], keep
+// flags [n_q + 8].
+struct QJobLayout {
+  int width, parts;
+  size_t bytes;
+};
+
+__host__ __device__ inline QJobLayout q_job_layout(int n_q, int n_k, int text_kv) {
+  QJobLayout l;
+  l.width = ((n_k - text_kv + 63) / 64) * 64;
+  if (l.width < 64) l.width = 64;
+  int parts = (16384 - n_q - 16) / (4 * l.width) - 1;
+  l.parts = parts < 1 ? 1 : (parts > 16 ? 16 : parts);
+  l.bytes = static_cast<size_t>(4) * l.width * (l.parts + 1) + n_q + 16;
+  return l;
+}
+
 template <typename T, int E>
-__global__ void __launch_bounds__(kThreads) q_symbols_kernel(ProducerArgs a) {
-  __shared__ float s_sum[E * 64];
-  __shared__ __align__(8) uint8_t s_keep[kMaxBlocks + 8];
-  const int b = blockIdx.x, tid = threadIdx.x, lane = tid & 63;
+__device__ __forceinline__ void q_symbols_job(const ProducerArgs& a, int b, uint8_t* lds) {
+  const QJobLayout lay = q_job_layout(a.n_q, a.n_k, a.text_kv);
+  const int width = lay.width, parts = lay.parts;
+  float* s_part = reinterpret_cast<float*>(lds);
+  float* s_sum = s_part + parts * width;
+  uint8_t* s_keep = reinterpret_cast<uint8_t*>(s_sum + width);
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int n_img = a.n_k - a.text_kv;
+  const int chunks = (n_img + 63) >> 6;
+  const int n_rows = a.heads * a.text_q;
   const T* base = static_cast<const T*>(a.scores) + static_cast<int64_t>(b) * a.heads * a.n_q * a.n_k;
-  for (int j = tid; j < n_img; j += kThreads) {
-    float acc = 0.f;
-    for (int h = 0; h < a.heads; ++h)
-      for (int q = 0; q < a.text_q; ++q)
-        acc += to_f32(base[(static_cast<int64_t>(h) * a.n_q + q) * a.n_k + a.text_kv + j]);
-    s_sum[j] = acc;
+  constexpr int kFlight = 8;
+  for (int item = wave; item < chunks * parts; item += kWaves) {
+    const int c = item / parts, part = item - c * parts;
+    const int j = c * 64 + lane;
+    float acc[kFlight];
+#pragma unroll
+    for (int u = 0; u < kFlight; ++u) acc[u] = 0.f;
+    if (j < n_img) {
+      const T* col = base + a.text_kv + j;
+      int r = part;
+      for (; r + (kFlight - 1) * parts < n_rows; r += kFlight * parts) {
+#pragma unroll
+        for (int u = 0; u < kFlight; ++u) {
+          const int row = r + u * parts;             // row = head * n_text_q + q
+          const int h = row / a.text_q, q = row - h * a.text_q;
+          acc[u] += to_f32(col[(static_cast<int64_t>(h) * a.n_q + q) * a.n_k]);
+        }
+      }
+      for (; r < n_rows; r += parts) {
+        const int h = r / a.text_q, q = r - h * a.text_q;
+        acc[0] += to_f32(col[(static_cast<int64_t>(h) * a.n_q + q) * a.n_k]);
+      }
+    }
+    float total = 0.f;
+#pragma unroll
+    for (int u = 0; u < kFlight; ++u) total += acc[u];
+    s_part[part * width + j] = total;
   }
   for (int q = tid; q < a.n_q + 8; q += kThreads) s_keep[q] = q < a.n_q ? 1 : 0;
+  __syncthreads();
+  for (int j = tid; j < n_img; j += kThreads) {
+    float acc = 0.f;
+    for (int part = 0; part < parts; ++part) acc += s_part[part * width + j];
+    s_sum[j] = acc;
+  }
   __syncthreads();
   if (tid < 64 && n_img > 0) {
     float score[E];
@@ -196,12 +248,19 @@ __global__ void __launch_bounds__(kThreads) q_symbols_kernel(ProducerArgs a) {
   }
 }
 
-// ---- kv symbols: one workgroup per eight consecutive (q_block, head) rows of a request ------------
+// ---- one launch: workgroups [0, batch) make the q symbols of a request each (they start first and
+// run beside the rest); every other workgroup makes the kv symbols of eight consecutive
+// (q_block, head) rows of a request ------------------------------------------------------------------
 template <typename T, int E>
-__global__ void __launch_bounds__(kThreads) kv_symbols_kernel(ProducerArgs a, int groups_per_request) {
-  extern __shared__ __align__(8) uint8_t s_flags[];  // kRowsPerGroup * n_k (+8) keep flags
-  const int b = blockIdx.x / groups_per_request;
-  const int g = blockIdx.x - b * groups_per_request;
+__global__ void __launch_bounds__(kThreads) symbols_kernel(ProducerArgs a, int groups_per_request) {
+  extern __shared__ __align__(16) uint8_t s_flags[];  // kv job: kRowsPerGroup * n_k (+8) keep flags
+  if (static_cast<int>(blockIdx.x) < a.batch) {
+    q_symbols_job<T, E>(a, blockIdx.x, s_flags);
+    return;
+  }
+  const int block = blockIdx.x - a.batch;
+  const int b = block / groups_per_request;
+  const int g = block - b * groups_per_request;
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int rows = a.n_q * a.heads;
   const int row0 = g * kRowsPerGroup;
@@ -247,14 +306,12 @@ constexpr int kSlots[] = {1, 2, 4, 6, 8, 10, 12, 16, 24, 32, 48, 64};
 
 template <typename T, int E>
 int launch_both(const ProducerArgs& a, hipStream_t stream) {
-  const int n_img = a.n_k - a.text_kv;
-  // the q kernel holds n_img <= n_k entries: the same slot count serves both
-  (void)n_img;
-  q_symbols_kernel<T, E><<<a.batch, kThreads, 0, stream>>>(a);
-  FO_CHECK_LAUNCH();
+  // the q job holds n_k - n_text_kv <= n_k entries: the same slot count serves both jobs
   const int groups = fo::ceil_div(static_cast<int64_t>(a.n_q) * a.heads, kRowsPerGroup);
-  const size_t lds = static_cast<size_t>(kRowsPerGroup) * a.n_k + 8;
-  kv_symbols_kernel<T, E><<<a.batch * groups, kThreads, lds, stream>>>(a, groups);
+  size_t lds = static_cast<size_t>(kRowsPerGroup) * a.n_k + 8;
+  const size_t lds_q = q_job_layout(a.n_q, a.n_k, a.text_kv).bytes;
+  if (lds_q > lds) lds = lds_q;
+  symbols_kernel<T, E><<<a.batch * (groups + 1), kThreads, lds, stream>>>(a, groups);
   FO_CHECK_LAUNCH();
   return FO_OK;
 }
