@@ -332,7 +332,10 @@ class BatchFlashOmniFAWithRaggedKVWrapper:
         else:
             tensors = [None] * 4
             key = "full"
-        if key == self._decode_key:
+        # a stream capture must record the decode: replays see new symbol contents without
+        # passing through this method again
+        capturing = torch.cuda.is_current_stream_capturing()
+        if key == self._decode_key and not capturing:
             return wl
         _lib.check(_lib.lib().fo_decode_sparse(
             _lib.ptr(tensors[0]), _lib.ptr(tensors[1]), _lib.ptr(tensors[2]), _lib.ptr(tensors[3]),
@@ -342,7 +345,7 @@ class BatchFlashOmniFAWithRaggedKVWrapper:
             _lib.ptr(wl.kv_idx), _lib.ptr(wl.counts), _lib.ptr(wl.order), _lib.ptr(wl.sched),
             _lib.ptr(wl.scratch), _lib.current_stream(self.device)))
         # the memo holds the tensors alive so a recycled address cannot alias the key
-        self._decode_key = key
+        self._decode_key = None if capturing else key
         self._decode_refs = (tensors, sparse_info, sparse_kv_info, sparse_info_indptr,
                              sparse_kv_info_indptr)
         return wl

@@ -1,0 +1,80 @@
+"""run() and the GEMMs under HIP graph capture (the reference declares run() capturable,
+flashomni/attention.py:140-141): a captured layer pass must give, on every replay, what the same
+calls give eagerly on the inputs of that moment, including symbols rewritten in place between
+replays."""
+import numpy as np
+import pytest
+import torch
+
+from helpers import make_ragged_masks
+
+pytestmark = pytest.mark.gpu
+
+
+def test_captured_layer_pass_replays(dev):
+    import flashomni_amd as fo
+    H, hidden = 4, 512
+    ql = [640, 300]
+    nnz = sum(ql)
+    g = torch.Generator().manual_seed(5)
+    rnd = lambda *s: torch.randn(*s, generator=g)
+    x = rnd(1, nnz, hidden).to(torch.bfloat16).to(dev)
+    wq = (rnd(hidden, hidden) * 0.05).to(torch.bfloat16).to(dev)
+    bq = (rnd(hidden) * 0.05).to(torch.bfloat16).to(dev)
+    wo = (rnd(hidden, hidden) * 0.05).to(torch.bfloat16).to(dev)
+    k = rnd(nnz, H, 128).to(torch.bfloat16).to(dev)
+    v = rnd(nnz, H, 128).to(torch.bfloat16).to(dev)
+
+    def symbols(seed):
+        m = make_ragged_masks(ql, ql, H, 0.7, 0.5, seed=seed)
+        return [torch.from_numpy(m[n]) for n in ("packed_info", "packed_keep", "info_indptr", "keep_indptr")]
+
+    info, kv_info, info_ip, kv_ip = [t.to(dev) for t in symbols(1)]
+    # the GEMMs see the two requests as one batch entry of nnz rows: their symbols index the
+    # 128-row blocks of that entry, so give them a single-request packing of the same size
+    n_blk = sum(-(-l // 128) for l in ql)
+    gemm_bits = torch.from_numpy((np.random.default_rng(2).random(n_blk * H) < 0.7))
+    gemm_info = fo.packbits(gemm_bits.to(dev), "little")
+    gemm_ip = torch.tensor([0, gemm_info.numel()], dtype=torch.int32, device=dev)
+
+    ws = torch.empty(32 << 20, dtype=torch.uint8, device=dev)
+    w = fo.BatchFlashOmniFAWithRaggedKVWrapper(ws)
+    indptr = torch.tensor([0, ql[0], nnz], dtype=torch.int32)
+    w.plan(indptr, indptr, H, H, 128, q_data_type=torch.bfloat16)
+
+    q_buf = torch.zeros(1, nnz, hidden, dtype=torch.bfloat16, device=dev)
+    o_buf = torch.zeros(nnz, H, 128, dtype=torch.bfloat16, device=dev)
+    y_buf = torch.zeros(1, nnz, hidden, dtype=torch.bfloat16, device=dev)
+
+    def layer_pass(q_out, o_out):
+        fo.flashomni_gemm(x, wq, H, gemm_info, gemm_ip, 0, bq, out=q_out)
+        w.run(q_out.view(nnz, H, 128), k, v, info, kv_info, info_ip, kv_ip, out=o_out)
+        return fo.flashomni_gemm_reduction(o_out.view(1, nnz, hidden), wo, H, gemm_info, gemm_ip, 0,
+                                           bias=None, is_for_cache=False)
+
+    # warm up on a side stream, then capture
+    s = torch.cuda.Stream(device=dev)
+    s.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(s):
+        layer_pass(q_buf, o_buf)
+    torch.cuda.current_stream().wait_stream(s)
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        y_graph = layer_pass(q_buf, o_buf)
+    for replay in range(4):
+        # new activations and, from the second replay on, new attention symbols, written in place
+        x.copy_(rnd(1, nnz, hidden).to(torch.bfloat16))
+        if replay >= 1:
+            for dst, src in zip((info, kv_info), symbols(10 + replay)[:2]):
+                dst.copy_(src)
+        q_buf.zero_(); o_buf.zero_()
+        graph.replay()
+        torch.cuda.synchronize()
+        got = (q_buf.clone(), o_buf.clone(), y_graph.clone())
+        # the same pass eagerly, into fresh buffers, with program work and a sync in between
+        q_ref = torch.zeros_like(q_buf); o_ref = torch.zeros_like(o_buf)
+        y_ref = layer_pass(q_ref, o_ref)
+        torch.cuda.synchronize()
+        for name, a, b in zip(("gemm_q", "attention", "gemm_o"), got, (q_ref, o_ref, y_ref)):
+            assert torch.equal(a, b), "replay %d: %s differs from the eager pass" % (replay, name)
