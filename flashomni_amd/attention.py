@@ -52,7 +52,7 @@ class DecodedWorkList:
     """Device buffers holding one decoded work list (canonical order).
 
     ``row_req/row_qb/row_head[n_rows]``, ``kv_row_ptr[n_rows+1]``, ``kv_idx[nnz]``, all int32;
-    ``counts = [n_rows, nnz, 0, 0]``; ``order[n_rows]`` / ``sched[32]`` are the execution order
+    ``counts = [n_rows, nnz, 0, 0]``; ``order[n_rows]`` / ``sched[256]`` are the execution order
     and queue words the attention kernel schedules from.  The sizes live on the device;
     ``sizes()`` copies them back (one synchronisation) for tests and reports."""
 
@@ -66,7 +66,7 @@ class DecodedWorkList:
         self.kv_idx = torch.empty(max(max_nnz, 1), dtype=torch.int32, device=device)
         self.counts = torch.zeros(4, dtype=torch.int32, device=device)
         self.order = torch.empty(n, dtype=torch.int32, device=device)
-        self.sched = torch.zeros(32, dtype=torch.int32, device=device)
+        self.sched = torch.zeros(256, dtype=torch.int32, device=device)
         self.scratch = torch.empty(2 * n + 8192, dtype=torch.int32, device=device)
 
     def sizes(self) -> Tuple[int, int]:
@@ -110,6 +110,7 @@ class BatchFlashOmniFAWithRaggedKVWrapper:
         _check_kv_layout(kv_layout)
         self._kv_layout = kv_layout
         self._float_workspace_buffer = float_workspace_buffer
+        self._share_rows = True   # let short work lists cut rows into parts (needs the float workspace)
         self.device = float_workspace_buffer.device
         if self.device.type != "cuda":
             raise ValueError("float_workspace_buffer must live on the GPU; there is no CPU path")
@@ -305,6 +306,17 @@ class BatchFlashOmniFAWithRaggedKVWrapper:
 
     begin_forward = plan
 
+    def _float_ws_bytes(self) -> int:
+        ws = self._float_workspace_buffer
+        return ws.numel() * ws.element_size()
+
+    def _split_ws_ok(self) -> bool:
+        """Whether the float workspace can hold the partial results of rows whose kv list is shared
+        between workgroups (the reference uses it for its split-kv partials, scheduler.cuh:322-328)."""
+        ws = self._float_workspace_buffer
+        return (self._share_rows and ws.data_ptr() % 16 == 0
+                and self._float_ws_bytes() >= _lib.lib().fo_sparse_fa_split_workspace_bytes())
+
     # ------------------------------------------------------------------------------------------
     def decode(self, sparse_info, sparse_kv_info, sparse_info_indptr, sparse_kv_info_indptr,
                is_full: bool = False) -> DecodedWorkList:
@@ -343,7 +355,7 @@ class BatchFlashOmniFAWithRaggedKVWrapper:
             self._n_q_blk, self._num_qo_heads, self._sparse_block_size_for_kv, int(bool(is_full)),
             _lib.ptr(wl.row_req), _lib.ptr(wl.row_qb), _lib.ptr(wl.row_head), _lib.ptr(wl.kv_row_ptr),
             _lib.ptr(wl.kv_idx), _lib.ptr(wl.counts), _lib.ptr(wl.order), _lib.ptr(wl.sched),
-            _lib.ptr(wl.scratch), _lib.current_stream(self.device)))
+            _lib.ptr(wl.scratch), int(self._split_ws_ok()), _lib.current_stream(self.device)))
         # the memo holds the tensors alive so a recycled address cannot alias the key
         self._decode_key = None if capturing else key
         self._decode_refs = (tensors, sparse_info, sparse_kv_info, sparse_info_indptr,
@@ -430,7 +442,9 @@ class BatchFlashOmniFAWithRaggedKVWrapper:
             _lib.ptr(wl.row_qb),
             _lib.ptr(wl.row_head), _lib.ptr(wl.kv_row_ptr), _lib.ptr(wl.kv_idx), _lib.ptr(wl.order),
             _lib.ptr(wl.sched), self._max_rows, q.size(1), q.size(2), self._sparse_block_size_for_q,
-            self._sparse_block_size_for_kv, float(sm_scale), _lib.current_stream(self.device)))
+            self._sparse_block_size_for_kv, float(sm_scale),
+            _lib.ptr(self._float_workspace_buffer) if self._split_ws_ok() else None,
+            self._float_ws_bytes(), _lib.current_stream(self.device)))
         return (out, lse) if return_lse else out
 
     run_return_lse = functools.partialmethod(run, return_lse=True)

@@ -13,7 +13,8 @@
 // to the longest row of the launch), which evens out the workgroups' finishing times when there are
 // only a few rows per CU.  sched[0..8] delimit the 8 per-XCD queues inside `order`, sched[16..23]
 // are the queue cursors, sched[24] a completion counter (all cleared here) and sched[25] the
-// longest row's kv count.  The order inside a length class is not deterministic (atomic cursors);
+// longest row's kv count.  sched[32..55] describe, per queue, the rows at its end that the attention
+// kernel shares between workgroups, and sched[64..191] are their arrival counters (cleared here).  The order inside a length class is not deterministic (atomic cursors);
 // results do not depend on it.
 // Integer work, bounded by HBM traffic and launch latency; bit-exact by construction.
 //
@@ -30,6 +31,9 @@ constexpr int kScanThreads = 1024;
 constexpr int kMaxHeads = 1024;
 constexpr int kXcds = 8;
 constexpr int kHistSlots = 8192;  // (head, length class) counters of the order layout
+// split rows (see the attention kernel): words of `sched` and limits
+constexpr int kSchedSplitStart = 32, kSchedSplitParts = 40, kSchedSplitSlot = 48, kSchedArrived = 64;
+constexpr int kMaxSplitSlots = 128, kMaxSplitParts = 4, kSplitMaxRounds = 1;
 
 // number of length classes for num_heads heads (32 up to 256 heads)
 __host__ __device__ __forceinline__ int len_classes(int32_t num_heads) {
@@ -116,7 +120,7 @@ __global__ void __launch_bounds__(kCountThreads) decode_count_kernel(
 __global__ void __launch_bounds__(kScanThreads) decode_scan_kernel(
     int64_t n_cand, int32_t num_heads, int32_t* __restrict__ act, int32_t* __restrict__ cnt,
     int32_t* __restrict__ kv_row_ptr, int32_t* __restrict__ counts,
-    int32_t* __restrict__ head_cursor, int32_t* __restrict__ sched) {
+    int32_t* __restrict__ head_cursor, int32_t* __restrict__ sched, int32_t cus_per_xcd) {
   __shared__ int32_t s_rows[kScanThreads];
   __shared__ int32_t s_kv[kScanThreads];
   __shared__ int32_t s_hist[kHistSlots];
@@ -210,6 +214,7 @@ __global__ void __launch_bounds__(kScanThreads) decode_scan_kernel(
       if (j % n_classes == 0 && slot / n_classes == qx) sched[qx] = pos;  // first head of queue qx
       pos += s_hist[slot];
     }
+    __syncthreads();  // every queue's first position is in sched
     if (tid == 0) {
       int32_t total = 0;
       for (int w = 0; w < kScanThreads / 64; ++w) total += s_rows[w];
@@ -218,7 +223,29 @@ __global__ void __launch_bounds__(kScanThreads) decode_scan_kernel(
       sched[kXcds] = total;
       for (int i = kXcds + 1; i < 32; ++i) sched[i] = 0;
       sched[25] = max_n;
+      // A queue's rows go to the cus_per_xcd workgroups of its XCD.  When there are so few rows that
+      // at most half of the workgroups would get one, every row is cut into 2..4 parts (consecutive
+      // ranges of its kv blocks) so that they all get work.  (With one or more full rounds of rows
+      // the parts' extra prologues and the merge cost what the better balance gains: measured.)
+      int32_t slot = 0;
+      for (int x = 0; x < kXcds; ++x) {
+        const int32_t len = sched[x + 1] - sched[x];
+        int32_t rest = 0, parts = 1;
+        if (cus_per_xcd > 1) {
+          const int32_t rounds = len / cus_per_xcd, rem = len - rounds * cus_per_xcd;
+          if (rounds < kSplitMaxRounds && rem > 0 && 2 * rem <= cus_per_xcd &&
+              slot + rem <= kMaxSplitSlots) {
+            rest = rem;
+            parts = min(kMaxSplitParts, cus_per_xcd / rem);
+          }
+        }
+        sched[kSchedSplitStart + x] = sched[x + 1] - rest;
+        sched[kSchedSplitParts + x] = parts;
+        sched[kSchedSplitSlot + x] = slot;
+        slot += rest;
+      }
     }
+    for (int i = tid; i < kMaxSplitSlots; i += kScanThreads) sched[kSchedArrived + i] = 0;
   }
 }
 
@@ -285,7 +312,8 @@ extern "C" int fo_decode_sparse(const uint8_t* sparse_info, const uint8_t* spars
                                 int32_t num_heads, int32_t block_kv, int is_full,
                                 int32_t* row_req, int32_t* row_qb, int32_t* row_head,
                                 int32_t* kv_row_ptr, int32_t* kv_idx, int32_t* counts,
-                                int32_t* order, int32_t* sched, int32_t* scratch, void* stream) {
+                                int32_t* order, int32_t* sched, int32_t* scratch, int split_rows,
+                                void* stream) {
   FO_REQUIRE(n_blk >= 0 && num_heads > 0 && num_heads <= kMaxHeads && block_kv > 0,
              "decode: bad sizes");
   FO_REQUIRE(counts && kv_row_ptr && order && sched, "decode: null output");
@@ -309,8 +337,9 @@ extern "C" int fo_decode_sparse(const uint8_t* sparse_info, const uint8_t* spars
         kv_indptr, n_cand, num_heads, block_kv, is_full, act, cnt);
     FO_CHECK_LAUNCH();
   }
+  const int32_t cus_per_xcd = split_rows ? fo_num_cu() / kXcds : 0;
   decode_scan_kernel<<<1, kScanThreads, 0, s>>>(n_cand, num_heads, act, cnt, kv_row_ptr, counts,
-                                                head_cursor, sched);
+                                                head_cursor, sched, cus_per_xcd);
   FO_CHECK_LAUNCH();
   if (n_cand > 0) {
     const int per_wg = kCountThreads / kWave;

@@ -99,6 +99,7 @@ struct FaParams {
   const int32_t* kv_idx;
   const int32_t* order;
   int32_t* sched;
+  float* split_ws;  // partial results of rows whose kv list is split over workgroups (or null)
   int32_t num_heads;
   int32_t n_q_blocks, n_kv_blocks;  // row lengths of q_scale / k_scale
   float sm_scale_log2;
@@ -175,16 +176,50 @@ __device__ __forceinline__ float max_across_halves(float x) {
   return fmaxf(__builtin_bit_cast(float, r[0]), __builtin_bit_cast(float, r[1]));
 }
 
-// Pop the next row for this workgroup: own XCD queue first, then the neighbours'.
-__device__ __forceinline__ int pop_row(const FaParams& p, int xcd) {
+// words of `sched` (written by the decoder): [0..8] queue bounds inside `order`, [16..23] queue
+// cursors, [24] completion counter, [32..39] first split position of each queue, [40..47] number
+// of parts its split rows are cut into, [48..55] first split slot of the queue, [64..191] arrival
+// counters of the split slots
+constexpr int kSchedSplitStart = 32, kSchedSplitParts = 40, kSchedSplitSlot = 48, kSchedArrived = 64;
+constexpr int kMaxSplitSlots = 128, kMaxSplitParts = 4;
+constexpr int kSplitPartFloats = 128 * 128 + 2 * 256;  // O (fp32) + (max, sum) per lane of kv group 0
+
+// Partial results cross workgroups (and XCDs, whose L2s are not coherent with each other) through
+// device-scope accesses that bypass the local L2 instead of through fences, which would write back
+// and invalidate a whole L2 that is busy serving K and V.
+__device__ __forceinline__ void store_pair_device(float* p, float a, float b) {
+  const uint64_t v = static_cast<uint64_t>(__float_as_uint(a)) | (static_cast<uint64_t>(__float_as_uint(b)) << 32);
+  __hip_atomic_store(reinterpret_cast<uint64_t*>(p), v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+__device__ __forceinline__ void load_pair_device(const float* p, float& a, float& b) {
+  const uint64_t v = __hip_atomic_load(reinterpret_cast<const uint64_t*>(p), __ATOMIC_RELAXED,
+                                       __HIP_MEMORY_SCOPE_AGENT);
+  a = __uint_as_float(static_cast<uint32_t>(v));
+  b = __uint_as_float(static_cast<uint32_t>(v >> 32));
+}
+
+struct Item {
+  int row;   // position in the canonical row list, -1 = queues are empty
+  int meta;  // part | parts << 4 | slot << 8
+};
+
+// Pop the next work item for this workgroup: own XCD queue first, then the neighbours'.  The last
+// rows of a queue may be cut into `parts` items that cover consecutive ranges of the row's kv
+// blocks: position ss + v of the queue then stands for part v % parts of row order[ss + v / parts].
+__device__ __forceinline__ Item pop_row(const FaParams& p, int xcd) {
   for (int a = 0; a < kXcds; ++a) {
     const int x = (xcd + a) & (kXcds - 1);
     const int beg = p.sched[x], end = p.sched[x + 1];
-    if (beg + __atomic_load_n(&p.sched[16 + x], __ATOMIC_RELAXED) >= end) continue;
-    const int i = atomicAdd(&p.sched[16 + x], 1);
-    if (beg + i < end) return p.order[beg + i];
+    const int ss = p.sched[kSchedSplitStart + x], parts = p.sched[kSchedSplitParts + x];
+    const int vend = end + (end - ss) * (parts - 1);
+    if (beg + __atomic_load_n(&p.sched[16 + x], __ATOMIC_RELAXED) >= vend) continue;
+    const int pos = beg + atomicAdd(&p.sched[16 + x], 1);
+    if (pos >= vend) continue;
+    if (pos < ss) return Item{p.order[pos], 1 << 4};
+    const int v = pos - ss, r = v / parts;
+    return Item{p.order[ss + r], (v - r * parts) | parts << 4 | (p.sched[kSchedSplitSlot + x] + r) << 8};
   }
-  return -1;
+  return Item{-1, 0};
 }
 
 // T: element type of V, P and O (and of Q, K unless kFp8).  kFp8: Q and K are e4m3fn bytes with one
@@ -200,7 +235,8 @@ __global__ void __launch_bounds__(kThreads) sparse_fa_kernel(const FaParams p) {
   using TQK = typename std::conditional<kFp8, uint8_t, T>::type;
   constexpr int kStageBytes = G::kStageBytes, kKBytes = G::kKBytes, kGroupBytes = G::kGroupBytes;
   extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
-  __shared__ int s_next_row[2];  // this row / the next one
+  __shared__ Item s_next_row[2];  // this item / the next one
+  __shared__ int s_arrived;
   __shared__ int32_t s_blk[kMaxRowBlocks];  // kv block list of the current row
 
   const int tid = threadIdx.x, lane = tid & 63;
@@ -247,8 +283,11 @@ __global__ void __launch_bounds__(kThreads) sparse_fa_kernel(const FaParams p) {
   if (tid == 0) s_next_row[0] = pop_row(p, blockIdx.x & (kXcds - 1));
   for (int row_it = 0;; ++row_it) {
     __syncthreads();  // s_next_row is published; everyone is done with the previous row's LDS data
-    const int w = __builtin_amdgcn_readfirstlane(s_next_row[row_it & 1]);  // uniform: scalar loads below
+    const int w = __builtin_amdgcn_readfirstlane(s_next_row[row_it & 1].row);  // uniform: scalar loads below
     if (w < 0) break;
+    const int meta = __builtin_amdgcn_readfirstlane(s_next_row[row_it & 1].meta);
+    const int part = meta & 15, split_slot = meta >> 8;
+    int parts = (meta >> 4) & 15;
 
     const int req = p.row_req[w], qb = p.row_qb[w], head = p.row_head[w];
     const int q_begin = p.qo_indptr[req] + qb * kBlockQ;
@@ -256,7 +295,21 @@ __global__ void __launch_bounds__(kThreads) sparse_fa_kernel(const FaParams p) {
     const int kv_begin = p.kv_indptr[req];
     const int kv_len = p.kv_indptr[req + 1] - kv_begin;
     // (a row longer than the LDS list is cut; the host side refuses such requests at plan time)
-    const int ptr0 = p.kv_row_ptr[w], nb = min(p.kv_row_ptr[w + 1] - ptr0, kMaxRowBlocks);
+    int ptr0 = p.kv_row_ptr[w], nb = min(p.kv_row_ptr[w + 1] - ptr0, kMaxRowBlocks);
+    if (parts > 1) {
+      if (nb < 2 * parts || p.split_ws == nullptr) {
+        // too short to share (or nowhere to put partial results): part 0 does the whole row
+        if (part > 0) {
+          if (tid == kGroupThreads) s_next_row[(row_it + 1) & 1] = pop_row(p, blockIdx.x & (kXcds - 1));
+          continue;
+        }
+        parts = 1;
+      } else {
+        const int b0 = nb * part / parts, b1 = nb * (part + 1) / parts;
+        ptr0 += b0;
+        nb = b1 - b0;
+      }
+    }
 
     const int my_row = qs * 32 + l32;  // q row of this lane inside the block
     const bool row_ok = my_row < q_rows;
@@ -692,6 +745,7 @@ __global__ void __launch_bounds__(kThreads) sparse_fa_kernel(const FaParams p) {
     }
     __syncthreads();
     if (tid == kGroupThreads) s_next_row[(row_it + 1) & 1] = pop_row(p, blockIdx.x & (kXcds - 1));
+    float m_all = 0.f, d_all = 0.f;  // kv group 0: row maximum and row sum over both groups
     if (kg == 0) {
       const float m1 = md[(qs * 64 + lane) * 2 + 0], d1 = md[(qs * 64 + lane) * 2 + 1];
       const float m = fmaxf(m_run, m1);
@@ -699,23 +753,101 @@ __global__ void __launch_bounds__(kThreads) sparse_fa_kernel(const FaParams p) {
       const float a1 = __builtin_amdgcn_exp2f(m1 - m);
       const float d_lane = d_part * a0 + d1 * a1;
       const float d_tot = d_lane + __shfl_xor(d_lane, 32, 64);
-      const float inv = __builtin_amdgcn_rcpf(d_tot);
-      const float w0 = a0 * inv, w1 = a1 * inv;
-      if (row_ok) {
-        T* dst = op + q_tok * p.o_sn + static_cast<int64_t>(head) * p.o_sh;
+      if (parts == 1) {
+        const float inv = __builtin_amdgcn_rcpf(d_tot);
+        const float w0 = a0 * inv, w1 = a1 * inv;
+        if (row_ok) {
+          T* dst = op + q_tok * p.o_sn + static_cast<int64_t>(head) * p.o_sh;
+#pragma unroll
+          for (int dt = 0; dt < 4; ++dt)
+#pragma unroll
+            for (int i4 = 0; i4 < 4; ++i4) {
+              const f32x4 t4 = mo[(qs * 16 + dt * 4 + i4) * 64 + lane];
+              x4 out;
+#pragma unroll
+              for (int j = 0; j < 4; ++j)
+                out[j] = static_cast<T>(o_acc[dt][i4 * 4 + j] * w0 + t4[j] * w1);
+              *reinterpret_cast<x4*>(dst + dt * 32 + i4 * 8 + g * 4) = out;
+            }
+          if (p.lse && g == 0)
+            p.lse[q_tok * p.num_heads + head] = __builtin_amdgcn_logf(d_tot) + m;
+        }
+      } else {
+        // one part of a split row: fold kv group 1 in without normalising and publish the partial
+        // result (same lane layout as the LDS merge area)
+        float* part_ws = p.split_ws +
+                         static_cast<int64_t>(split_slot * kMaxSplitParts + part) * kSplitPartFloats;
 #pragma unroll
         for (int dt = 0; dt < 4; ++dt)
 #pragma unroll
           for (int i4 = 0; i4 < 4; ++i4) {
             const f32x4 t4 = mo[(qs * 16 + dt * 4 + i4) * 64 + lane];
-            x4 out;
+            float u[4];
 #pragma unroll
-            for (int j = 0; j < 4; ++j)
-              out[j] = static_cast<T>(o_acc[dt][i4 * 4 + j] * w0 + t4[j] * w1);
-            *reinterpret_cast<x4*>(dst + dt * 32 + i4 * 8 + g * 4) = out;
+            for (int j = 0; j < 4; ++j) u[j] = o_acc[dt][i4 * 4 + j] * a0 + t4[j] * a1;
+            // two planes of 8-byte pairs: each store instruction covers 512 contiguous bytes
+            float* dst = part_ws + ((qs * 16 + dt * 4 + i4) * 2 * 64 + lane) * 2;
+            store_pair_device(dst, u[0], u[1]);
+            store_pair_device(dst + 128, u[2], u[3]);
           }
-        if (p.lse && g == 0)
-          p.lse[q_tok * p.num_heads + head] = __builtin_amdgcn_logf(d_tot) + m;
+        store_pair_device(part_ws + 128 * 128 + (qs * 64 + lane) * 2, m, d_tot);
+      }
+    }
+    if (parts > 1) {
+      // whoever arrives last at the row's slot combines the parts and writes the row
+      __builtin_amdgcn_s_waitcnt(0x0f70);  // vmcnt(0): this lane's partial results have left
+      __syncthreads();
+      if (tid == 0) s_arrived = atomicAdd(&p.sched[kSchedArrived + split_slot], 1);
+      __syncthreads();
+      if (s_arrived == parts - 1) {
+        if (kg == 0) {
+          // every part is read back, this workgroup's own included, and added in part order: the
+          // row does not depend on which part arrived last
+          const float* slot_ws = p.split_ws + static_cast<int64_t>(split_slot * kMaxSplitParts) * kSplitPartFloats;
+          float m_p[kMaxSplitParts], d_p[kMaxSplitParts];
+          m_all = kNegInf;
+          for (int i = 0; i < parts; ++i) {
+            load_pair_device(slot_ws + i * kSplitPartFloats + 128 * 128 + (qs * 64 + lane) * 2, m_p[i], d_p[i]);
+            m_all = fmaxf(m_all, m_p[i]);
+          }
+          d_all = 0.f;
+#pragma unroll
+          for (int dt = 0; dt < 4; ++dt)
+#pragma unroll
+            for (int e = 0; e < 16; ++e) o_acc[dt][e] = 0.f;
+          for (int i = 0; i < parts; ++i) {
+            const float* part_ws = slot_ws + i * kSplitPartFloats;
+            const float a = __builtin_amdgcn_exp2f(m_p[i] - m_all);
+            d_all += d_p[i] * a;
+#pragma unroll
+            for (int dt = 0; dt < 4; ++dt)
+#pragma unroll
+              for (int i4 = 0; i4 < 4; ++i4) {
+                const float* src = part_ws + ((qs * 16 + dt * 4 + i4) * 2 * 64 + lane) * 2;
+                float u[4];
+                load_pair_device(src, u[0], u[1]);
+                load_pair_device(src + 128, u[2], u[3]);
+#pragma unroll
+                for (int j = 0; j < 4; ++j) o_acc[dt][i4 * 4 + j] += u[j] * a;
+              }
+          }
+          const float inv = __builtin_amdgcn_rcpf(d_all);
+          if (row_ok) {
+            T* dst = op + q_tok * p.o_sn + static_cast<int64_t>(head) * p.o_sh;
+#pragma unroll
+            for (int dt = 0; dt < 4; ++dt)
+#pragma unroll
+              for (int i4 = 0; i4 < 4; ++i4) {
+                x4 out;
+#pragma unroll
+                for (int j = 0; j < 4; ++j) out[j] = static_cast<T>(o_acc[dt][i4 * 4 + j] * inv);
+                *reinterpret_cast<x4*>(dst + dt * 32 + i4 * 8 + g * 4) = out;
+              }
+            if (p.lse && g == 0)
+              p.lse[q_tok * p.num_heads + head] = __builtin_amdgcn_logf(d_all) + m_all;
+          }
+        }
+        if (tid == 0) p.sched[kSchedArrived + split_slot] = 0;  // re-armed for the next launch
       }
     }
   }
@@ -743,13 +875,18 @@ int launch(const FaParams& p, int64_t max_rows, hipStream_t stream) {
   int num_cu = fo_num_cu();
   if (num_cu <= 0) return fo::fail(FO_ERR_HIP, "sparse_fa: no device");
   int64_t grid = num_cu;  // one persistent workgroup per CU (LDS bound)
-  if (grid > max_rows) grid = max_rows;
+  const int64_t max_items = p.split_ws ? max_rows * kMaxSplitParts : max_rows;
+  if (grid > max_items) grid = max_items;
   sparse_fa_kernel<T, kFp8><<<static_cast<unsigned>(grid), kThreads, kSmemBytes, stream>>>(p);
   FO_CHECK_LAUNCH();
   return FO_OK;
 }
 
 }  // namespace
+
+extern "C" int64_t fo_sparse_fa_split_workspace_bytes(void) {
+  return static_cast<int64_t>(kMaxSplitSlots) * kMaxSplitParts * kSplitPartFloats * sizeof(float);
+}
 
 extern "C" int fo_sparse_fa_run(const void* q, const void* k, const void* v, void* o, float* lse,
                                 int dtype, const float* q_scale, const float* k_scale,
@@ -763,7 +900,8 @@ extern "C" int fo_sparse_fa_run(const void* q, const void* k, const void* v, voi
                                 const int32_t* kv_row_ptr, const int32_t* kv_idx,
                                 const int32_t* order, int32_t* sched, int64_t max_rows,
                                 int32_t num_heads, int32_t head_dim, int32_t block_q,
-                                int32_t block_kv, float sm_scale, void* stream) {
+                                int32_t block_kv, float sm_scale, void* split_workspace,
+                                int64_t split_workspace_bytes, void* stream) {
   FO_REQUIRE(head_dim == kHeadDim, "sparse_fa: head_dim %d is not supported (only 128)", head_dim);
   FO_REQUIRE(block_q == kBlockQ && block_kv == kBlockKV,
              "sparse_fa: sparse block sizes (%d, %d) are not supported (only 128, 128)", block_q,
@@ -798,6 +936,13 @@ extern "C" int fo_sparse_fa_run(const void* q, const void* k, const void* v, voi
   p.q_blk_base = q_blk_base; p.kv_blk_base = kv_blk_base;
   p.row_req = row_req; p.row_qb = row_qb; p.row_head = row_head;
   p.kv_row_ptr = kv_row_ptr; p.kv_idx = kv_idx; p.order = order; p.sched = sched;
+  // without room for partial results every split row is computed whole by its first part
+  p.split_ws = nullptr;
+  if (split_workspace != nullptr && split_workspace_bytes >= fo_sparse_fa_split_workspace_bytes()) {
+    FO_REQUIRE((reinterpret_cast<uintptr_t>(split_workspace) & 15) == 0,
+               "sparse_fa: split_workspace must be 16-byte aligned");
+    p.split_ws = static_cast<float*>(split_workspace);
+  }
   p.num_heads = num_heads; p.n_q_blocks = n_q_blocks; p.n_kv_blocks = n_kv_blocks;
   p.sm_scale_log2 = sm_scale * 1.44269504088896340736f;
   hipStream_t s = static_cast<hipStream_t>(stream);

@@ -90,9 +90,16 @@ int fo_prefill_plan(void* float_ws, size_t float_ws_bytes, void* int_ws_dev, voi
  *   order [n_rows]   execution order for the attention kernel: canonical row positions grouped by
  *                    head, heads dealt round-robin to 8 queues (head % 8, one queue per XCD);
  *                    inside one head longer rows first (up to 32 length classes), otherwise unspecified
- *   sched [32]       sched[0..8] = queue boundaries inside `order`, sched[16..23] = queue cursors
+ *   sched [256]      sched[0..8] = queue boundaries inside `order`, sched[16..23] = queue cursors
  *                    and sched[24] = completion counter, both cleared to 0; sched[25] = kv count of
- *                    the longest row
+ *                    the longest row; sched[32..39] = first split position of each queue,
+ *                    sched[40..47] = parts per split row, sched[48..55] = first split slot,
+ *                    sched[64..191] = arrival counters of the split slots (cleared to 0)
+ * split_rows != 0: when a queue holds so few rows that at most half of the workgroups of its XCD
+ * would get one, the attention kernel cuts each row into 2..4 parts (consecutive ranges of its kv
+ * blocks) that different workgroups compute
+ * (the counterpart of the reference's split-kv plan, scheduler.cuh:35-64, decided on the device
+ * from the decoded row count).  The canonical lists do not change.
  * is_full != 0 ignores the symbol tensors (which may be NULL) and lists everything
  * (csrc/batch_sparseFA.cu:123-128).
  * `scratch` needs 2*n_blk*H + 8192 int32.
@@ -109,7 +116,7 @@ int fo_decode_sparse(const uint8_t* sparse_info, const uint8_t* sparse_kv_info,
                      int32_t n_blk, int32_t num_heads, int32_t block_kv, int is_full,
                      int32_t* row_req, int32_t* row_qb, int32_t* row_head, int32_t* kv_row_ptr,
                      int32_t* kv_idx, int32_t* counts, int32_t* order, int32_t* sched,
-                     int32_t* scratch, void* stream);
+                     int32_t* scratch, int split_rows, void* stream);
 
 /* ---------------------------------------------------------------------------------------------
  * Ragged block-sparse FlashAttention prefill over a decoded work list.
@@ -128,8 +135,14 @@ int fo_decode_sparse(const uint8_t* sparse_info, const uint8_t* sparse_kv_info,
  * Rows are taken from the queues described by `order` / `sched` (see fo_decode_sparse); the
  * kernel leaves the queue cursors rewound, so one decoded list can be run any number of times,
  * but two launches sharing one `sched` must not overlap in time.
+ * split_workspace: device memory of fo_sparse_fa_split_workspace_bytes() bytes, 16-byte aligned,
+ * for the unnormalised partial results (fp32 O, row maximum, row sum) of split rows: the part that
+ * arrives last combines them (replaces the reference's float workspace + merge kernels,
+ * scheduler.cuh:322-328, cascade.cuh:346-437).  NULL or too small: every split row is computed
+ * whole by the workgroup that pops its first part.  Launches sharing it must not overlap in time.
  * Supported: D = 128, block_q = 128, block_kv = 128.  max_rows bounds the number of rows.
  * ------------------------------------------------------------------------------------------- */
+int64_t fo_sparse_fa_split_workspace_bytes(void);
 int fo_sparse_fa_run(const void* q, const void* k, const void* v, void* o, float* lse, int dtype,
                      const float* q_scale, const float* k_scale, int64_t q_stride_n,
                      int64_t q_stride_h, int64_t k_stride_n, int64_t k_stride_h,
@@ -139,7 +152,8 @@ int fo_sparse_fa_run(const void* q, const void* k, const void* v, void* o, float
                      int32_t n_kv_blocks, const int32_t* row_req, const int32_t* row_qb, const int32_t* row_head,
                      const int32_t* kv_row_ptr, const int32_t* kv_idx, const int32_t* order,
                      int32_t* sched, int64_t max_rows, int32_t num_heads, int32_t head_dim,
-                     int32_t block_q, int32_t block_kv, float sm_scale, void* stream);
+                     int32_t block_q, int32_t block_kv, float sm_scale, void* split_workspace,
+                     int64_t split_workspace_bytes, void* stream);
 
 /* ---------------------------------------------------------------------------------------------
  * GEMM-Q: y[b, tile] = x[b] . w^T + bias for every (128-row, 128-column) tile whose symbol bit

@@ -257,3 +257,76 @@ def test_logits_that_move_the_running_max(dev, sign):
     # |logits| reach ~50 here: the one extra bf16 rounding of q (scale folded into Q) shows as a
     # relative error of the lse
     assert float(((lse.cpu() - exp_lse).abs() / (1.0 + exp_lse.abs())).max()) < 2e-3
+
+
+def _split_case(dev, ql, kl, heads, seed, share, dtype=torch.bfloat16, pk=0.6):
+    """Run one launch (twice, to see the arrival counters re-armed) with or without rows shared
+    between workgroups; returns (out, lse, sched words, expectations)."""
+    import flashomni_amd as fo
+    m = make_ragged_masks(ql, kl, heads, 1.0, pk, seed=seed)
+    g = torch.Generator().manual_seed(seed)
+    nq, nk = int(m["qo_indptr"][-1]), int(m["kv_indptr"][-1])
+    q = torch.randn(nq, heads, 128, generator=g).to(dtype)
+    k = torch.randn(nk, heads, 128, generator=g).to(dtype)
+    v = torch.randn(nk, heads, 128, generator=g).to(dtype)
+    t = lambda a: torch.from_numpy(a).to(dev)
+    w = fo.BatchFlashOmniFAWithRaggedKVWrapper(torch.empty(64 << 20, dtype=torch.uint8, device=dev))
+    w._share_rows = share
+    w.plan(t(m["qo_indptr"]), t(m["kv_indptr"]), heads, heads, 128, q_data_type=dtype)
+    args = (t(m["packed_info"]), t(m["packed_keep"]), t(m["info_indptr"]), t(m["keep_indptr"]))
+    qd, kd, vd = q.to(dev), k.to(dev), v.to(dev)
+    out1, lse1 = w.run(qd, kd, vd, *args, return_lse=True)
+    out1, lse1 = out1.clone(), lse1.clone()
+    out2, lse2 = w.run(qd, kd, vd, *args, return_lse=True)
+    assert torch.equal(out1, out2) and torch.equal(lse1, lse2), "second launch over the same list differs"
+    sched = w._worklist.sched.cpu().numpy()
+    exp_lse = torch.full((nq, heads), float("nan"))
+    exp = oracle.sparse_attention(q, k, v, m["packed_info"], m["packed_keep"], m["info_indptr"],
+                                  m["keep_indptr"], m["qo_indptr"], m["kv_indptr"],
+                                  out=torch.zeros(nq, heads, 128, dtype=dtype), lse=exp_lse)
+    return out2.cpu(), lse2.cpu(), sched, exp, exp_lse
+
+
+@pytest.mark.parametrize("case", [
+    ([1024], [4096], 2, 4),          # 8 rows per queue: cut in four
+    ([1536], [2048 + 77], 8, 2),     # 12 rows per queue: cut in two, ragged kv tail in the last part
+    ([128 * 9], [128 * 9], 1, 3),    # 9 rows in one queue: cut in three, rows of 9 * 0.6 blocks: some too short
+])
+def test_rows_shared_between_workgroups(dev, case):
+    """Few rows per XCD: the decoder marks them for sharing and the parts' partial results are
+    combined by the last arrival.  Checked against the oracle, against the same launch with sharing
+    switched off (every row computed whole), and for the counters being left re-armed."""
+    ql, kl, heads, parts = case
+    out, lse, sched, exp, exp_lse = _split_case(dev, ql, kl, heads, seed=31, share=True)
+    n_queues = min(heads, 8)
+    assert (sched[40:40 + n_queues] == parts).all(), sched[32:56]
+    assert (sched[64:192] == 0).all() and (sched[16:25] == 0).all()
+    assert max_abs(out, exp) <= MAX_ABS and rel_l2(out, exp) <= REL_L2
+    assert torch.allclose(lse, exp_lse, atol=2e-3, rtol=1e-3)
+    whole, lse_w, sched_w, _, _ = _split_case(dev, ql, kl, heads, seed=31, share=False)
+    assert (sched_w[40:48] == 1).all()          # the decoder was told not to mark anything
+    assert max_abs(out, whole) <= 8e-3          # same math, the parts' sums are combined in another order
+    assert torch.allclose(lse, lse_w, atol=1e-3, rtol=1e-4)
+
+
+def test_shared_rows_fp8(dev):
+    import flashomni_amd as fo
+    ql, kl, heads = [1024], [2048], 2
+    m = make_ragged_masks(ql, kl, heads, 1.0, 0.7, seed=33)
+    g = torch.Generator().manual_seed(33)
+    q = torch.randn(ql[0], heads, 128, generator=g).to(torch.bfloat16)
+    k = torch.randn(kl[0], heads, 128, generator=g).to(torch.bfloat16)
+    v = torch.randn(kl[0], heads, 128, generator=g).to(torch.bfloat16)
+    t = lambda a: torch.from_numpy(a).to(dev)
+    args = (t(m["packed_info"]), t(m["packed_keep"]), t(m["info_indptr"]), t(m["keep_indptr"]))
+    outs = []
+    for share in (True, False):
+        w = fo.BatchFlashOmniFAWithRaggedKVWrapper(torch.empty(64 << 20, dtype=torch.uint8, device=dev))
+        w._share_rows = share
+        w.plan(t(m["qo_indptr"]), t(m["kv_indptr"]), heads, heads, 128, q_data_type=torch.float8_e4m3fn)
+        q8, qs = fo.quant_fp8_block(q.to(dev), t(m["qo_indptr"]))
+        k8, ks = fo.quant_fp8_block(k.to(dev), t(m["kv_indptr"]))
+        outs.append(w.run(q8, k8, v.to(dev), *args, q_scale=qs, k_scale=ks).cpu())
+        parts = w._worklist.sched.cpu().numpy()[40:42]
+        assert (parts == (4 if share else 1)).all()
+    assert max_abs(outs[0], outs[1]) <= 8e-3
