@@ -64,20 +64,27 @@ constexpr int kTileKV = 64;
 constexpr int kRowBytes = 256;   // one K or V row of 128 16-bit elements, unpadded (swizzled)
 constexpr int kRowBytes8 = 128;  // one fp8 K row
 constexpr int kVBytes = kTileKV * kRowBytes;
+constexpr int kMergeOBytes = 4 * 16 * 64 * 16;
+constexpr int kOutTileOff = kMergeOBytes + 4 * 64 * 8;  // behind the merge area
+constexpr int kOutRowBytes = 256 + 16;                  // one output row of 128 16-bit elements, padded
+constexpr int kOutTileBytes = 128 * kOutRowBytes;
 // LDS geometry of one kv group: two stages of (K tile, V tile); K is 16-bit or fp8
 template <bool kFp8>
 struct Geom {
   static constexpr int kKBytes = kTileKV * (kFp8 ? kRowBytes8 : kRowBytes);
   static constexpr int kStageBytes = kKBytes + kVBytes;
   static constexpr int kGroupBytes = 2 * kStageBytes;
-  static constexpr int kSmemBytes = 2 * kGroupBytes;
+  static constexpr int kTilesBytes = 2 * kGroupBytes;
+  // the epilogue reuses the tile buffers: kv group 1's partial O (64 KB fp32) + its (max, sum)
+  // pairs (2 KB), then the finished row as a padded tile for the coalesced store
+  static constexpr int kSmemBytes = kTilesBytes > kOutTileOff + kOutTileBytes ? kTilesBytes
+                                                                              : kOutTileOff + kOutTileBytes;
 };
 constexpr int kXcds = 8;
 constexpr int kMaxRowBlocks = 4096;  // kv blocks of one row held in LDS (512 Ki tokens per request)
 constexpr float kLazyLog2 = 8.0f;  // the running max is raised only past a 2^8 overshoot
 // merge area (reuses the tile buffers): O^T of kv group 1, then its (m, d)
-constexpr int kMergeOBytes = 4 * 16 * 64 * 16;
-static_assert(kMergeOBytes + 4 * 64 * 8 <= Geom<true>::kSmemBytes, "merge area must fit");
+static_assert(kOutTileOff + kOutTileBytes <= Geom<true>::kSmemBytes, "merge area must fit");
 
 struct FaParams {
   const void* q;
@@ -206,19 +213,26 @@ struct Item {
 // Pop the next work item for this workgroup: own XCD queue first, then the neighbours'.  The last
 // rows of a queue may be cut into `parts` items that cover consecutive ranges of the row's kv
 // blocks: position ss + v of the queue then stands for part v % parts of row order[ss + v / parts].
-__device__ __forceinline__ Item pop_row(const FaParams& p, int xcd) {
-  for (int a = 0; a < kXcds; ++a) {
+// `first` is the first queue that may still hold items: a queue found empty stays empty for the rest
+// of the launch, so it is not asked again.  `q` is the launch's copy of the queue words
+// (q[x] = bounds, q[9 + x] = split start, q[17 + x] = parts, q[25 + x] = first slot): the pop itself
+// is one atomic and one load.
+__device__ __forceinline__ Item pop_row(const FaParams& p, int xcd, const int* q, int* first) {
+  for (int a = *first; a < kXcds; ++a) {
     const int x = (xcd + a) & (kXcds - 1);
-    const int beg = p.sched[x], end = p.sched[x + 1];
-    const int ss = p.sched[kSchedSplitStart + x], parts = p.sched[kSchedSplitParts + x];
+    const int beg = q[x], end = q[x + 1], ss = q[9 + x], parts = q[17 + x];
     const int vend = end + (end - ss) * (parts - 1);
-    if (beg + __atomic_load_n(&p.sched[16 + x], __ATOMIC_RELAXED) >= vend) continue;
-    const int pos = beg + atomicAdd(&p.sched[16 + x], 1);
-    if (pos >= vend) continue;
-    if (pos < ss) return Item{p.order[pos], 1 << 4};
-    const int v = pos - ss, r = v / parts;
-    return Item{p.order[ss + r], (v - r * parts) | parts << 4 | (p.sched[kSchedSplitSlot + x] + r) << 8};
+    if (beg < vend) {
+      const int pos = beg + atomicAdd(&p.sched[16 + x], 1);
+      if (pos < vend) {
+        *first = a;
+        if (pos < ss) return Item{p.order[pos], 1 << 4};
+        const int v = pos - ss, r = v / parts;
+        return Item{p.order[ss + r], (v - r * parts) | parts << 4 | (q[25 + x] + r) << 8};
+      }
+    }
   }
+  *first = kXcds;
   return Item{-1, 0};
 }
 
@@ -237,6 +251,7 @@ __global__ void __launch_bounds__(kThreads) sparse_fa_kernel(const FaParams p) {
   extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
   __shared__ Item s_next_row[2];  // this item / the next one
   __shared__ int s_arrived;
+  __shared__ int s_queue[40];  // the queue words of `sched`, read once
   __shared__ int32_t s_blk[kMaxRowBlocks];  // kv block list of the current row
 
   const int tid = threadIdx.x, lane = tid & 63;
@@ -280,7 +295,12 @@ __global__ void __launch_bounds__(kThreads) sparse_fa_kernel(const FaParams p) {
 
   // The next row is popped by kv group 1 while kv group 0 combines and stores the current one
   // (group 1 has nothing else to do then), so the queue atomics are off the critical path.
-  if (tid == 0) s_next_row[0] = pop_row(p, blockIdx.x & (kXcds - 1));
+  if (tid < 9) s_queue[tid] = p.sched[tid];
+  if (tid >= 64 && tid < 64 + 24)
+    s_queue[9 + tid - 64] = p.sched[kSchedSplitStart + tid - 64];  // split start, parts, first slot
+  __syncthreads();
+  int first_queue = 0;  // kept by the popping lane (the first pop is lane 0's, the others lane 256's)
+  if (tid == 0) s_next_row[0] = pop_row(p, blockIdx.x & (kXcds - 1), s_queue, &first_queue);
   for (int row_it = 0;; ++row_it) {
     __syncthreads();  // s_next_row is published; everyone is done with the previous row's LDS data
     const int w = __builtin_amdgcn_readfirstlane(s_next_row[row_it & 1].row);  // uniform: scalar loads below
@@ -300,7 +320,7 @@ __global__ void __launch_bounds__(kThreads) sparse_fa_kernel(const FaParams p) {
       if (nb < 2 * parts || p.split_ws == nullptr) {
         // too short to share (or nowhere to put partial results): part 0 does the whole row
         if (part > 0) {
-          if (tid == kGroupThreads) s_next_row[(row_it + 1) & 1] = pop_row(p, blockIdx.x & (kXcds - 1));
+          if (tid == kGroupThreads) s_next_row[(row_it + 1) & 1] = pop_row(p, blockIdx.x & (kXcds - 1), s_queue, &first_queue);
           continue;
         }
         parts = 1;
@@ -324,7 +344,7 @@ __global__ void __launch_bounds__(kThreads) sparse_fa_kernel(const FaParams p) {
         for (int j = 0; j < 8; ++j) reinterpret_cast<u32x4*>(dst)[j] = z;
         if (p.lse && g == 0) p.lse[q_tok * p.num_heads + head] = kNegInf;
       }
-      if (tid == kGroupThreads) s_next_row[(row_it + 1) & 1] = pop_row(p, blockIdx.x & (kXcds - 1));
+      if (tid == kGroupThreads) s_next_row[(row_it + 1) & 1] = pop_row(p, blockIdx.x & (kXcds - 1), s_queue, &first_queue);
       continue;
     }
 
@@ -744,8 +764,13 @@ __global__ void __launch_bounds__(kThreads) sparse_fa_kernel(const FaParams p) {
       md[(qs * 64 + lane) * 2 + 1] = d_part;
     }
     __syncthreads();
-    if (tid == kGroupThreads) s_next_row[(row_it + 1) & 1] = pop_row(p, blockIdx.x & (kXcds - 1));
+    if (tid == kGroupThreads) s_next_row[(row_it + 1) & 1] = pop_row(p, blockIdx.x & (kXcds - 1), s_queue, &first_queue);
     float m_all = 0.f, d_all = 0.f;  // kv group 0: row maximum and row sum over both groups
+    // A lane owns one q row and runs of four d: stored from here, a row would leave as 32 scattered
+    // 8-byte pieces per instruction (measured: ~12 k cycles per row).  The finished row goes through
+    // a padded LDS tile instead and leaves in 16-byte pieces, 16 consecutive lanes per 256-byte row.
+    uint8_t* const out_row = smem + kOutTileOff + my_row * kOutRowBytes;
+    bool store_row = parts == 1;
     if (kg == 0) {
       const float m1 = md[(qs * 64 + lane) * 2 + 0], d1 = md[(qs * 64 + lane) * 2 + 1];
       const float m = fmaxf(m_run, m1);
@@ -756,22 +781,24 @@ __global__ void __launch_bounds__(kThreads) sparse_fa_kernel(const FaParams p) {
       if (parts == 1) {
         const float inv = __builtin_amdgcn_rcpf(d_tot);
         const float w0 = a0 * inv, w1 = a1 * inv;
-        if (row_ok) {
-          T* dst = op + q_tok * p.o_sn + static_cast<int64_t>(head) * p.o_sh;
+        // all sixteen reads of the partner's partial first (the registers of the tile operands are
+        // free here), so their latencies overlap
+        f32x4 t4[16];
 #pragma unroll
-          for (int dt = 0; dt < 4; ++dt)
+        for (int e = 0; e < 16; ++e) t4[e] = mo[(qs * 16 + e) * 64 + lane];
+        __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
-            for (int i4 = 0; i4 < 4; ++i4) {
-              const f32x4 t4 = mo[(qs * 16 + dt * 4 + i4) * 64 + lane];
-              x4 out;
+        for (int dt = 0; dt < 4; ++dt)
 #pragma unroll
-              for (int j = 0; j < 4; ++j)
-                out[j] = static_cast<T>(o_acc[dt][i4 * 4 + j] * w0 + t4[j] * w1);
-              *reinterpret_cast<x4*>(dst + dt * 32 + i4 * 8 + g * 4) = out;
-            }
-          if (p.lse && g == 0)
-            p.lse[q_tok * p.num_heads + head] = __builtin_amdgcn_logf(d_tot) + m;
-        }
+          for (int i4 = 0; i4 < 4; ++i4) {
+            x4 out;
+#pragma unroll
+            for (int j = 0; j < 4; ++j)
+              out[j] = static_cast<T>(o_acc[dt][i4 * 4 + j] * w0 + t4[dt * 4 + i4][j] * w1);
+            *reinterpret_cast<x4*>(out_row + (dt * 32 + i4 * 8 + g * 4) * sizeof(T)) = out;
+          }
+        if (row_ok && p.lse && g == 0)
+          p.lse[q_tok * p.num_heads + head] = __builtin_amdgcn_logf(d_tot) + m;
       } else {
         // one part of a split row: fold kv group 1 in without normalising and publish the partial
         // result (same lane layout as the LDS merge area)
@@ -832,23 +859,38 @@ __global__ void __launch_bounds__(kThreads) sparse_fa_kernel(const FaParams p) {
               }
           }
           const float inv = __builtin_amdgcn_rcpf(d_all);
-          if (row_ok) {
-            T* dst = op + q_tok * p.o_sn + static_cast<int64_t>(head) * p.o_sh;
 #pragma unroll
-            for (int dt = 0; dt < 4; ++dt)
+          for (int dt = 0; dt < 4; ++dt)
 #pragma unroll
-              for (int i4 = 0; i4 < 4; ++i4) {
-                x4 out;
+            for (int i4 = 0; i4 < 4; ++i4) {
+              x4 out;
 #pragma unroll
-                for (int j = 0; j < 4; ++j) out[j] = static_cast<T>(o_acc[dt][i4 * 4 + j] * inv);
-                *reinterpret_cast<x4*>(dst + dt * 32 + i4 * 8 + g * 4) = out;
-              }
-            if (p.lse && g == 0)
-              p.lse[q_tok * p.num_heads + head] = __builtin_amdgcn_logf(d_all) + m_all;
-          }
+              for (int j = 0; j < 4; ++j) out[j] = static_cast<T>(o_acc[dt][i4 * 4 + j] * inv);
+              *reinterpret_cast<x4*>(out_row + (dt * 32 + i4 * 8 + g * 4) * sizeof(T)) = out;
+            }
+          if (row_ok && p.lse && g == 0)
+            p.lse[q_tok * p.num_heads + head] = __builtin_amdgcn_logf(d_all) + m_all;
         }
         if (tid == 0) p.sched[kSchedArrived + split_slot] = 0;  // re-armed for the next launch
+        store_row = true;
       }
+    }
+    if (store_row) {
+      __syncthreads();  // the row is complete in the LDS tile
+      T* dst = op + static_cast<int64_t>(q_begin) * p.o_sn + static_cast<int64_t>(head) * p.o_sh;
+      // (the lane index is made opaque here: otherwise the per-lane address terms are computed once
+      // per kernel, spilled, and every reload waits for the store before it)
+      int ln = lane;
+      asm volatile("" : "+v"(ln));
+      const int r0 = wv * 16 + (ln >> 4), chunk = ln & 15;
+      u32x4 v[4];
+#pragma unroll
+      for (int i = 0; i < 4; ++i)
+        v[i] = *reinterpret_cast<const u32x4*>(smem + kOutTileOff + (r0 + i * 4) * kOutRowBytes + chunk * 16);
+      T* d0 = dst + static_cast<int64_t>(r0) * p.o_sn + chunk * 8;
+#pragma unroll
+      for (int i = 0; i < 4; ++i)
+        if (r0 + i * 4 < q_rows) *reinterpret_cast<u32x4*>(d0 + i * 4 * p.o_sn) = v[i];
     }
   }
 
