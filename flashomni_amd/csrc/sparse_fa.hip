@@ -249,7 +249,12 @@ __global__ void __launch_bounds__(kThreads) sparse_fa_kernel(const FaParams p) {
   using TQK = typename std::conditional<kFp8, uint8_t, T>::type;
   constexpr int kStageBytes = G::kStageBytes, kKBytes = G::kKBytes, kGroupBytes = G::kGroupBytes;
   extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
-  __shared__ Item s_next_row[2];  // this item / the next one
+  // this item / the next one, with everything the row's prologue needs: fetched by the popping lane
+  // while the rest of the workgroup finishes the current row
+  struct RowInfo {
+    int row, part, parts, slot, req, qb, head, q_begin, q_rows, kv_begin, kv_len, ptr0, nb;
+  };
+  __shared__ RowInfo s_next_row[2];
   __shared__ int s_arrived;
   __shared__ int s_queue[40];  // the queue words of `sched`, read once
   __shared__ int32_t s_blk[kMaxRowBlocks];  // kv block list of the current row
@@ -300,36 +305,57 @@ __global__ void __launch_bounds__(kThreads) sparse_fa_kernel(const FaParams p) {
     s_queue[9 + tid - 64] = p.sched[kSchedSplitStart + tid - 64];  // split start, parts, first slot
   __syncthreads();
   int first_queue = 0;  // kept by the popping lane (the first pop is lane 0's, the others lane 256's)
-  if (tid == 0) s_next_row[0] = pop_row(p, blockIdx.x & (kXcds - 1), s_queue, &first_queue);
+  // one lane: pop the next item and gather its row's metadata (two rounds of loads) into LDS
+  auto fetch_next = [&](int slot_idx) {
+    RowInfo ri;
+    for (;;) {
+      const Item item = pop_row(p, blockIdx.x & (kXcds - 1), s_queue, &first_queue);
+      ri.row = item.row;
+      if (item.row < 0) break;
+      const int w = item.row;
+      ri.part = item.meta & 15;
+      ri.parts = (item.meta >> 4) & 15;
+      ri.slot = item.meta >> 8;
+      ri.req = p.row_req[w];
+      ri.qb = p.row_qb[w];
+      ri.head = p.row_head[w];
+      ri.ptr0 = p.kv_row_ptr[w];
+      // (a row longer than the LDS list is cut; the host side refuses such requests at plan time)
+      ri.nb = min(p.kv_row_ptr[w + 1] - ri.ptr0, kMaxRowBlocks);
+      ri.q_begin = p.qo_indptr[ri.req] + ri.qb * kBlockQ;
+      ri.q_rows = min(kBlockQ, p.qo_indptr[ri.req + 1] - ri.q_begin);
+      ri.kv_begin = p.kv_indptr[ri.req];
+      ri.kv_len = p.kv_indptr[ri.req + 1] - ri.kv_begin;
+      if (ri.parts > 1) {
+        if (ri.nb < 2 * ri.parts || p.split_ws == nullptr) {
+          // too short to share (or nowhere to put partial results): part 0 does the whole row
+          if (ri.part > 0) continue;
+          ri.parts = 1;
+        } else {
+          const int b0 = ri.nb * ri.part / ri.parts, b1 = ri.nb * (ri.part + 1) / ri.parts;
+          ri.ptr0 += b0;
+          ri.nb = b1 - b0;
+        }
+      }
+      break;
+    }
+    s_next_row[slot_idx] = ri;
+  };
+  if (tid == 0) fetch_next(0);
   for (int row_it = 0;; ++row_it) {
     __syncthreads();  // s_next_row is published; everyone is done with the previous row's LDS data
-    const int w = __builtin_amdgcn_readfirstlane(s_next_row[row_it & 1].row);  // uniform: scalar loads below
+    const RowInfo& ri = s_next_row[row_it & 1];
+    const int w = __builtin_amdgcn_readfirstlane(ri.row);  // uniform values, kept in scalar registers
     if (w < 0) break;
-    const int meta = __builtin_amdgcn_readfirstlane(s_next_row[row_it & 1].meta);
-    const int part = meta & 15, split_slot = meta >> 8;
-    int parts = (meta >> 4) & 15;
-
-    const int req = p.row_req[w], qb = p.row_qb[w], head = p.row_head[w];
-    const int q_begin = p.qo_indptr[req] + qb * kBlockQ;
-    const int q_rows = min(kBlockQ, p.qo_indptr[req + 1] - q_begin);
-    const int kv_begin = p.kv_indptr[req];
-    const int kv_len = p.kv_indptr[req + 1] - kv_begin;
-    // (a row longer than the LDS list is cut; the host side refuses such requests at plan time)
-    int ptr0 = p.kv_row_ptr[w], nb = min(p.kv_row_ptr[w + 1] - ptr0, kMaxRowBlocks);
-    if (parts > 1) {
-      if (nb < 2 * parts || p.split_ws == nullptr) {
-        // too short to share (or nowhere to put partial results): part 0 does the whole row
-        if (part > 0) {
-          if (tid == kGroupThreads) s_next_row[(row_it + 1) & 1] = pop_row(p, blockIdx.x & (kXcds - 1), s_queue, &first_queue);
-          continue;
-        }
-        parts = 1;
-      } else {
-        const int b0 = nb * part / parts, b1 = nb * (part + 1) / parts;
-        ptr0 += b0;
-        nb = b1 - b0;
-      }
-    }
+    const int part = __builtin_amdgcn_readfirstlane(ri.part), parts = __builtin_amdgcn_readfirstlane(ri.parts);
+    const int split_slot = __builtin_amdgcn_readfirstlane(ri.slot);
+    const int req = __builtin_amdgcn_readfirstlane(ri.req), qb = __builtin_amdgcn_readfirstlane(ri.qb);
+    const int head = __builtin_amdgcn_readfirstlane(ri.head);
+    const int q_begin = __builtin_amdgcn_readfirstlane(ri.q_begin);
+    const int q_rows = __builtin_amdgcn_readfirstlane(ri.q_rows);
+    const int kv_begin = __builtin_amdgcn_readfirstlane(ri.kv_begin);
+    const int kv_len = __builtin_amdgcn_readfirstlane(ri.kv_len);
+    const int ptr0 = __builtin_amdgcn_readfirstlane(ri.ptr0), nb = __builtin_amdgcn_readfirstlane(ri.nb);
 
     const int my_row = qs * 32 + l32;  // q row of this lane inside the block
     const bool row_ok = my_row < q_rows;
@@ -344,44 +370,41 @@ __global__ void __launch_bounds__(kThreads) sparse_fa_kernel(const FaParams p) {
         for (int j = 0; j < 8; ++j) reinterpret_cast<u32x4*>(dst)[j] = z;
         if (p.lse && g == 0) p.lse[q_tok * p.num_heads + head] = kNegInf;
       }
-      if (tid == kGroupThreads) s_next_row[(row_it + 1) & 1] = pop_row(p, blockIdx.x & (kXcds - 1), s_queue, &first_queue);
+      if (tid == kGroupThreads) fetch_next((row_it + 1) & 1);
       continue;
     }
 
-    // Q operand, requested first so that its latency overlaps the staging below: lane holds q row
-    // l32 of its q sub-tile, d = ks*16 + g*8 .. +7 (fp8: d = slab*64 + g*32 .. +31 for the two
-    // 64-wide slabs)
+    // Q operand.  A lane needs q row l32 of its sub-tile, 16 bytes out of every 32 (fp8: 32 of 64):
+    // fetched straight from memory that is 64 scattered pieces per instruction (measured: ~4 k
+    // cycles per row).  The 128 q rows are copied into LDS like a K tile instead (64 rows per kv
+    // group, into the V half of its stage 1, which is free until the first MFMA block) and read
+    // from there.  Requested first so that the latency overlaps the staging below.
     x8 qreg[kFp8 ? 1 : 8];
     i32x8 qreg8[kFp8 ? 2 : 1];
-    if constexpr (kFp8) {
-      const uint8_t* src = qp + q_tok * p.q_sn + static_cast<int64_t>(head) * p.q_sh + g * 32;
+    const uint32_t lds_group = static_cast<uint32_t>(reinterpret_cast<uintptr_t>((lds_void*)group_smem));
+    {
+      const uint8_t* q_head = reinterpret_cast<const uint8_t*>(
+          qp + static_cast<int64_t>(q_begin) * p.q_sn + static_cast<int64_t>(head) * p.q_sh);
+      const uint32_t qdst = lds_group + kStageBytes + kKBytes + qs * 1024;
 #pragma unroll
-      for (int sl = 0; sl < 2; ++sl) {
-        const i32x4 lo = *reinterpret_cast<const i32x4*>(src + sl * 64);
-        const i32x4 hi = *reinterpret_cast<const i32x4*>(src + sl * 64 + 16);
-        qreg8[sl] = i32x8{lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
+      for (int n = 0; n < (kFp8 ? 2 : 4); ++n) {
+        int r = kg * 64 + (kFp8 ? 8 * (4 * n + qs) + cp8_row : 4 * (4 * n + qs) + cp_row);
+        r = r < q_rows ? r : q_rows - 1;  // ragged last q block: re-read the last row
+        const uint32_t off = kFp8 ? static_cast<uint32_t>(r * p.q_sn + cp8_chunk)
+                                  : static_cast<uint32_t>((r * p.q_sn + cp_chunk) * sizeof(T));
+        copy16_to_lds(q_head, off, qdst + n * 4096);
       }
-    } else {
-      const T* src = reinterpret_cast<const T*>(qp) + q_tok * p.q_sn + static_cast<int64_t>(head) * p.q_sh + g * 8;
-#pragma unroll
-      for (int ks = 0; ks < 8; ++ks) qreg[ks] = *reinterpret_cast<const x8*>(src + ks * 16);
     }
     // the row's kv block list goes to LDS: the main loop then has no global loads besides the
     // tile copies, whose completion it tracks by counting (s_waitcnt vmcnt)
     for (int i = tid; i < nb; i += kThreads) s_blk[i] = p.kv_idx[ptr0 + i];
+    __builtin_amdgcn_s_waitcnt(0x0f70);  // vmcnt(0): the compiler does not count the copies above
     __syncthreads();
     // number of 64-key tiles; only the last listed block can be the request's ragged tail
     int n_tiles = 2 * nb;
     if (kv_len - s_blk[nb - 1] * kBlockKV <= kTileKV) n_tiles -= 1;
     const int my_tiles = (n_tiles - kg + 1) >> 1;  // tiles kg, kg+2, ...
 
-    // (bf16/fp16) the softmax scale (log2 domain) is folded into Q, so S^T needs no multiply
-    if constexpr (!kFp8) {
-#pragma unroll
-      for (int ks = 0; ks < 8; ++ks)
-#pragma unroll
-        for (int e = 0; e < 8; ++e) qreg[ks][e] = static_cast<T>(static_cast<float>(qreg[ks][e]) * c);
-    }
     // softmax scale in the log2 domain; with fp8 operands the per-block dequantisation scales of
     // q (one per row of the list) and k (one per kv block) are folded in tile by tile
     float cq = c;
@@ -420,7 +443,6 @@ __global__ void __launch_bounds__(kThreads) sparse_fa_kernel(const FaParams p) {
                                  : static_cast<uint32_t>((4 * qs + cp_row) * p.k_sn + cp_chunk) * sizeof(T);
     const int64_t k_jstep = (kFp8 ? 32 : 16) * p.k_sn * static_cast<int64_t>(sizeof(TQK));
     const int64_t v_jstep = 16 * p.v_sn * static_cast<int64_t>(sizeof(T));
-    const uint32_t lds_group = static_cast<uint32_t>(reinterpret_cast<uintptr_t>((lds_void*)group_smem));
     constexpr int kKCopies = kFp8 ? 2 : 4, kVCopies = 4;  // copy instructions per wavefront and tile
     auto tile_start = [&](int j) { return s_blk[j] * kBlockKV + kg * kTileKV; };
     auto tile_valid = [&](int j) { return min(kTileKV, kv_len - tile_start(j)); };
@@ -512,6 +534,30 @@ __global__ void __launch_bounds__(kThreads) sparse_fa_kernel(const FaParams p) {
         copy_v_address(1);
       }
     }
+    // Q from LDS while the first tile copies are in flight: rows (qs % 2) * 32 + l32 of the tile that
+    // kv group qs / 2 copied, addressed like a K operand
+    {
+      const uint8_t* qt = smem + (qs >> 1) * kGroupBytes + kStageBytes + kKBytes +
+                          (qs & 1) * 32 * (kFp8 ? kRowBytes8 : kRowBytes) + k_rd_base;
+      if constexpr (kFp8) {
+#pragma unroll
+        for (int sl = 0; sl < 2; ++sl) {
+          const i32x4 lo = *reinterpret_cast<const i32x4*>(qt + (k_rd_x ^ (sl << 6)));
+          const i32x4 hi = *reinterpret_cast<const i32x4*>(qt + ((k_rd_x ^ (sl << 6)) ^ 16));
+          qreg8[sl] = i32x8{lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
+        }
+      } else {
+#pragma unroll
+        for (int ks = 0; ks < 8; ++ks) qreg[ks] = *reinterpret_cast<const x8*>(qt + (k_rd_x ^ (ks << 5)));
+        // the softmax scale (log2 domain) is folded into Q, so S^T needs no multiply
+#pragma unroll
+        for (int ks = 0; ks < 8; ++ks)
+#pragma unroll
+          for (int e = 0; e < 8; ++e) qreg[ks][e] = static_cast<T>(static_cast<float>(qreg[ks][e]) * c);
+      }
+    }
+    // (every wavefront holds its Q before the first barrier: the V copies of tile 1 overwrite it after)
+    __builtin_amdgcn_s_waitcnt(0xc07f);  // lgkmcnt(0)
     if (kg == 1) __builtin_amdgcn_s_barrier();
 
     f32x16 s[2];
@@ -764,12 +810,14 @@ __global__ void __launch_bounds__(kThreads) sparse_fa_kernel(const FaParams p) {
       md[(qs * 64 + lane) * 2 + 1] = d_part;
     }
     __syncthreads();
-    if (tid == kGroupThreads) s_next_row[(row_it + 1) & 1] = pop_row(p, blockIdx.x & (kXcds - 1), s_queue, &first_queue);
+    if (tid == kGroupThreads) fetch_next((row_it + 1) & 1);
     float m_all = 0.f, d_all = 0.f;  // kv group 0: row maximum and row sum over both groups
     // A lane owns one q row and runs of four d: stored from here, a row would leave as 32 scattered
     // 8-byte pieces per instruction (measured: ~12 k cycles per row).  The finished row goes through
     // a padded LDS tile instead and leaves in 16-byte pieces, 16 consecutive lanes per 256-byte row.
-    uint8_t* const out_row = smem + kOutTileOff + my_row * kOutRowBytes;
+    int ln_out = l32;
+    asm volatile("" : "+v"(ln_out));  // (not hoisted out of the row loop and spilled)
+    uint8_t* const out_row = smem + kOutTileOff + (qs * 32 + ln_out) * kOutRowBytes;
     bool store_row = parts == 1;
     if (kg == 0) {
       const float m1 = md[(qs * 64 + lane) * 2 + 0], d1 = md[(qs * 64 + lane) * 2 + 1];
@@ -804,20 +852,24 @@ __global__ void __launch_bounds__(kThreads) sparse_fa_kernel(const FaParams p) {
         // result (same lane layout as the LDS merge area)
         float* part_ws = p.split_ws +
                          static_cast<int64_t>(split_slot * kMaxSplitParts + part) * kSplitPartFloats;
+        // (opaque lane index: see the row store below)
+        int ln = lane;
+        asm volatile("" : "+v"(ln));
+        float* lane_ws = part_ws + (qs * 16 * 2 * 64 + ln) * 2;
+        f32x4 t4[16];
 #pragma unroll
-        for (int dt = 0; dt < 4; ++dt)
+        for (int e = 0; e < 16; ++e) t4[e] = mo[(qs * 16 + e) * 64 + lane];
+        __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
-          for (int i4 = 0; i4 < 4; ++i4) {
-            const f32x4 t4 = mo[(qs * 16 + dt * 4 + i4) * 64 + lane];
-            float u[4];
+        for (int e = 0; e < 16; ++e) {
+          float u[4];
 #pragma unroll
-            for (int j = 0; j < 4; ++j) u[j] = o_acc[dt][i4 * 4 + j] * a0 + t4[j] * a1;
-            // two planes of 8-byte pairs: each store instruction covers 512 contiguous bytes
-            float* dst = part_ws + ((qs * 16 + dt * 4 + i4) * 2 * 64 + lane) * 2;
-            store_pair_device(dst, u[0], u[1]);
-            store_pair_device(dst + 128, u[2], u[3]);
-          }
-        store_pair_device(part_ws + 128 * 128 + (qs * 64 + lane) * 2, m, d_tot);
+          for (int j = 0; j < 4; ++j) u[j] = o_acc[e >> 2][(e & 3) * 4 + j] * a0 + t4[e][j] * a1;
+          // two planes of 8-byte pairs: each store instruction covers 512 contiguous bytes
+          store_pair_device(lane_ws + e * 256, u[0], u[1]);
+          store_pair_device(lane_ws + e * 256 + 128, u[2], u[3]);
+        }
+        store_pair_device(part_ws + 128 * 128 + (qs * 64 + ln) * 2, m, d_tot);
       }
     }
     if (parts > 1) {
@@ -842,21 +894,27 @@ __global__ void __launch_bounds__(kThreads) sparse_fa_kernel(const FaParams p) {
           for (int dt = 0; dt < 4; ++dt)
 #pragma unroll
             for (int e = 0; e < 16; ++e) o_acc[dt][e] = 0.f;
+          int ln = lane;
+          asm volatile("" : "+v"(ln));
           for (int i = 0; i < parts; ++i) {
-            const float* part_ws = slot_ws + i * kSplitPartFloats;
+            const float* lane_ws = slot_ws + i * kSplitPartFloats + (qs * 16 * 2 * 64 + ln) * 2;
             const float a = __builtin_amdgcn_exp2f(m_p[i] - m_all);
             d_all += d_p[i] * a;
+            // half of the part's values at a time, all loads of a half in flight together
 #pragma unroll
-            for (int dt = 0; dt < 4; ++dt)
+            for (int half = 0; half < 2; ++half) {
+              float u[8][4];
 #pragma unroll
-              for (int i4 = 0; i4 < 4; ++i4) {
-                const float* src = part_ws + ((qs * 16 + dt * 4 + i4) * 2 * 64 + lane) * 2;
-                float u[4];
-                load_pair_device(src, u[0], u[1]);
-                load_pair_device(src + 128, u[2], u[3]);
-#pragma unroll
-                for (int j = 0; j < 4; ++j) o_acc[dt][i4 * 4 + j] += u[j] * a;
+              for (int e = 0; e < 8; ++e) {
+                load_pair_device(lane_ws + (half * 8 + e) * 256, u[e][0], u[e][1]);
+                load_pair_device(lane_ws + (half * 8 + e) * 256 + 128, u[e][2], u[e][3]);
               }
+              __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+              for (int e = 0; e < 8; ++e)
+#pragma unroll
+                for (int j = 0; j < 4; ++j) o_acc[half * 2 + (e >> 2)][(e & 3) * 4 + j] += u[e][j] * a;
+            }
           }
           const float inv = __builtin_amdgcn_rcpf(d_all);
 #pragma unroll
@@ -960,8 +1018,9 @@ extern "C" int fo_sparse_fa_run(const void* q, const void* k, const void* v, voi
   for (int i = 0; i < 8; ++i)
     FO_REQUIRE(strides[i] % (dtype == FO_FP8_E4M3 && i < 4 ? 16 : 8) == 0 && strides[i] > 0,
                "sparse_fa: strides must be positive multiples of 16 bytes (128-bit accesses)");
-  FO_REQUIRE(k_stride_n < (int64_t(1) << 23) && v_stride_n < (int64_t(1) << 23),
-             "sparse_fa: k/v token strides must be below 2^23 elements (32-bit tile offsets)");
+  FO_REQUIRE(q_stride_n < (int64_t(1) << 23) && k_stride_n < (int64_t(1) << 23) &&
+                 v_stride_n < (int64_t(1) << 23),
+             "sparse_fa: q/k/v token strides must be below 2^23 elements (32-bit tile offsets)");
   if (dtype == FO_FP8_E4M3)
     FO_REQUIRE(q_scale && k_scale && q_blk_base && kv_blk_base && n_q_blocks > 0 && n_kv_blocks > 0,
                "sparse_fa: fp8 q/k need q_scale, k_scale, the block numbering and the scale row lengths");
