@@ -39,6 +39,8 @@
 // that XCD's L2.
 #include "fo_common.h"
 
+#include <type_traits>
+
 namespace {
 
 typedef __attribute__((ext_vector_type(8))) __bf16 bf16x8;
@@ -276,6 +278,7 @@ __global__ void __launch_bounds__(kThreads) gemm_kernel(const GemmParams p) {
   extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
   __shared__ int32_t s_heads[kMaxHeads + 1];  // GEMM-O: head | (row0 selects) << 16 | (row1 selects) << 17
   __shared__ int32_t s_nsel;
+  __shared__ __attribute__((aligned(16))) uint8_t s_scrap[1024];
   // GEMM-O: per k step, k offset | (row0 selects) << 16 | (row1 selects) << 17; four entries past
   // the end repeat the last step
   __shared__ int32_t s_step[kReduce ? kMaxSteps + 4 : 1];
@@ -422,9 +425,11 @@ __global__ void __launch_bounds__(kThreads) gemm_kernel(const GemmParams p) {
         return (it < n_iter ? it : n_iter - 1) * kBK;
       }
     };
+    // copies past the last k step (kept so that every step issues the same instructions) land in a
+    // scrap kilobyte, so the ring is free for the epilogue as soon as the last reads are done
     auto copy_one = [&](int it, int entry, int j) {
-      uint8_t* dst = smem + (it % kStages) * kStageBytes + wv * 1024;
-      copy16_to_lds(cp_src[j] + (entry & 0xFFFF), dst + j * kUnitBytes);
+      uint8_t* dst = it < n_iter ? smem + (it % kStages) * kStageBytes + wv * 1024 + j * kUnitBytes : s_scrap;
+      copy16_to_lds(cp_src[j] + (entry & 0xFFFF), dst);
     };
     auto copy_stage = [&](int it) {
       const int entry = step_entry(it);
@@ -447,88 +452,30 @@ __global__ void __launch_bounds__(kThreads) gemm_kernel(const GemmParams p) {
           __builtin_amdgcn_s_barrier();
           copy_stage(it + 3);
         }
+        __builtin_amdgcn_s_barrier();  // the others' "ring is free" barrier before their epilogue
       }
       continue;
     }
 
-    // ---- accumulators, initialised from bias / cached partial ----
+    // ---- accumulators (bias / cached partial are added in the epilogue) ----
     // acc[nt][mt][i]: n = n0 + nt*32 + (i/4)*8 + g*4 + i%4, m = m0 + mt*32 + l32
-    // All init loads are issued before the first copies and converted after them; vector-memory
-    // loads return in order, so "tile 0 landed" below also covers them.
     const int m0 = r[wr] * kTile + wh * 64;
     const int n0 = c[wc] * kTile;
     const int64_t y_batch = static_cast<int64_t>(bz) * p.m * p.n;
-    int64_t row_off[MT];
-#pragma unroll
-    for (int mt = 0; mt < MT; ++mt) {
-      const int mrow = m0 + mt * 32 + l32;
-      row_off[mt] = y_batch + static_cast<int64_t>(mrow < p.m ? mrow : p.m - 1) * p.n + n0 + g * 4;
-    }
-    auto first_copies = [&]() {
-      __builtin_amdgcn_sched_barrier(0);
-#pragma unroll
-      for (int s = 0; s < kStages - 1; ++s)
-        if (n_iter > 0) copy_stage(s);
-      __builtin_amdgcn_sched_barrier(0);
-    };
     f32x16 acc[NT][MT];
     // the previous work item's stores are complete: from here on vmcnt counts loads only
     __builtin_amdgcn_s_waitcnt(0x0f70);
-    if (p.bias_kind == FO_BIAS_VECTOR) {
-      x4 bv[NT][4];
+    __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
-      for (int nt = 0; nt < NT; ++nt)
+    for (int s = 0; s < kStages - 1; ++s)
+      if (n_iter > 0) copy_stage(s);
+    __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
-        for (int i4 = 0; i4 < 4; ++i4)
-          bv[nt][i4] = *reinterpret_cast<const x4*>(static_cast<const T*>(p.bias) + n0 + g * 4 + nt * 32 + i4 * 8);
-      first_copies();
+    for (int nt = 0; nt < NT; ++nt)
 #pragma unroll
-      for (int nt = 0; nt < NT; ++nt)
+      for (int mt = 0; mt < MT; ++mt)
 #pragma unroll
-        for (int mt = 0; mt < MT; ++mt)
-#pragma unroll
-          for (int i = 0; i < 16; ++i) acc[nt][mt][i] = static_cast<float>(bv[nt][i >> 2][i & 3]);
-    } else if (p.bias_kind == FO_BIAS_MATRIX && p.bias_f32) {
-      f32x4 bm[NT][MT][4];
-#pragma unroll
-      for (int nt = 0; nt < NT; ++nt)
-#pragma unroll
-        for (int mt = 0; mt < MT; ++mt)
-#pragma unroll
-          for (int i4 = 0; i4 < 4; ++i4)
-            bm[nt][mt][i4] = *reinterpret_cast<const f32x4*>(static_cast<const float*>(p.bias) + row_off[mt] + nt * 32 + i4 * 8);
-      first_copies();
-#pragma unroll
-      for (int nt = 0; nt < NT; ++nt)
-#pragma unroll
-        for (int mt = 0; mt < MT; ++mt)
-#pragma unroll
-          for (int i = 0; i < 16; ++i) acc[nt][mt][i] = bm[nt][mt][i >> 2][i & 3];
-    } else if (p.bias_kind == FO_BIAS_MATRIX) {
-      x4 bm[NT][MT][4];
-#pragma unroll
-      for (int nt = 0; nt < NT; ++nt)
-#pragma unroll
-        for (int mt = 0; mt < MT; ++mt)
-#pragma unroll
-          for (int i4 = 0; i4 < 4; ++i4)
-            bm[nt][mt][i4] = *reinterpret_cast<const x4*>(static_cast<const T*>(p.bias) + row_off[mt] + nt * 32 + i4 * 8);
-      first_copies();
-#pragma unroll
-      for (int nt = 0; nt < NT; ++nt)
-#pragma unroll
-        for (int mt = 0; mt < MT; ++mt)
-#pragma unroll
-          for (int i = 0; i < 16; ++i) acc[nt][mt][i] = static_cast<float>(bm[nt][mt][i >> 2][i & 3]);
-    } else {
-      first_copies();
-#pragma unroll
-      for (int nt = 0; nt < NT; ++nt)
-#pragma unroll
-        for (int mt = 0; mt < MT; ++mt)
-#pragma unroll
-          for (int i = 0; i < 16; ++i) acc[nt][mt][i] = 0.f;
-    }
+        for (int i = 0; i < 16; ++i) acc[nt][mt][i] = 0.f;
 
     // LDS byte offsets of this wavefront's operand rows inside a stage
     const int a_base = (2 + wc) * kUnitBytes + l32 * kRowBytes;        // W rows nt*32 + l32
@@ -600,33 +547,80 @@ __global__ void __launch_bounds__(kThreads) gemm_kernel(const GemmParams p) {
     }
 
     // ---- epilogue ----
+    // In the accumulator layout a lane owns one output row and runs of four columns: written from
+    // there, a store instruction is 64 scattered 8-byte pieces (measured: ~12 % of the FLUX-sized
+    // launches; the bias matrix read the same way, as much again).  Each wavefront therefore turns
+    // its 64 x 128 block through its own 16 KB of the ring, 32 rows at a time in fp32, and adds the
+    // bias and stores from a layout in which 32 consecutive lanes cover one row.
+    if (n_iter > 0) __builtin_amdgcn_s_barrier();  // every wavefront is done reading the ring
     {
+      // (the lane index is made opaque: otherwise the per-lane address terms are computed once per
+      // kernel, spilled, and every reload waits for the store before it)
+      int ln = lane;
+      asm volatile("" : "+v"(ln));
+      const int col4 = ln & 31, rsub = ln >> 5, wl32 = ln & 31, wg = ln >> 5;
+      uint8_t* region = smem + wv * (kSmemBytes / 8);
+      const int64_t y_batch = static_cast<int64_t>(bz) * p.m * p.n;
+      float bvec[4] = {0.f, 0.f, 0.f, 0.f};
+      if (p.bias_kind == FO_BIAS_VECTOR) {
+        const x4 bv = *reinterpret_cast<const x4*>(static_cast<const T*>(p.bias) + n0 + col4 * 4);
 #pragma unroll
-      for (int mt = 0; mt < MT; ++mt) {
-        if (m0 + mt * 32 + l32 >= p.m) continue;
-        if (p.y_f32) {
-          float* yrow = static_cast<float*>(p.y) + row_off[mt];
+        for (int j = 0; j < 4; ++j) bvec[j] = static_cast<float>(bv[j]);
+      }
+      // one half (32 rows) of the block; BiasT: element type of the bias matrix, if there is one
+      auto turn_half = [&](int mt, auto bias_tag) {
+        using BiasT = decltype(bias_tag);
+        const int row_base = m0 + mt * 32;
+        // 16-byte chunk c of row r sits at chunk position c ^ r (rows are 512 bytes = 32 chunks)
 #pragma unroll
-          for (int nt = 0; nt < NT; ++nt)
+        for (int nt = 0; nt < NT; ++nt)
 #pragma unroll
-            for (int i4 = 0; i4 < 4; ++i4) {
-              f32x4 out;
+          for (int i4 = 0; i4 < 4; ++i4) {
+            f32x4 v;
 #pragma unroll
-              for (int j = 0; j < 4; ++j) out[j] = acc[nt][mt][i4 * 4 + j];
-              *reinterpret_cast<f32x4*>(yrow + nt * 32 + i4 * 8) = out;
-            }
-        } else {
-          T* yrow = static_cast<T*>(p.y) + row_off[mt];
+            for (int j = 0; j < 4; ++j) v[j] = acc[nt][mt][i4 * 4 + j];
+            const int chunk = nt * 8 + i4 * 2 + wg;
+            *reinterpret_cast<f32x4*>(region + wl32 * 512 + ((chunk ^ wl32) << 4)) = v;
+          }
+        // cached partial of these rows: all sixteen loads in flight together
+        using BiasVec = typename std::conditional<sizeof(BiasT) == 4, f32x4, x4>::type;
+        BiasVec bm[16];
+        const bool has_matrix = p.bias_kind == FO_BIAS_MATRIX;
+        if (has_matrix) {
 #pragma unroll
-          for (int nt = 0; nt < NT; ++nt)
+          for (int i = 0; i < 16; ++i) {
+            int grow = row_base + i * 2 + rsub;
+            grow = grow < p.m ? grow : p.m - 1;
+            const int64_t off = y_batch + static_cast<int64_t>(grow) * p.n + n0 + col4 * 4;
+            bm[i] = *reinterpret_cast<const BiasVec*>(static_cast<const BiasT*>(p.bias) + off);
+          }
+        }
 #pragma unroll
-            for (int i4 = 0; i4 < 4; ++i4) {
+        for (int i = 0; i < 16; ++i) {
+          const int row = i * 2 + rsub;
+          f32x4 v = *reinterpret_cast<const f32x4*>(region + row * 512 + ((col4 ^ row) << 4));
+#pragma unroll
+          for (int j = 0; j < 4; ++j) v[j] += has_matrix ? static_cast<float>(bm[i][j]) : bvec[j];
+          const int grow = row_base + row;
+          if (grow < p.m) {
+            const int64_t off = y_batch + static_cast<int64_t>(grow) * p.n + n0 + col4 * 4;
+            if (p.y_f32) {
+              *reinterpret_cast<f32x4*>(static_cast<float*>(p.y) + off) = v;
+            } else {
               x4 out;
 #pragma unroll
-              for (int j = 0; j < 4; ++j) out[j] = static_cast<T>(acc[nt][mt][i4 * 4 + j]);
-              *reinterpret_cast<x4*>(yrow + nt * 32 + i4 * 8) = out;
+              for (int j = 0; j < 4; ++j) out[j] = static_cast<T>(v[j]);
+              *reinterpret_cast<x4*>(static_cast<T*>(p.y) + off) = out;
             }
+          }
         }
+      };
+      if (p.bias_kind == FO_BIAS_MATRIX && p.bias_f32) {
+#pragma unroll
+        for (int mt = 0; mt < MT; ++mt) turn_half(mt, 0.f);
+      } else {
+#pragma unroll
+        for (int mt = 0; mt < MT; ++mt) turn_half(mt, T{});
       }
     }
   }
