@@ -257,7 +257,7 @@ __global__ void __launch_bounds__(kThreads) sparse_fa_kernel(const FaParams p) {
   __shared__ RowInfo s_next_row[2];
   __shared__ int s_arrived;
   __shared__ int s_queue[40];  // the queue words of `sched`, read once
-  __shared__ int32_t s_blk[kMaxRowBlocks];  // kv block list of the current row
+  __shared__ uint16_t s_blk2[2][kMaxRowBlocks];  // kv block list of this row / the next one
 
   const int tid = threadIdx.x, lane = tid & 63;
   const int wv = __builtin_amdgcn_readfirstlane(tid >> 6);  // wavefront index, kept scalar
@@ -305,43 +305,54 @@ __global__ void __launch_bounds__(kThreads) sparse_fa_kernel(const FaParams p) {
     s_queue[9 + tid - 64] = p.sched[kSchedSplitStart + tid - 64];  // split start, parts, first slot
   __syncthreads();
   int first_queue = 0;  // kept by the popping lane (the first pop is lane 0's, the others lane 256's)
-  // one lane: pop the next item and gather its row's metadata (two rounds of loads) into LDS
+  // One wavefront: lane 0 pops the next item and gathers its row's metadata (two rounds of loads),
+  // then all lanes copy the row's kv block list; both go to LDS for the whole workgroup.
   auto fetch_next = [&](int slot_idx) {
     RowInfo ri;
-    for (;;) {
-      const Item item = pop_row(p, blockIdx.x & (kXcds - 1), s_queue, &first_queue);
-      ri.row = item.row;
-      if (item.row < 0) break;
-      const int w = item.row;
-      ri.part = item.meta & 15;
-      ri.parts = (item.meta >> 4) & 15;
-      ri.slot = item.meta >> 8;
-      ri.req = p.row_req[w];
-      ri.qb = p.row_qb[w];
-      ri.head = p.row_head[w];
-      ri.ptr0 = p.kv_row_ptr[w];
-      // (a row longer than the LDS list is cut; the host side refuses such requests at plan time)
-      ri.nb = min(p.kv_row_ptr[w + 1] - ri.ptr0, kMaxRowBlocks);
-      ri.q_begin = p.qo_indptr[ri.req] + ri.qb * kBlockQ;
-      ri.q_rows = min(kBlockQ, p.qo_indptr[ri.req + 1] - ri.q_begin);
-      ri.kv_begin = p.kv_indptr[ri.req];
-      ri.kv_len = p.kv_indptr[ri.req + 1] - ri.kv_begin;
-      if (ri.parts > 1) {
-        if (ri.nb < 2 * ri.parts || p.split_ws == nullptr) {
-          // too short to share (or nowhere to put partial results): part 0 does the whole row
-          if (ri.part > 0) continue;
-          ri.parts = 1;
-        } else {
-          const int b0 = ri.nb * ri.part / ri.parts, b1 = ri.nb * (ri.part + 1) / ri.parts;
-          ri.ptr0 += b0;
-          ri.nb = b1 - b0;
+    ri.row = -1;
+    ri.ptr0 = 0;
+    ri.nb = 0;
+    if (lane == 0) {
+      for (;;) {
+        const Item item = pop_row(p, blockIdx.x & (kXcds - 1), s_queue, &first_queue);
+        ri.row = item.row;
+        if (item.row < 0) break;
+        const int w = item.row;
+        ri.part = item.meta & 15;
+        ri.parts = (item.meta >> 4) & 15;
+        ri.slot = item.meta >> 8;
+        ri.req = p.row_req[w];
+        ri.qb = p.row_qb[w];
+        ri.head = p.row_head[w];
+        ri.ptr0 = p.kv_row_ptr[w];
+        // (a row longer than the LDS list is cut; the host side refuses such requests at plan time)
+        ri.nb = min(p.kv_row_ptr[w + 1] - ri.ptr0, kMaxRowBlocks);
+        ri.q_begin = p.qo_indptr[ri.req] + ri.qb * kBlockQ;
+        ri.q_rows = min(kBlockQ, p.qo_indptr[ri.req + 1] - ri.q_begin);
+        ri.kv_begin = p.kv_indptr[ri.req];
+        ri.kv_len = p.kv_indptr[ri.req + 1] - ri.kv_begin;
+        if (ri.parts > 1) {
+          if (ri.nb < 2 * ri.parts || p.split_ws == nullptr) {
+            // too short to share (or nowhere to put partial results): part 0 does the whole row
+            if (ri.part > 0) continue;
+            ri.parts = 1;
+          } else {
+            const int b0 = ri.nb * ri.part / ri.parts, b1 = ri.nb * (ri.part + 1) / ri.parts;
+            ri.ptr0 += b0;
+            ri.nb = b1 - b0;
+          }
         }
+        break;
       }
-      break;
+      s_next_row[slot_idx] = ri;
     }
-    s_next_row[slot_idx] = ri;
+    const int row = __builtin_amdgcn_readfirstlane(ri.row);
+    if (row >= 0) {
+      const int list0 = __builtin_amdgcn_readfirstlane(ri.ptr0), n = __builtin_amdgcn_readfirstlane(ri.nb);
+      for (int i = lane; i < n; i += 64) s_blk2[slot_idx][i] = static_cast<uint16_t>(p.kv_idx[list0 + i]);
+    }
   };
-  if (tid == 0) fetch_next(0);
+  if (wv == 0) fetch_next(0);
   for (int row_it = 0;; ++row_it) {
     __syncthreads();  // s_next_row is published; everyone is done with the previous row's LDS data
     const RowInfo& ri = s_next_row[row_it & 1];
@@ -355,7 +366,8 @@ __global__ void __launch_bounds__(kThreads) sparse_fa_kernel(const FaParams p) {
     const int q_rows = __builtin_amdgcn_readfirstlane(ri.q_rows);
     const int kv_begin = __builtin_amdgcn_readfirstlane(ri.kv_begin);
     const int kv_len = __builtin_amdgcn_readfirstlane(ri.kv_len);
-    const int ptr0 = __builtin_amdgcn_readfirstlane(ri.ptr0), nb = __builtin_amdgcn_readfirstlane(ri.nb);
+    const int nb = __builtin_amdgcn_readfirstlane(ri.nb);
+    const uint16_t* const s_blk = s_blk2[row_it & 1];
 
     const int my_row = qs * 32 + l32;  // q row of this lane inside the block
     const bool row_ok = my_row < q_rows;
@@ -370,7 +382,7 @@ __global__ void __launch_bounds__(kThreads) sparse_fa_kernel(const FaParams p) {
         for (int j = 0; j < 8; ++j) reinterpret_cast<u32x4*>(dst)[j] = z;
         if (p.lse && g == 0) p.lse[q_tok * p.num_heads + head] = kNegInf;
       }
-      if (tid == kGroupThreads) fetch_next((row_it + 1) & 1);
+      if (wv == 4) fetch_next((row_it + 1) & 1);
       continue;
     }
 
@@ -395,11 +407,8 @@ __global__ void __launch_bounds__(kThreads) sparse_fa_kernel(const FaParams p) {
         copy16_to_lds(q_head, off, qdst + n * 4096);
       }
     }
-    // the row's kv block list goes to LDS: the main loop then has no global loads besides the
-    // tile copies, whose completion it tracks by counting (s_waitcnt vmcnt)
-    for (int i = tid; i < nb; i += kThreads) s_blk[i] = p.kv_idx[ptr0 + i];
-    __builtin_amdgcn_s_waitcnt(0x0f70);  // vmcnt(0): the compiler does not count the copies above
-    __syncthreads();
+    // (the row's kv block list is in LDS already: the main loop has no global loads besides the
+    // tile copies, whose completion it tracks by counting, s_waitcnt vmcnt)
     // number of 64-key tiles; only the last listed block can be the request's ragged tail
     int n_tiles = 2 * nb;
     if (kv_len - s_blk[nb - 1] * kBlockKV <= kTileKV) n_tiles -= 1;
@@ -534,6 +543,16 @@ __global__ void __launch_bounds__(kThreads) sparse_fa_kernel(const FaParams p) {
         copy_v_address(1);
       }
     }
+    // Q has landed once only the tile copies issued after it are outstanding; then for every
+    // wavefront after the barrier
+    if (my_tiles > 1) {
+      __builtin_amdgcn_s_waitcnt(0x0f70 | (2 * kKCopies + kVCopies));
+    } else if (my_tiles == 1) {
+      __builtin_amdgcn_s_waitcnt(0x0f70 | (kKCopies + kVCopies));
+    } else {
+      __builtin_amdgcn_s_waitcnt(0x0f70);
+    }
+    __builtin_amdgcn_s_barrier();
     // Q from LDS while the first tile copies are in flight: rows (qs % 2) * 32 + l32 of the tile that
     // kv group qs / 2 copied, addressed like a K operand
     {
@@ -810,7 +829,7 @@ __global__ void __launch_bounds__(kThreads) sparse_fa_kernel(const FaParams p) {
       md[(qs * 64 + lane) * 2 + 1] = d_part;
     }
     __syncthreads();
-    if (tid == kGroupThreads) fetch_next((row_it + 1) & 1);
+    if (wv == 4) fetch_next((row_it + 1) & 1);
     float m_all = 0.f, d_all = 0.f;  // kv group 0: row maximum and row sum over both groups
     // A lane owns one q row and runs of four d: stored from here, a row would leave as 32 scattered
     // 8-byte pieces per instruction (measured: ~12 k cycles per row).  The finished row goes through
