@@ -26,11 +26,12 @@
 // keeps logical 16-byte chunk c at position c ^ ((r >> 2) & 3), applied on the global side; the
 // 128-bit operand reads of 16 consecutive rows then cover all 64 banks.
 //
-// The product is formed transposed (A operand = W rows, B operand = X rows) so that in the 32 x 32
-// accumulator layout a lane owns one output row and runs of 4 consecutive columns: the epilogue
-// reads the init matrix and writes the result with 8/16-byte accesses without going through LDS.
-// fp32 accumulation starts from the init value converted to fp32; one round-to-nearest cast at
-// the end.
+// The product is formed transposed (A operand = W rows, B operand = X rows): in the 32 x 32
+// accumulator layout a lane owns one output row and runs of 4 consecutive columns.  Stored (or the
+// init matrix read) from that layout, a wavefront instruction is 64 scattered 8-byte pieces, so the
+// epilogue turns each wavefront's block through its own part of the (by then free) operand ring,
+// 32 rows at a time in fp32, into a layout where 32 consecutive lanes cover one row; there the bias
+// vector or the cached partial is added in fp32 and the result is rounded once and stored.
 //
 // Work order.  Workgroups are persistent (one per CU).  The quad list is ordered by token window,
 // then column pair, then row pair, and XCD x (= blockIdx % 8) owns the x-th contiguous eighth of it.

@@ -30,6 +30,16 @@
 // Work distribution: workgroups are persistent and pop rows from 8 queues (one per XCD, chosen by
 // blockIdx % 8) that the decoder filled head by head, so one XCD's L2 serves a few heads' K/V; an
 // idle XCD steals from its neighbours.  The last workgroup to finish resets the queue cursors.
+// When a queue is so short that half of its XCD's workgroups would stay idle, its positions stand
+// for parts of rows (ranges of a row's kv blocks): parts publish unnormalised partial results to
+// the caller's workspace and the last one to arrive combines them (see the end of the row loop).
+//
+// Between rows: while kv group 0 combines the two groups' states, one wavefront of group 1 pops the
+// next item, gathers its row's metadata and copies its kv block list into LDS, so the next row
+// starts with everything at hand: Q (copied into LDS like a K tile, then read as an operand) and
+// the first K/V tiles are requested together.  The finished row goes through a padded LDS tile and
+// leaves in 16-byte pieces, 16 consecutive lanes per 256-byte output row.  (Both were measured:
+// fetched or stored from the accumulator layout, a wavefront instruction is 64 scattered pieces.)
 //
 // Numerics follow the reference kernel (include/flashomni/attention/prefill.cuh:759-962): base-2
 // softmax p = exp2(s*c - m*c) with c = sm_scale*log2(e), P rounded to the activation type before
