@@ -363,8 +363,8 @@ def main():
         "frac": round(fa_flops / (fa_ms * 1e-3) / 1e12 / PEAK_BF16, 4),
         # HBM bytes per launch from two rocprofv3 --pmc runs of this command (FETCH_SIZE 72074.6 KiB x 2.0,
         # the factor a 256 MiB copy kernel gives for that counter, + WRITE_SIZE 39257.7 KiB x 1.0);
-        # the algorithmic bytes of the launch are 98.6e6 (the excess includes ~50e6 of register spill
-        # traffic: per-lane constants parked in scratch memory across the main loop)
+        # the algorithmic bytes of the launch are 98.6e6 (the excess is K/V re-fetched after falling out
+        # of an XCD's L2, which three heads share)
         "traffic": FA_C0_HBM_BYTES if 0 in configs else None, "traffic_unit": "bytes/launch",
         "launch_ms": round(fa_ms, 5), "algorithmic_flop_per_launch": fa_flops,
     }
