@@ -190,6 +190,13 @@ def bench_big_gemms(dev, index, iters, warmup):
     res = {}
     ms = time_gpu(lambda: fo.flashomni_gemm(x, wq, s.heads, info, ip, 0, bq, out=out), iters, warmup)
     res["gemm_q"] = entry(ms, flops=wl.gemm_q_flops())
+    # the same projection with the fp8 quantisation of its result fused in (no 16-bit result written)
+    q8 = torch.empty(1, s.seq, s.hidden, dtype=torch.float8_e4m3fn, device=dev)
+    q8s = torch.empty(s.heads, s.n_blocks, dtype=torch.float32, device=dev)
+    ms = time_gpu(lambda: fo.flashomni_gemm(x, wq, s.heads, info, ip, 0, bq, out=False, quant_out=(q8, q8s)),
+                  iters, warmup)
+    res["gemm_q_fused_fp8"] = entry(ms, flops=wl.gemm_q_flops())
+    del q8, q8s
     ms = time_gpu(lambda: fo.flashomni_gemm_reduction(x, wq, s.heads, info, ip, 0, bias=bq,
                                                       is_for_cache=True), iters, warmup)
     res["gemm_o_cache"] = entry(ms, flops=wl.gemm_o_flops(True))

@@ -32,6 +32,8 @@ SIGNATURES = {
     "fo_gemm_workspace_bytes": ([c_i32, c_i32, c_i32], c_i64),
     "fo_gemm_q": ([c_vp] * 4 + [c_int] + [c_i32] * 6 + [c_vp, c_vp, c_i32, c_int, c_vp, c_i64, c_vp],
                   c_int),
+    "fo_gemm_q_quant": ([c_vp] * 6 + [c_int] + [c_i32] * 6 + [c_vp, c_vp, c_i32, c_int, c_vp, c_i64, c_vp],
+                        c_int),
     "fo_gemm_o": ([c_vp] * 4 + [c_int] * 4 + [c_i32] * 6 + [c_vp, c_vp, c_i32, c_int, c_vp, c_i64, c_vp],
                   c_int),
     "fo_quant_fp8_block": ([c_vp, c_int, c_i64, c_i64, c_vp, c_vp, c_vp, c_vp, c_i32, c_i32, c_i32,

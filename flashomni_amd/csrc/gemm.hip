@@ -106,6 +106,11 @@ struct GemmParams {
   int32_t bias_kind;  // FO_BIAS_*
   int32_t bias_f32;   // matrix bias is fp32
   int32_t y_f32;      // output is fp32
+  // GEMM-Q with fused quantisation: e4m3fn bytes [B, M, N] and one scale per (head, token block),
+  // y_scale[head * scale_row_len + b * n_row_tiles + token block]; y may then be null
+  uint8_t* y8;
+  float* y_scale;
+  int32_t scale_row_len;
 };
 
 // 64 lanes x 16 bytes, global -> LDS at lds_base + lane*16 (lds_base is wavefront-uniform)
@@ -280,6 +285,7 @@ __global__ void __launch_bounds__(kThreads) gemm_kernel(const GemmParams p) {
   __shared__ int32_t s_heads[kMaxHeads + 1];  // GEMM-O: head | (row0 selects) << 16 | (row1 selects) << 17
   __shared__ int32_t s_nsel;
   __shared__ __attribute__((aligned(16))) uint8_t s_scrap[1024];
+  __shared__ float s_amax[kThreads / 64];
   // GEMM-O: per k step, k offset | (row0 selects) << 16 | (row1 selects) << 17; four entries past
   // the end repeat the last step
   __shared__ int32_t s_step[kReduce ? kMaxSteps + 4 : 1];
@@ -455,6 +461,9 @@ __global__ void __launch_bounds__(kThreads) gemm_kernel(const GemmParams p) {
         }
         __builtin_amdgcn_s_barrier();  // the others' "ring is free" barrier before their epilogue
       }
+      if constexpr (!kReduce) {
+        if (p.y8) __builtin_amdgcn_s_barrier();  // ... and the one of their absmax exchange
+      }
       continue;
     }
 
@@ -563,7 +572,48 @@ __global__ void __launch_bounds__(kThreads) gemm_kernel(const GemmParams p) {
       uint8_t* region = smem + wv * (kSmemBytes / 8);
       const int64_t y_batch = static_cast<int64_t>(bz) * p.m * p.n;
       float bvec[4] = {0.f, 0.f, 0.f, 0.f};
-      if (p.bias_kind == FO_BIAS_VECTOR) {
+      // Fused quantisation (GEMM-Q): a unit is one (token block, head) slab, owned by two wavefronts.
+      // Its absmax needs the final values, so the bias is added in the accumulator layout here; the
+      // two wavefronts exchange their maxima through LDS; scale = absmax / 448 (1 for a zero slab).
+      float qscale = 1.f;
+      bool bias_added = false;
+      if constexpr (!kReduce) {
+        if (p.y8) {
+          if (p.bias_kind == FO_BIAS_VECTOR) {
+#pragma unroll
+            for (int nt = 0; nt < NT; ++nt)
+#pragma unroll
+              for (int i4 = 0; i4 < 4; ++i4) {
+                const x4 bv = *reinterpret_cast<const x4*>(static_cast<const T*>(p.bias) + n0 + nt * 32 +
+                                                           i4 * 8 + wg * 4);
+#pragma unroll
+                for (int mt = 0; mt < MT; ++mt)
+#pragma unroll
+                  for (int j = 0; j < 4; ++j) acc[nt][mt][i4 * 4 + j] += static_cast<float>(bv[j]);
+              }
+            bias_added = true;
+          }
+          float amax = 0.f;
+#pragma unroll
+          for (int mt = 0; mt < MT; ++mt)
+            if (m0 + mt * 32 + wl32 < p.m) {
+#pragma unroll
+              for (int nt = 0; nt < NT; ++nt)
+#pragma unroll
+                for (int i = 0; i < 16; ++i) amax = fmaxf(amax, fabsf(acc[nt][mt][i]));
+            }
+#pragma unroll
+          for (int off = 32; off > 0; off >>= 1) amax = fmaxf(amax, __shfl_xor(amax, off, 64));
+          if (lane == 0) s_amax[wv] = amax;
+          __builtin_amdgcn_s_waitcnt(0xc07f);  // lgkmcnt(0)
+          __builtin_amdgcn_s_barrier();
+          amax = fmaxf(s_amax[wv], s_amax[7 - wv]);  // the other half of the unit is wavefront 7 - wv
+          qscale = amax > 0.f ? amax / 448.0f : 1.0f;
+          if (wh == 0 && lane == 0)
+            p.y_scale[static_cast<int64_t>(c[wc]) * p.scale_row_len + bz * p.n_row_tiles + r[wr]] = qscale;
+        }
+      }
+      if (p.bias_kind == FO_BIAS_VECTOR && !bias_added) {
         const x4 bv = *reinterpret_cast<const x4*>(static_cast<const T*>(p.bias) + n0 + col4 * 4);
 #pragma unroll
         for (int j = 0; j < 4; ++j) bvec[j] = static_cast<float>(bv[j]);
@@ -607,11 +657,22 @@ __global__ void __launch_bounds__(kThreads) gemm_kernel(const GemmParams p) {
             const int64_t off = y_batch + static_cast<int64_t>(grow) * p.n + n0 + col4 * 4;
             if (p.y_f32) {
               *reinterpret_cast<f32x4*>(static_cast<float*>(p.y) + off) = v;
-            } else {
+            } else if (p.y) {
               x4 out;
 #pragma unroll
               for (int j = 0; j < 4; ++j) out[j] = static_cast<T>(v[j]);
               *reinterpret_cast<x4*>(static_cast<T*>(p.y) + off) = out;
+            }
+            if constexpr (!kReduce) {
+              if (p.y8) {
+                float f[4];
+#pragma unroll
+                for (int j = 0; j < 4; ++j) f[j] = fminf(fmaxf(v[j] / qscale, -448.0f), 448.0f);
+                unsigned w8 = 0;
+                w8 = __builtin_amdgcn_cvt_pk_fp8_f32(f[0], f[1], w8, false);
+                w8 = __builtin_amdgcn_cvt_pk_fp8_f32(f[2], f[3], w8, true);
+                *reinterpret_cast<unsigned*>(p.y8 + off) = w8;
+              }
             }
           }
         }
@@ -720,14 +781,16 @@ extern "C" int64_t fo_gemm_workspace_bytes(int32_t batch, int32_t m, int32_t n) 
   return 4 * workspace_ints(make_geom(batch, m, n), nullptr);
 }
 
-extern "C" int fo_gemm_q(const void* x, const void* w, const void* bias, void* y, int dtype,
-                         int32_t batch, int32_t m, int32_t n, int32_t k, int32_t sparse_q_size,
-                         int32_t num_qo_heads, const uint8_t* sparse_info,
-                         const int32_t* sparse_info_indptr, int32_t num_text_tokens, int is_full,
-                         void* workspace, int64_t workspace_bytes, void* stream) {
-  if (int rc = check_common(x, w, y, dtype, batch, m, n, k, sparse_q_size, num_qo_heads, workspace,
-                            workspace_bytes, !is_full))
+namespace {
+int gemm_q_impl(const void* x, const void* w, const void* bias, void* y, uint8_t* y8, float* y_scale,
+                int dtype, int32_t batch, int32_t m, int32_t n, int32_t k, int32_t sparse_q_size,
+                int32_t num_qo_heads, const uint8_t* sparse_info, const int32_t* sparse_info_indptr,
+                int32_t num_text_tokens, int is_full, void* workspace, int64_t workspace_bytes,
+                void* stream) {
+  if (int rc = check_common(x, w, y8 ? static_cast<void*>(y8) : y, dtype, batch, m, n, k, sparse_q_size,
+                            num_qo_heads, workspace, workspace_bytes, !is_full))
     return rc;
+  FO_REQUIRE((reinterpret_cast<uintptr_t>(y) & 15) == 0, "gemm: x, w, y must be 16-byte aligned");
   FO_REQUIRE(is_full || (sparse_info && sparse_info_indptr),
              "gemm: sparse_info and sparse_info_indptr are required unless is_full");
   FO_REQUIRE(num_text_tokens >= 0, "gemm: negative num_text_tokens");
@@ -742,9 +805,40 @@ extern "C" int fo_gemm_q(const void* x, const void* w, const void* bias, void* y
   p.flag = is_full ? 1 : 0;
   p.bias_kind = bias ? FO_BIAS_VECTOR : FO_BIAS_NONE;
   const ListGeom gm = make_geom(batch, m, n);
+  if (y8) {
+    FO_REQUIRE(y_scale, "gemm_q_quant: y_scale is null");
+    FO_REQUIRE(p.head_dim == kTile, "gemm_q_quant: head width %d is not supported (only 128)", p.head_dim);
+    p.y8 = y8;
+    p.y_scale = y_scale;
+    p.scale_row_len = batch * gm.n_row_tiles;
+  }
   hipStream_t s = static_cast<hipStream_t>(stream);
   return dtype == FO_BF16 ? launch<__bf16, false>(p, gm, !is_full, workspace, s)
                           : launch<_Float16, false>(p, gm, !is_full, workspace, s);
+}
+}  // namespace
+
+extern "C" int fo_gemm_q(const void* x, const void* w, const void* bias, void* y, int dtype,
+                         int32_t batch, int32_t m, int32_t n, int32_t k, int32_t sparse_q_size,
+                         int32_t num_qo_heads, const uint8_t* sparse_info,
+                         const int32_t* sparse_info_indptr, int32_t num_text_tokens, int is_full,
+                         void* workspace, int64_t workspace_bytes, void* stream) {
+  FO_REQUIRE(y, "gemm: null pointer");
+  return gemm_q_impl(x, w, bias, y, nullptr, nullptr, dtype, batch, m, n, k, sparse_q_size,
+                     num_qo_heads, sparse_info, sparse_info_indptr, num_text_tokens, is_full, workspace,
+                     workspace_bytes, stream);
+}
+
+extern "C" int fo_gemm_q_quant(const void* x, const void* w, const void* bias, void* y, uint8_t* y8,
+                               float* y_scale, int dtype, int32_t batch, int32_t m, int32_t n,
+                               int32_t k, int32_t sparse_q_size, int32_t num_qo_heads,
+                               const uint8_t* sparse_info, const int32_t* sparse_info_indptr,
+                               int32_t num_text_tokens, int is_full, void* workspace,
+                               int64_t workspace_bytes, void* stream) {
+  FO_REQUIRE(y8, "gemm_q_quant: y8 is null");
+  return gemm_q_impl(x, w, bias, y, y8, y_scale, dtype, batch, m, n, k, sparse_q_size, num_qo_heads,
+                     sparse_info, sparse_info_indptr, num_text_tokens, is_full, workspace,
+                     workspace_bytes, stream);
 }
 
 extern "C" int fo_gemm_o(const void* x, const void* w, const void* bias, void* y, int dtype,

@@ -41,12 +41,27 @@ def flashomni_gemm(
     out: torch.Tensor = None,
     sparse_q_size: int = 128,
     is_full: bool = False,
+    quant_out=None,
 ) -> torch.Tensor:
     """``out[b, tile] = A[b] @ B.T + bias`` for every (128-token block, 128-column) tile whose
     ``sparse_info`` bit is 1; the other tiles of ``out`` are left untouched (a fresh ``out`` is
-    ``torch.empty``, as in the reference)."""
+    ``torch.empty``, as in the reference).
+
+    ``quant_out`` (keyword-only extension, heads of width 128): ``(q8, scale)`` or ``True``.  The
+    computed tiles are also written as fp8 e4m3fn with one absmax scale per (head, 128-token block),
+    taken from the fp32 results before they are rounded: ``q8`` ``[B, M, N]`` float8_e4m3fn and
+    ``scale`` ``[H, B * ceil(M / 128)]`` float32, the operands
+    :meth:`BatchFlashOmniFAWithRaggedKVWrapper.run` takes as ``q`` and ``q_scale`` (what
+    :func:`quant_fp8_block` would make of ``out`` in a second pass).  With ``quant_out`` given and
+    ``out=False`` the 16-bit result is not written at all.  Returns ``out``, or ``(out, q8, scale)``
+    when ``quant_out`` is given (``out`` is None if it was not written)."""
     _check_gemm_operands(A, B, "flashomni_gemm")
-    if out is None:
+    skip_out = out is False
+    if skip_out:
+        if quant_out is None:
+            raise RuntimeError("flashomni_gemm: out=False needs quant_out")
+        out = None
+    elif out is None:
         out = torch.empty((A.shape[0], A.shape[1], B.shape[0]), device=A.device, dtype=A.dtype)
     elif out.shape != (A.shape[0], A.shape[1], B.shape[0]) or out.dtype != A.dtype \
             or not out.is_contiguous() or out.device != A.device:
@@ -61,12 +76,33 @@ def flashomni_gemm(
     L = _lib.lib()
     ws_bytes = L.fo_gemm_workspace_bytes(A.shape[0], A.shape[1], B.shape[0])
     workspace = torch.empty(ws_bytes, dtype=torch.uint8, device=A.device)  # tile-list scratch
-    _lib.check(L.fo_gemm_q(
-        _lib.ptr(A), _lib.ptr(B), _lib.ptr(bias), _lib.ptr(out), _lib.dtype_code(A.dtype),
-        A.shape[0], A.shape[1], B.shape[0], A.shape[2], sparse_q_size, num_qo_heads,
+    if quant_out is None:
+        _lib.check(L.fo_gemm_q(
+            _lib.ptr(A), _lib.ptr(B), _lib.ptr(bias), _lib.ptr(out), _lib.dtype_code(A.dtype),
+            A.shape[0], A.shape[1], B.shape[0], A.shape[2], sparse_q_size, num_qo_heads,
+            _lib.ptr(info), _lib.ptr(indptr), num_text_tokens, int(bool(is_full)),
+            _lib.ptr(workspace), ws_bytes, _lib.current_stream(A.device)))
+        return out
+    Bsz, M, N = A.shape[0], A.shape[1], B.shape[0]
+    n_blk = Bsz * ((M + 127) // 128)
+    if quant_out is True:
+        q8 = torch.empty((Bsz, M, N), dtype=torch.float8_e4m3fn, device=A.device)
+        scale = torch.empty((num_qo_heads, n_blk), dtype=torch.float32, device=A.device)
+    else:
+        q8, scale = quant_out
+        if q8.shape != (Bsz, M, N) or q8.dtype not in (torch.float8_e4m3fn, torch.uint8) \
+                or not q8.is_contiguous() or q8.device != A.device:
+            raise RuntimeError("flashomni_gemm: quant_out[0] must be a contiguous [B, M, N] float8_e4m3fn tensor")
+        if scale.shape != (num_qo_heads, n_blk) or scale.dtype != torch.float32 \
+                or not scale.is_contiguous() or scale.device != A.device:
+            raise RuntimeError("flashomni_gemm: quant_out[1] must be a contiguous [H, B * ceil(M / 128)] "
+                               "float32 tensor")
+    _lib.check(L.fo_gemm_q_quant(
+        _lib.ptr(A), _lib.ptr(B), _lib.ptr(bias), _lib.ptr(out), _lib.ptr(q8), _lib.ptr(scale),
+        _lib.dtype_code(A.dtype), Bsz, M, N, A.shape[2], sparse_q_size, num_qo_heads,
         _lib.ptr(info), _lib.ptr(indptr), num_text_tokens, int(bool(is_full)),
         _lib.ptr(workspace), ws_bytes, _lib.current_stream(A.device)))
-    return out
+    return out, q8, scale
 
 
 def flashomni_gemm_reduction(

@@ -195,6 +195,21 @@ int fo_gemm_o(const void* x, const void* w, const void* bias, void* y, int dtype
               void* workspace, int64_t workspace_bytes, void* stream);
 
 /* ---------------------------------------------------------------------------------------------
+ * GEMM-Q with the fp8 quantisation of its result fused into the epilogue.
+ * No counterpart in the reference (it has no fp8 product, see fo_quant_fp8_block); for callers that
+ * feed the projection straight into fp8 attention.  As fo_gemm_q, plus: y8 [batch, m, n] e4m3fn
+ * bytes and y_scale[num_qo_heads][batch * ceil(m / 128)] fp32, written for the computed tiles only:
+ * scale = absmax of the (128-token block, head) slab of the fp32 result (bias included) / 448 (1 for
+ * an all-zero slab), y8 = rne(result / scale).  y may be NULL (the 16-bit result is then not
+ * written).  Needs n / num_qo_heads == 128.
+ * ------------------------------------------------------------------------------------------- */
+int fo_gemm_q_quant(const void* x, const void* w, const void* bias, void* y, uint8_t* y8,
+                    float* y_scale, int dtype, int32_t batch, int32_t m, int32_t n, int32_t k,
+                    int32_t sparse_q_size, int32_t num_qo_heads, const uint8_t* sparse_info,
+                    const int32_t* sparse_info_indptr, int32_t num_text_tokens, int is_full,
+                    void* workspace, int64_t workspace_bytes, void* stream);
+
+/* ---------------------------------------------------------------------------------------------
  * fp8 e4m3fn quantiser with one absmax scale per (head, 128-token block).
  * No counterpart in the reference (its quantization.cuh only packs bits).
  * x [nnz,H,D] bf16/f16 (strides in elements), x8 [nnz,H,D] bytes contiguous,

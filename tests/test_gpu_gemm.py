@@ -192,3 +192,82 @@ def test_dense_tile_enumeration_geometries(dev, shape):
                                         is_for_cache=False)
     exp = torch.matmul(a.float(), wo.float().t())       # cache + final = the full product
     assert max_abs(final.cpu(), exp) <= 4e-2 and rel_l2(final.cpu(), exp) <= REL_L2
+
+
+@pytest.mark.parametrize("shape", [(1, 512, 384, 256, 0.6), (2, 300, 256, 128, 0.7), (1, 1200, 512, 96, 1.0)])
+@pytest.mark.parametrize("write_out", [True, False])
+def test_gemm_q_with_fused_fp8_quantisation(dev, shape, write_out):
+    """GEMM-Q that also emits fp8 e4m3fn tiles + one absmax scale per (head, 128-token block).
+    The reference has no such step (parity unpinned against it); pinned by the closed form
+    scale = absmax / 448, the e4m3 rounding bound, untouched skipped tiles, and by the attention
+    kernel accepting the pair like the separate quantiser's."""
+    import flashomni_amd as fo
+    batch, m, n, k, p_active = shape
+    heads, dtype = n // 128, torch.bfloat16
+    nqb = (m + 127) // 128
+    info, packed, indptr = _flags(batch, nqb, heads, p_active, seed=m + k)
+    x, w, b = _operands(batch, m, n, k, dtype, seed=k + 1)
+    out0 = sentinel_like((batch, m, n), dtype)
+    q8_0 = torch.full((batch, m, n), 0x5A, dtype=torch.uint8)
+    sc_0 = torch.full((heads, batch * nqb), -7.0)
+    args = (x.to(dev), w.to(dev), heads, torch.from_numpy(packed).to(dev), torch.from_numpy(indptr).to(dev), 0, b.to(dev))
+    plain = fo.flashomni_gemm(*args, out=out0.clone().to(dev)).cpu()
+    q8 = q8_0.clone().to(dev).view(torch.float8_e4m3fn)
+    sc = sc_0.clone().to(dev)
+    res = fo.flashomni_gemm(*args, out=out0.clone().to(dev) if write_out else False, quant_out=(q8, sc))
+    assert res[1].data_ptr() == q8.data_ptr() and res[2].data_ptr() == sc.data_ptr()
+    if write_out:
+        assert torch.equal(res[0].cpu().view(torch.int16), plain.view(torch.int16)), "16-bit result changed"
+    else:
+        assert res[0] is None
+    # fp32 result of the flagged tiles (the oracle leaves the sentinel elsewhere)
+    ref = oracle.gemm_q(x, w, heads, packed, indptr, 0, b, out=torch.zeros(batch, m, n, dtype=torch.float32))
+    q8c, scc = q8.cpu(), sc.cpu()
+    deq_all = q8c.float()
+    for bi in range(batch):
+        for iy in range(nqb):
+            rows = slice(iy * 128, min(m, (iy + 1) * 128))
+            for h in range(heads):
+                cols = slice(h * 128, (h + 1) * 128)
+                blk = bi * nqb + iy
+                if not info[bi, iy, h]:
+                    assert torch.equal(q8c.view(torch.uint8)[bi, rows, cols], q8_0[bi, rows, cols])
+                    assert scc[h, blk] == -7.0
+                    continue
+                y = ref[bi, rows, cols].float()
+                s = float(scc[h, blk])
+                amax = float(y.abs().max())
+                assert abs(s - amax / 448.0) <= 2e-3 * amax / 448.0 + 1e-12
+                deq = deq_all[bi, rows, cols] * s
+                # e4m3: 3 mantissa bits -> half a step is 2^-4 relative; subnormal step 2^-9 of the scale
+                bound = 0.0625 * y.abs() + s * 2.0 ** -9 + 2e-3 * amax
+                assert bool(((deq - y).abs() <= bound).all())
+                assert float(deq_all[bi, rows, cols].abs().max()) == 448.0 or amax == 0.0
+    # the pair is what fp8 attention takes: against the separate quantiser on the 16-bit result
+    if write_out and batch == 1 and p_active == 1.0:
+        ws = torch.empty(64 << 20, dtype=torch.uint8, device=dev)
+        wr = fo.BatchFlashOmniFAWithRaggedKVWrapper(ws)
+        ip = torch.tensor([0, m], dtype=torch.int32)
+        wr.plan(ip, ip, heads, heads, 128, q_data_type=torch.float8_e4m3fn)
+        g = torch.Generator().manual_seed(3)
+        kk = torch.randn(m, heads, 128, generator=g).to(dtype).to(dev)
+        vv = torch.randn(m, heads, 128, generator=g).to(dtype).to(dev)
+        k8, ks = fo.quant_fp8_block(kk, ip)
+        q_sep, qs_sep = fo.quant_fp8_block(res[0].view(m, heads, 128), ip)
+        o_fused = wr.run(q8.view(m, heads, 128), k8, vv, is_full=True, q_scale=sc, k_scale=ks)
+        o_sep = wr.run(q_sep, k8, vv, is_full=True, q_scale=qs_sep, k_scale=ks)
+        assert rel_l2(o_fused.cpu(), o_sep.cpu()) <= 3e-2
+
+
+def test_gemm_q_quant_argument_errors(dev):
+    import flashomni_amd as fo
+    x = torch.zeros(1, 128, 64, dtype=torch.bfloat16, device=dev)
+    w = torch.zeros(256, 64, dtype=torch.bfloat16, device=dev)
+    with pytest.raises(RuntimeError, match="out=False needs quant_out"):
+        fo.flashomni_gemm(x, w, 2, is_full=True, out=False)
+    with pytest.raises(RuntimeError, match="only 128"):
+        fo.flashomni_gemm(x, w, 1, is_full=True, quant_out=True)       # one head of width 256
+    with pytest.raises(RuntimeError, match=r"quant_out\[1\]"):
+        fo.flashomni_gemm(x, w, 2, is_full=True,
+                          quant_out=(torch.empty(1, 128, 256, dtype=torch.float8_e4m3fn, device=dev),
+                                     torch.empty(2, 3, device=dev)))
