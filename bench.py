@@ -212,6 +212,64 @@ def bench_big_gemms(dev, index, iters, warmup):
     return res
 
 
+def bench_wan_chain(dev, iters, warmup):
+    """Config 4 end to end: GEMM-Q (fp8 result from its epilogue) -> fp8 quantisation of K -> symbol
+    decode + sparse FA (fp8 Q.K^T) -> GEMM-O final pass; and the same chain in bf16 without any
+    quantisation.  K, V drawn directly (the chain of the task has no K/V projection)."""
+    import flashomni_amd as fo
+    from flashomni_amd.workloads import make_workload
+    wl = make_workload(4, tensors=False)
+    s = wl.shape
+    g = torch.Generator(device=dev).manual_seed(3004)
+    rnd = lambda *shape: torch.randn(*shape, generator=g, device=dev, dtype=torch.float32)
+    x = rnd(1, s.seq, s.hidden).to(torch.bfloat16)
+    wq = (rnd(s.hidden, s.hidden) * 0.02).to(torch.bfloat16)
+    wo = (rnd(s.hidden, s.hidden) * 0.02).to(torch.bfloat16)
+    bq = (rnd(s.hidden) * 0.02).to(torch.bfloat16)
+    k = rnd(s.seq, s.heads, 128).to(torch.bfloat16)
+    v = rnd(s.seq, s.heads, 128).to(torch.bfloat16)
+    info, ip = wl.packed_info.to(dev), wl.info_indptr.to(dev)
+    kv_info, kv_ip = wl.packed_kv_info.to(dev), wl.kv_info_indptr.to(dev)
+    ws = torch.empty(128 << 20, dtype=torch.uint8, device=dev)
+    w8 = fo.BatchFlashOmniFAWithRaggedKVWrapper(ws)
+    w8.plan(wl.qo_indptr, wl.kv_indptr, s.heads, s.heads, 128, q_data_type=torch.float8_e4m3fn)
+    w16 = fo.BatchFlashOmniFAWithRaggedKVWrapper(ws)
+    w16.plan(wl.qo_indptr, wl.kv_indptr, s.heads, s.heads, 128, q_data_type=torch.bfloat16)
+    blocks = tuple(t.to(dev) for t in fo.token_blocks(wl.kv_indptr))
+    q8 = torch.zeros(1, s.seq, s.hidden, dtype=torch.float8_e4m3fn, device=dev)
+    q8s = torch.ones(s.heads, s.n_blocks, dtype=torch.float32, device=dev)
+    q16 = torch.zeros(1, s.seq, s.hidden, dtype=torch.bfloat16, device=dev)
+    o = torch.zeros(s.seq, s.heads, 128, dtype=torch.bfloat16, device=dev)
+    cache = fo.flashomni_gemm_reduction(o.view(1, s.seq, s.hidden), wo, s.heads, info, ip, 0, bias=None,
+                                        is_for_cache=True)
+
+    def chain_fp8():
+        fo.flashomni_gemm(x, wq, s.heads, info, ip, 0, bq, out=False, quant_out=(q8, q8s))
+        k8, ks = fo.quant_fp8_block(k, wl.kv_indptr, blocks=blocks)
+        w8._decode_key = None
+        w8.run(q8.view(s.seq, s.heads, 128), k8, v, info, kv_info, ip, kv_ip, out=o, q_scale=q8s, k_scale=ks)
+        return fo.flashomni_gemm_reduction(o.view(1, s.seq, s.hidden), wo, s.heads, info, ip, 0, bias=cache,
+                                           is_for_cache=False)
+
+    def chain_bf16():
+        fo.flashomni_gemm(x, wq, s.heads, info, ip, 0, bq, out=q16)
+        w16._decode_key = None
+        w16.run(q16.view(s.seq, s.heads, 128), k, v, info, kv_info, ip, kv_ip, out=o)
+        return fo.flashomni_gemm_reduction(o.view(1, s.seq, s.hidden), wo, s.heads, info, ip, 0, bias=cache,
+                                           is_for_cache=False)
+
+    flops = wl.gemm_q_flops() + wl.attention_flops() + wl.gemm_o_flops(False)
+    res = {}
+    y16 = chain_bf16().float()
+    y8 = chain_fp8().float()
+    res["chain_bf16"] = entry(time_gpu(chain_bf16, iters, warmup), flops=flops)
+    res["chain_fp8qk"] = entry(time_gpu(chain_fp8, iters, warmup), flops=flops)
+    res["chain_fp8qk"]["rel_l2_vs_bf16_chain"] = round(float((y8 - y16).norm() / y16.norm()), 4)
+    del x, wq, wo, k, v, q8, q16, o, cache, y8, y16
+    torch.cuda.empty_cache()
+    return res
+
+
 def cpu_baseline(layer):
     """The oracle (fp32 dense-masked CPU path) on the whole FLUX layer with the same masks:
     all active attention rows, GEMM-Q and GEMM-O final over all 36 token blocks; one warm-up pass,
@@ -360,6 +418,8 @@ def main():
             if idx == 4:
                 log("[bench] config 4 GEMMs + quantiser")
                 res.update(bench_big_gemms(dev, idx, big_iters, big_warm))
+                log("[bench] config 4 chain end to end")
+                res.update(bench_wan_chain(dev, big_iters, big_warm))
             kernels[SHAPES[idx].name] = res
             log("[bench]", SHAPES[idx].name, json.dumps(res))
 

@@ -404,17 +404,25 @@ __global__ void __launch_bounds__(kThreads) sparse_fa_kernel(const FaParams p) {
     x8 qreg[kFp8 ? 1 : 8];
     i32x8 qreg8[kFp8 ? 2 : 1];
     const uint32_t lds_group = static_cast<uint32_t>(reinterpret_cast<uintptr_t>((lds_void*)group_smem));
-    {
+    if constexpr (kFp8) {
+      // (fp8 Q, half the bytes, is still fetched directly: with the LDS detour hipcc arranges the
+      // main loop of this instantiation less well, which costs more than the detour saves)
+      const uint8_t* src = qp + q_tok * p.q_sn + static_cast<int64_t>(head) * p.q_sh + g * 32;
+#pragma unroll
+      for (int sl = 0; sl < 2; ++sl) {
+        const i32x4 lo = *reinterpret_cast<const i32x4*>(src + sl * 64);
+        const i32x4 hi = *reinterpret_cast<const i32x4*>(src + sl * 64 + 16);
+        qreg8[sl] = i32x8{lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
+      }
+    } else {
       const uint8_t* q_head = reinterpret_cast<const uint8_t*>(
           qp + static_cast<int64_t>(q_begin) * p.q_sn + static_cast<int64_t>(head) * p.q_sh);
       const uint32_t qdst = lds_group + kStageBytes + kKBytes + qs * 1024;
 #pragma unroll
-      for (int n = 0; n < (kFp8 ? 2 : 4); ++n) {
-        int r = kg * 64 + (kFp8 ? 8 * (4 * n + qs) + cp8_row : 4 * (4 * n + qs) + cp_row);
+      for (int n = 0; n < 4; ++n) {
+        int r = kg * 64 + 4 * (4 * n + qs) + cp_row;
         r = r < q_rows ? r : q_rows - 1;  // ragged last q block: re-read the last row
-        const uint32_t off = kFp8 ? static_cast<uint32_t>(r * p.q_sn + cp8_chunk)
-                                  : static_cast<uint32_t>((r * p.q_sn + cp_chunk) * sizeof(T));
-        copy16_to_lds(q_head, off, qdst + n * 4096);
+        copy16_to_lds(q_head, static_cast<uint32_t>((r * p.q_sn + cp_chunk) * sizeof(T)), qdst + n * 4096);
       }
     }
     // (the row's kv block list is in LDS already: the main loop has no global loads besides the
@@ -555,35 +563,28 @@ __global__ void __launch_bounds__(kThreads) sparse_fa_kernel(const FaParams p) {
     }
     // Q has landed once only the tile copies issued after it are outstanding; then for every
     // wavefront after the barrier
-    if (my_tiles > 1) {
-      __builtin_amdgcn_s_waitcnt(0x0f70 | (2 * kKCopies + kVCopies));
-    } else if (my_tiles == 1) {
-      __builtin_amdgcn_s_waitcnt(0x0f70 | (kKCopies + kVCopies));
-    } else {
-      __builtin_amdgcn_s_waitcnt(0x0f70);
+    if constexpr (!kFp8) {
+      if (my_tiles > 1) {
+        __builtin_amdgcn_s_waitcnt(0x0f70 | (2 * kKCopies + kVCopies));
+      } else if (my_tiles == 1) {
+        __builtin_amdgcn_s_waitcnt(0x0f70 | (kKCopies + kVCopies));
+      } else {
+        __builtin_amdgcn_s_waitcnt(0x0f70);
+      }
     }
     __builtin_amdgcn_s_barrier();
     // Q from LDS while the first tile copies are in flight: rows (qs % 2) * 32 + l32 of the tile that
     // kv group qs / 2 copied, addressed like a K operand
-    {
-      const uint8_t* qt = smem + (qs >> 1) * kGroupBytes + kStageBytes + kKBytes +
-                          (qs & 1) * 32 * (kFp8 ? kRowBytes8 : kRowBytes) + k_rd_base;
-      if constexpr (kFp8) {
+    if constexpr (!kFp8) {
+      const uint8_t* qt = smem + (qs >> 1) * kGroupBytes + kStageBytes + kKBytes + (qs & 1) * 32 * kRowBytes +
+                          k_rd_base;
 #pragma unroll
-        for (int sl = 0; sl < 2; ++sl) {
-          const i32x4 lo = *reinterpret_cast<const i32x4*>(qt + (k_rd_x ^ (sl << 6)));
-          const i32x4 hi = *reinterpret_cast<const i32x4*>(qt + ((k_rd_x ^ (sl << 6)) ^ 16));
-          qreg8[sl] = i32x8{lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
-        }
-      } else {
+      for (int ks = 0; ks < 8; ++ks) qreg[ks] = *reinterpret_cast<const x8*>(qt + (k_rd_x ^ (ks << 5)));
+      // the softmax scale (log2 domain) is folded into Q, so S^T needs no multiply
 #pragma unroll
-        for (int ks = 0; ks < 8; ++ks) qreg[ks] = *reinterpret_cast<const x8*>(qt + (k_rd_x ^ (ks << 5)));
-        // the softmax scale (log2 domain) is folded into Q, so S^T needs no multiply
+      for (int ks = 0; ks < 8; ++ks)
 #pragma unroll
-        for (int ks = 0; ks < 8; ++ks)
-#pragma unroll
-          for (int e = 0; e < 8; ++e) qreg[ks][e] = static_cast<T>(static_cast<float>(qreg[ks][e]) * c);
-      }
+        for (int e = 0; e < 8; ++e) qreg[ks][e] = static_cast<T>(static_cast<float>(qreg[ks][e]) * c);
     }
     // (every wavefront holds its Q before the first barrier: the V copies of tile 1 overwrite it after)
     __builtin_amdgcn_s_waitcnt(0xc07f);  // lgkmcnt(0)
