@@ -202,9 +202,8 @@ class BatchFlashOmniFAWithRaggedKVWrapper:
             raise NotImplementedError(
                 "positional encoding, logits soft cap and fp16 logits are not part of the sparse "
                 "prefill path")
-        if num_qo_heads != num_kv_heads:
-            raise NotImplementedError("grouped-query attention (num_qo_heads != num_kv_heads) is not "
-                                      "supported by the sparse prefill path")
+        if num_kv_heads <= 0 or num_qo_heads % num_kv_heads != 0:
+            raise ValueError("num_qo_heads must be a multiple of num_kv_heads")
         if head_dim_qk != 128 or head_dim_vo != 128:
             raise NotImplementedError("only head_dim 128 is supported")
         if sparse_block_size_for_q != 128 or sparse_block_size_for_kv != 128:
@@ -288,6 +287,7 @@ class BatchFlashOmniFAWithRaggedKVWrapper:
         self._decode_key = None
 
         self._num_qo_heads = num_qo_heads
+        self._num_kv_heads = num_kv_heads
         self._sparse_block_size_for_q = sparse_block_size_for_q
         self._sparse_block_size_for_kv = sparse_block_size_for_kv
         self._causal = causal
@@ -416,6 +416,9 @@ class BatchFlashOmniFAWithRaggedKVWrapper:
             raise ValueError(f"Invalid device of q: expected {self.device}, got {q.device}")
         if q.size(1) != self._num_qo_heads or q.size(2) != 128:
             raise ValueError("q does not match the head count / head_dim given to plan()")
+        kv_head_dim = 1 if self._kv_layout == "NHD" else 0
+        if k.size(kv_head_dim) != self._num_kv_heads or v.size(kv_head_dim) != self._num_kv_heads:
+            raise ValueError("k / v do not match the kv head count given to plan()")
         for name, t in (("q", q), ("k", k), ("v", v), ("out", out)):
             if t.stride(-1) != 1:
                 raise ValueError(f"{name} must have a contiguous last dimension")
@@ -430,8 +433,10 @@ class BatchFlashOmniFAWithRaggedKVWrapper:
         if fp8:
             q_scale = q_scale.to(torch.float32).contiguous()
             k_scale = k_scale.to(torch.float32).contiguous()
-            if q_scale.shape != (q.size(1), self._n_q_blk) or k_scale.shape != (q.size(1), self._n_kv_blk):
-                raise ValueError("q_scale / k_scale must be [H, number of 128-token blocks]")
+            if q_scale.shape != (q.size(1), self._n_q_blk) or \
+                    k_scale.shape != (self._num_kv_heads, self._n_kv_blk):
+                raise ValueError("q_scale / k_scale must be [H, number of 128-token blocks] "
+                                 "(k_scale: one row per kv head)")
         _lib.check(_lib.lib().fo_sparse_fa_run(
             _lib.ptr(q), _lib.ptr(k), _lib.ptr(v), _lib.ptr(out), _lib.ptr(lse if return_lse else None),
             _lib.dtype_code(q.dtype), _lib.ptr(q_scale if fp8 else None),
@@ -441,7 +446,8 @@ class BatchFlashOmniFAWithRaggedKVWrapper:
             _lib.ptr(self._kv_blk_base), self._n_q_blk, self._n_kv_blk, _lib.ptr(wl.row_req),
             _lib.ptr(wl.row_qb),
             _lib.ptr(wl.row_head), _lib.ptr(wl.kv_row_ptr), _lib.ptr(wl.kv_idx), _lib.ptr(wl.order),
-            _lib.ptr(wl.sched), self._max_rows, q.size(1), q.size(2), self._sparse_block_size_for_q,
+            _lib.ptr(wl.sched), self._max_rows, q.size(1), self._num_kv_heads, q.size(2),
+            self._sparse_block_size_for_q,
             self._sparse_block_size_for_kv, float(sm_scale),
             _lib.ptr(self._float_workspace_buffer) if self._split_ws_ok() else None,
             self._float_ws_bytes(), _lib.current_stream(self.device)))

@@ -118,6 +118,7 @@ struct FaParams {
   int32_t* sched;
   float* split_ws;  // partial results of rows whose kv list is split over workgroups (or null)
   int32_t num_heads;
+  int32_t kv_group;  // q heads per kv head (grouped-query attention); 1 = one kv head per q head
   int32_t n_q_blocks, n_kv_blocks;  // row lengths of q_scale / k_scale
   float sm_scale_log2;
 };
@@ -437,7 +438,8 @@ __global__ void __launch_bounds__(kThreads) sparse_fa_kernel(const FaParams p) {
     float cq = c;
     if constexpr (kFp8) cq *= p.q_scale[static_cast<int64_t>(head) * p.n_q_blocks + p.q_blk_base[req] + qb];
     const float* ksc = nullptr;
-    if constexpr (kFp8) ksc = p.k_scale + static_cast<int64_t>(head) * p.n_kv_blocks + p.kv_blk_base[req];
+    const int kv_head = head / p.kv_group;
+    if constexpr (kFp8) ksc = p.k_scale + static_cast<int64_t>(kv_head) * p.n_kv_blocks + p.kv_blk_base[req];
 
     f32x16 o_acc[4];
 #pragma unroll
@@ -462,8 +464,8 @@ __global__ void __launch_bounds__(kThreads) sparse_fa_kernel(const FaParams p) {
     //   K of tile j+2 at the start of the VALU block of tile j   (K of tile j was consumed by S(j))
     //   V of tile j+1 during the MFMA block of tile j            (V of tile j-1 is in registers)
     // so a K copy has about two block periods to land and a V copy more than one.
-    const TQK* k_head = kp + static_cast<int64_t>(kv_begin) * p.k_sn + static_cast<int64_t>(head) * p.k_sh;
-    const T* v_head = vp + static_cast<int64_t>(kv_begin) * p.v_sn + static_cast<int64_t>(head) * p.v_sh;
+    const TQK* k_head = kp + static_cast<int64_t>(kv_begin) * p.k_sn + static_cast<int64_t>(kv_head) * p.k_sh;
+    const T* v_head = vp + static_cast<int64_t>(kv_begin) * p.v_sn + static_cast<int64_t>(kv_head) * p.v_sh;
     // lane offsets of copy instruction 0; instruction n adds a uniform 16 (fp8 K: 32) rows
     const uint32_t v_voff = static_cast<uint32_t>((4 * qs + cp_row) * p.v_sn + cp_chunk) * sizeof(T);
     const uint32_t k_voff = kFp8 ? static_cast<uint32_t>((8 * qs + cp8_row) * p.k_sn + cp8_chunk)
@@ -1029,7 +1031,7 @@ extern "C" int fo_sparse_fa_run(const void* q, const void* k, const void* v, voi
                                 const int32_t* row_qb, const int32_t* row_head,
                                 const int32_t* kv_row_ptr, const int32_t* kv_idx,
                                 const int32_t* order, int32_t* sched, int64_t max_rows,
-                                int32_t num_heads, int32_t head_dim, int32_t block_q,
+                                int32_t num_heads, int32_t num_kv_heads, int32_t head_dim, int32_t block_q,
                                 int32_t block_kv, float sm_scale, void* split_workspace,
                                 int64_t split_workspace_bytes, void* stream) {
   FO_REQUIRE(head_dim == kHeadDim, "sparse_fa: head_dim %d is not supported (only 128)", head_dim);
@@ -1039,6 +1041,8 @@ extern "C" int fo_sparse_fa_run(const void* q, const void* k, const void* v, voi
   FO_REQUIRE(dtype == FO_BF16 || dtype == FO_F16 || dtype == FO_FP8_E4M3,
              "sparse_fa: unsupported dtype code %d", dtype);
   FO_REQUIRE(num_heads > 0 && max_rows >= 0, "sparse_fa: bad sizes");
+  FO_REQUIRE(num_kv_heads > 0 && num_heads % num_kv_heads == 0,
+             "sparse_fa: num_qo_heads %d is not a multiple of num_kv_heads %d", num_heads, num_kv_heads);
   if (max_rows == 0) return FO_OK;
   FO_REQUIRE(q && k && v && o && qo_indptr && kv_indptr && row_req && row_qb && row_head &&
                  kv_row_ptr && kv_idx && order && sched,
@@ -1074,7 +1078,7 @@ extern "C" int fo_sparse_fa_run(const void* q, const void* k, const void* v, voi
                "sparse_fa: split_workspace must be 16-byte aligned");
     p.split_ws = static_cast<float*>(split_workspace);
   }
-  p.num_heads = num_heads; p.n_q_blocks = n_q_blocks; p.n_kv_blocks = n_kv_blocks;
+  p.num_heads = num_heads; p.kv_group = num_heads / num_kv_heads; p.n_q_blocks = n_q_blocks; p.n_kv_blocks = n_kv_blocks;
   p.sm_scale_log2 = sm_scale * 1.44269504088896340736f;
   hipStream_t s = static_cast<hipStream_t>(stream);
   if (dtype == FO_BF16) return launch<__bf16, false>(p, max_rows, s);

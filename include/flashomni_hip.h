@@ -124,8 +124,9 @@ int fo_decode_sparse(const uint8_t* sparse_info, const uint8_t* sparse_kv_info,
  *           include/flashomni/attention/prefill.cuh:1203-1531 (mask none, no positional
  *           encoding, fp32 logits: the only variant the reference builds, setup.py:98-111).
  *
- * q [nnz_q,H,D], k,v [nnz_kv,H,D], o [nnz_q,H,D]; strides in elements (the innermost stride is
- * 1).  dtype FO_BF16 / FO_F16: q,k,v,o share it.  dtype FO_FP8_E4M3: q and k are e4m3fn bytes
+ * q [nnz_q,H,D], k,v [nnz_kv,H_kv,D], o [nnz_q,H,D]; strides in elements (the innermost stride is
+ * 1).  num_heads = H must be a multiple of num_kv_heads = H_kv: q head h reads kv head
+ * h / (H / H_kv) (grouped-query attention, prefill.cuh:410-413); k_scale then has H_kv rows.  dtype FO_BF16 / FO_F16: q,k,v,o share it.  dtype FO_FP8_E4M3: q and k are e4m3fn bytes
  * with dequantisation scales q_scale[H][n_q_blocks], k_scale[H][n_kv_blocks] (fp32, blocks
  * numbered request by request: q_blk_base / kv_blk_base [batch+1] give each request's first
  * block); v and o are bf16.  (The fp8 form has no counterpart in the reference.)
@@ -151,7 +152,7 @@ int fo_sparse_fa_run(const void* q, const void* k, const void* v, void* o, float
                      const int32_t* q_blk_base, const int32_t* kv_blk_base, int32_t n_q_blocks,
                      int32_t n_kv_blocks, const int32_t* row_req, const int32_t* row_qb, const int32_t* row_head,
                      const int32_t* kv_row_ptr, const int32_t* kv_idx, const int32_t* order,
-                     int32_t* sched, int64_t max_rows, int32_t num_heads, int32_t head_dim,
+                     int32_t* sched, int64_t max_rows, int32_t num_heads, int32_t num_kv_heads, int32_t head_dim,
                      int32_t block_q, int32_t block_kv, float sm_scale, void* split_workspace,
                      int64_t split_workspace_bytes, void* stream);
 

@@ -33,6 +33,7 @@ def sparse_attention(q, k, v, sparse_info, sparse_kv_info, sparse_info_indptr,
     q_scale/k_scale: optional fp32 [H, n_blocks] dequantisation scales for fp8 q/k
     (no reference counterpart)."""
     H, D = q.shape[1], q.shape[2]
+    group = H // k.shape[1]   # q heads per kv head (prefill.cuh:410-413); 1 without grouped-query attention
     if sm_scale is None:
         sm_scale = 1.0 / math.sqrt(D)
     out_dtype = q.dtype if q.dtype in (torch.float16, torch.bfloat16, torch.float32) else torch.bfloat16
@@ -64,13 +65,13 @@ def sparse_attention(q, k, v, sparse_info, sparse_kv_info, sparse_info_indptr,
                               for b in kept])
         tok_t = torch.from_numpy(tok)
         qf = q[q0:q1, h].float()
-        kf = k[tok_t, h].float()
-        vf = v[tok_t, h].float()
+        kf = k[tok_t, h // group].float()
+        vf = v[tok_t, h // group].float()
         if q_scale is not None:
             qf = qf * float(q_scale[h, int(q_blk_base[r]) + qb])
         if k_scale is not None:
             blk = torch.from_numpy((tok - kv0) // block_kv + int(kv_blk_base[r]))
-            kf = kf * k_scale[h][blk].float()[:, None]
+            kf = kf * k_scale[h // group][blk].float()[:, None]
         s = qf @ kf.T
         m = s.max(dim=-1, keepdim=True).values
         p = torch.exp2((s - m) * c)

@@ -330,3 +330,38 @@ def test_shared_rows_fp8(dev):
         parts = w._worklist.sched.cpu().numpy()[40:42]
         assert (parts == (4 if share else 1)).all()
     assert max_abs(outs[0], outs[1]) <= 8e-3
+
+
+@pytest.mark.parametrize("heads", [(4, 2), (6, 1), (8, 8)])
+@pytest.mark.parametrize("layout", ["NHD", "HND"])
+def test_grouped_query_attention(dev, heads, layout):
+    """num_kv_heads < num_qo_heads: q head h reads kv head h / group (prefill.cuh:410-413)."""
+    import flashomni_amd as fo
+    hq, hkv = heads
+    ql, kl = [300, 1, 640], [77, 513, 640]
+    m = make_ragged_masks(ql, kl, hq, 0.8, 0.5, seed=41)
+    g = torch.Generator().manual_seed(41)
+    nq, nk = sum(ql), sum(kl)
+    q = torch.randn(nq, hq, 128, generator=g).to(torch.bfloat16)
+    k = torch.randn(nk, hkv, 128, generator=g).to(torch.bfloat16)
+    v = torch.randn(nk, hkv, 128, generator=g).to(torch.bfloat16)
+    t = lambda a: torch.from_numpy(a).to(dev)
+    w = fo.BatchFlashOmniFAWithRaggedKVWrapper(torch.empty(256 << 20, dtype=torch.uint8, device=dev), layout)
+    w.plan(t(m["qo_indptr"]), t(m["kv_indptr"]), hq, hkv, 128, q_data_type=torch.bfloat16)
+    kd, vd = k.to(dev), v.to(dev)
+    if layout == "HND":
+        kd, vd = kd.transpose(0, 1).contiguous(), vd.transpose(0, 1).contiguous()
+    out0 = sentinel_like((nq, hq, 128), torch.bfloat16)
+    out, lse = w.run(q.to(dev), kd, vd, t(m["packed_info"]), t(m["packed_keep"]), t(m["info_indptr"]),
+                     t(m["keep_indptr"]), out=out0.clone().to(dev), return_lse=True)
+    exp_lse = torch.full((nq, hq), float("nan"))
+    exp = oracle.sparse_attention(q, k, v, m["packed_info"], m["packed_keep"], m["info_indptr"],
+                                  m["keep_indptr"], m["qo_indptr"], m["kv_indptr"], out=out0.clone(), lse=exp_lse)
+    _check(out.cpu(), exp, out0, m, hq)
+    ok = ~torch.isnan(exp_lse)
+    assert torch.allclose(lse.cpu()[ok], exp_lse[ok], atol=2e-3, rtol=1e-3)
+    with pytest.raises(ValueError, match="kv head count"):
+        w.run(q.to(dev), torch.zeros(nk, hkv + 1, 128, dtype=torch.bfloat16, device=dev).transpose(0, 1 if layout == "HND" else 0),
+              vd, t(m["packed_info"]), t(m["packed_keep"]), t(m["info_indptr"]), t(m["keep_indptr"]))
+    with pytest.raises(ValueError, match="multiple of num_kv_heads"):
+        w.plan(t(m["qo_indptr"]), t(m["kv_indptr"]), 6, 4, 128, q_data_type=torch.bfloat16)
