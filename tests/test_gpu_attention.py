@@ -365,3 +365,50 @@ def test_grouped_query_attention(dev, heads, layout):
               vd, t(m["packed_info"]), t(m["packed_keep"]), t(m["info_indptr"]), t(m["keep_indptr"]))
     with pytest.raises(ValueError, match="multiple of num_kv_heads"):
         w.plan(t(m["qo_indptr"]), t(m["kv_indptr"]), 6, 4, 128, q_data_type=torch.bfloat16)
+
+
+@pytest.mark.parametrize("config", [3, 4])
+def test_video_shapes_sampled_rows(dev, config):
+    """Configs 3 and 4 at full size (H=40, seq 17776 and 76112, ragged last block): the kernel runs
+    the whole work list; every row of the first and last q-block plus 64 seeded random rows are
+    checked against the oracle, and skipped (q-block, head) strips keep their bytes."""
+    import flashomni_amd as fo
+    from flashomni_amd.workloads import make_workload
+    wl = make_workload(config, tensors=False)
+    s = wl.shape
+    g = torch.Generator(device=dev).manual_seed(100 + config)
+    draw = lambda: torch.randn(s.seq, s.heads, 128, generator=g, device=dev, dtype=torch.float32).to(torch.bfloat16)
+    q, k, v = draw(), draw(), draw()
+    out = torch.full((s.seq, s.heads, 128), -7.0, dtype=torch.bfloat16, device=dev)
+    w = fo.BatchFlashOmniFAWithRaggedKVWrapper(torch.empty(256 << 20, dtype=torch.uint8, device=dev))
+    w.plan(wl.qo_indptr, wl.kv_indptr, s.heads, s.heads, 128, q_data_type=torch.bfloat16)
+    w.run(q, k, v, wl.packed_info.to(dev), wl.packed_kv_info.to(dev), wl.info_indptr.to(dev),
+          wl.kv_info_indptr.to(dev), out=out)
+    torch.cuda.synchronize()
+
+    active = wl.sparse_info.to(dev).repeat_interleave(128, dim=0)[:s.seq]      # [seq, H]
+    assert bool((out[~active] == -7.0).all())
+    assert bool(torch.isfinite(out[active].float()).all())
+
+    _, row_qb, row_head, ptr, _ = oracle.decode_kv_csr(
+        wl.packed_info.numpy(), wl.packed_kv_info.numpy(), wl.info_indptr.numpy(),
+        wl.kv_info_indptr.numpy(), wl.qo_indptr.numpy(), wl.kv_indptr.numpy(), s.heads, 128, 128)
+    edge = np.nonzero((row_qb == 0) | (row_qb == s.n_blocks - 1))[0]
+    rng = np.random.default_rng(config)
+    rows = np.unique(np.concatenate([edge, rng.choice(len(row_qb), 64, replace=False)]))
+    assert (row_qb[rows] == s.n_blocks - 1).any()                              # the short block is covered
+    exp = torch.full((s.seq, s.heads, 128), -7.0, dtype=torch.bfloat16)
+    oracle.sparse_attention(q.cpu(), k.cpu(), v.cpu(), wl.packed_info, wl.packed_kv_info,
+                            wl.info_indptr, wl.kv_info_indptr, wl.qo_indptr, wl.kv_indptr,
+                            out=exp, rows=[int(i) for i in rows])
+    got = out.cpu()
+    worst_abs, num, den = 0.0, 0.0, 0.0
+    for i in rows:
+        q0 = int(row_qb[i]) * 128
+        sl = (slice(q0, min(s.seq, q0 + 128)), int(row_head[i]))
+        a, b = got[sl].float(), exp[sl].float()
+        worst_abs = max(worst_abs, float((a - b).abs().max()))
+        num += float(((a - b) ** 2).sum())
+        den += float((b ** 2).sum())
+    assert worst_abs <= MAX_ABS
+    assert math.sqrt(num / den) <= REL_L2

@@ -271,3 +271,50 @@ def test_gemm_q_quant_argument_errors(dev):
         fo.flashomni_gemm(x, w, 2, is_full=True,
                           quant_out=(torch.empty(1, 128, 256, dtype=torch.float8_e4m3fn, device=dev),
                                      torch.empty(2, 3, device=dev)))
+
+
+def test_video_gemms_sampled_token_blocks(dev):
+    """The 14B-video shape at full size (M=76112 with an 80-row last block, K=N=5120, 40 heads):
+    GEMM-Q, the GEMM-O cache pass and the final pass run over the whole matrix; the first, the last
+    and 10 seeded random token blocks are checked against the oracle, which is run on each block's
+    rows alone with the text-token offset that makes it read that block's flags.  The oracle keeps
+    fp32 outputs, so the bound covers the kernel's one bf16 rounding (outputs stay below 4)."""
+    import flashomni_amd as fo
+    from flashomni_amd.workloads import make_workload
+    wl = make_workload(4, tensors=False)
+    s = wl.shape
+    M, C, H = s.seq, s.hidden, s.heads
+    g = torch.Generator(device=dev).manual_seed(41)
+    rand = lambda *sz, std=1.0: (torch.randn(*sz, generator=g, device=dev) * std).to(torch.bfloat16)
+    x, w_q, b_q, w_o, b_o = rand(1, M, C), rand(C, C, std=0.01), rand(C, std=0.02), rand(C, C, std=0.01), rand(C, std=0.02)
+    pk, ip = wl.packed_info.to(dev), wl.info_indptr.to(dev)
+    y = torch.full((1, M, C), -7.0, dtype=torch.bfloat16, device=dev)
+    fo.flashomni_gemm(x, w_q, H, pk, ip, 0, b_q, out=y)
+    active = wl.sparse_info.to(dev).repeat_interleave(128, 0)[:M].repeat_interleave(128, 1)[None]
+    assert bool((y[~active] == -7.0).all())
+    del active
+    cache = fo.flashomni_gemm_reduction(x, w_o, H, pk, ip, 0, bias=b_o, is_for_cache=True,
+                                        out_dtype=torch.float32)
+    final = fo.flashomni_gemm_reduction(x, w_o, H, pk, ip, 0, bias=cache, is_for_cache=False)
+    torch.cuda.synchronize()
+
+    rng = np.random.default_rng(4)
+    blocks = sorted({0, s.n_blocks - 1, *rng.choice(s.n_blocks, 10, replace=False).tolist()})
+    wq_c, bq_c, wo_c, bo_c = w_q.cpu(), b_q.cpu(), w_o.cpu(), b_o.cpu()
+    for iy in blocks:
+        r0, r1 = iy * 128, min(M, iy * 128 + 128)
+        xs = x[:, r0:r1].cpu()
+        exp = oracle.gemm_q(xs, wq_c, H, wl.packed_info, wl.info_indptr, r0, bq_c,
+                            out=torch.full((1, r1 - r0, C), -7.0, dtype=torch.float32))
+        got = y[:, r0:r1].cpu()
+        assert max_abs(got, exp) <= MAX_ABS, iy
+        assert rel_l2(got, exp) <= REL_L2, iy
+        exp_cache = oracle.gemm_o(xs, wo_c, H, wl.packed_info, wl.info_indptr, r0, bias=bo_c,
+                                  is_for_cache=True, out_dtype=torch.float32)
+        got_cache = cache[:, r0:r1].cpu()
+        assert max_abs(got_cache, exp_cache) <= 2e-3, iy
+        exp_final = oracle.gemm_o(xs, wo_c, H, wl.packed_info, wl.info_indptr, r0, bias=exp_cache,
+                                  is_for_cache=False, out_dtype=torch.float32)
+        got_final = final[:, r0:r1].cpu()
+        assert max_abs(got_final, exp_final) <= MAX_ABS, iy
+        assert rel_l2(got_final, exp_final) <= REL_L2, iy
