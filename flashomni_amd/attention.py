@@ -280,6 +280,14 @@ class BatchFlashOmniFAWithRaggedKVWrapper:
         self._q_blk_base = q_base.to(torch.int32).to(self.device)
         self._kv_blk_base = kv_base.to(torch.int32).to(self.device)
         self._n_kv_blk = int(kv_base[-1])
+        # sizes the tensors given to run() must have (checked there without reading the device):
+        # token counts, and the packed bytes of the byte-aligned per-request segments
+        self._total_q_rows = total_num_rows
+        self._total_kv_rows = int(kv_indptr_host[-1]) if kv_indptr_host.numel() else 0
+        nqb = q_base[1:] - q_base[:-1]
+        nkb = kv_base[1:] - kv_base[:-1]
+        self._min_info_bytes = int(((nqb * num_qo_heads + 7) // 8).sum())
+        self._min_kv_info_bytes = int(((nqb * nkb * num_qo_heads + 7) // 8).sum())
         if (self._worklist is None or self._worklist.max_rows < max_rows
                 or self._worklist.max_nnz < max_nnz):
             self._worklist = DecodedWorkList(max_rows, max_nnz, num_qo_heads, self.device)
@@ -339,6 +347,14 @@ class BatchFlashOmniFAWithRaggedKVWrapper:
                 if t.device != self.device:
                     raise ValueError(f"Invalid device of {name}: expected {self.device}, got {t.device}")
                 tensors.append(t.to(dt).contiguous())
+            for name, t, need in (("sparse_info", tensors[0], self._min_info_bytes),
+                                  ("sparse_kv_info", tensors[1], self._min_kv_info_bytes)):
+                if t.numel() < need:
+                    raise ValueError(f"{name} holds {t.numel()} bytes; the planned batch needs {need}")
+            n_req = self._qo_indptr_buf.numel() - 1
+            for name, t in (("sparse_info_indptr", tensors[2]), ("sparse_kv_info_indptr", tensors[3])):
+                if t.numel() != n_req + 1:
+                    raise ValueError(f"{name} must have {n_req + 1} entries, got {t.numel()}")
             key = tuple((t.data_ptr(), t._version, t.numel()) for t in
                         (sparse_info, sparse_kv_info, sparse_info_indptr, sparse_kv_info_indptr))
         else:
@@ -391,6 +407,8 @@ class BatchFlashOmniFAWithRaggedKVWrapper:
         """
         if self._plan_info is None:
             raise RuntimeError("plan() must be called before run()")
+        if q.dim() != 3 or k.dim() != 3 or v.dim() != 3 or k.size(2) != 128 or v.size(2) != 128:
+            raise ValueError("q, k and v must be 3-dimensional with head_dim 128")
         _check_cached_qkv_data_type(q, k, self._cached_q_data_type, self._cached_kv_data_type)
         sm_scale = self._sm_scale
         if sm_scale is None:
@@ -419,6 +437,12 @@ class BatchFlashOmniFAWithRaggedKVWrapper:
         kv_head_dim = 1 if self._kv_layout == "NHD" else 0
         if k.size(kv_head_dim) != self._num_kv_heads or v.size(kv_head_dim) != self._num_kv_heads:
             raise ValueError("k / v do not match the kv head count given to plan()")
+        n_kv = min(k.size(1 - kv_head_dim), v.size(1 - kv_head_dim))
+        if q.size(0) < self._total_q_rows or n_kv < self._total_kv_rows:
+            raise ValueError(f"q / k, v hold {q.size(0)} / {n_kv} tokens; the planned "
+                             f"batch has {self._total_q_rows} / {self._total_kv_rows}")
+        if return_lse and not lse.is_contiguous():
+            raise ValueError("lse must be contiguous")
         for name, t in (("q", q), ("k", k), ("v", v), ("out", out)):
             if t.stride(-1) != 1:
                 raise ValueError(f"{name} must have a contiguous last dimension")

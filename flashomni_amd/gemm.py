@@ -22,11 +22,27 @@ def _check_gemm_operands(A: torch.Tensor, B: torch.Tensor, name: str):
         raise RuntimeError(f"{name}: A and B must be contiguous")
 
 
-def _symbols(sparse_info, sparse_info_indptr, device):
+def _symbols(sparse_info, sparse_info_indptr, device, name, batch, m, num_qo_heads,
+             num_text_tokens, sparse_q_size):
+    """Packed symbols and their byte offsets on ``device``.  The kernels read bit
+    ``((num_text_tokens + row) // sparse_q_size) * num_qo_heads + head`` of a request's segment, so
+    a segment shorter than the last such bit is refused here (the offsets themselves live on the
+    device and are not read back)."""
     if sparse_info is None:
         return None, None
+    if sparse_info_indptr is None:
+        raise RuntimeError(f"{name}: sparse_info needs sparse_info_indptr")
     info = sparse_info.to(device=device, dtype=torch.uint8).contiguous()
     indptr = sparse_info_indptr.to(device=device, dtype=torch.int32).contiguous()
+    if indptr.numel() != batch + 1:
+        raise RuntimeError(f"{name}: sparse_info_indptr must have batch + 1 = {batch + 1} entries, "
+                           f"got {indptr.numel()}")
+    if m > 0:
+        last_block = (num_text_tokens + m - 1) // sparse_q_size
+        need = ((last_block + 1) * num_qo_heads + 7) // 8
+        if info.numel() < need:
+            raise RuntimeError(f"{name}: sparse_info holds {info.numel()} bytes, a request needs {need} "
+                               f"({last_block + 1} token blocks x {num_qo_heads} heads)")
     return info, indptr
 
 
@@ -70,7 +86,12 @@ def flashomni_gemm(
         if bias.dtype != A.dtype or bias.numel() != B.shape[0] or bias.device != A.device:
             raise RuntimeError("flashomni_gemm: bias must be [N] with A's dtype on A's device")
         bias = bias.contiguous()
-    info, indptr = _symbols(sparse_info, sparse_info_indptr, A.device)
+    if num_qo_heads <= 0 or B.shape[0] % num_qo_heads != 0 or num_text_tokens < 0 or sparse_q_size <= 0:
+        raise RuntimeError("flashomni_gemm: N must be a multiple of num_qo_heads; num_text_tokens >= 0; "
+                           "sparse_q_size > 0")
+    info, indptr = (None, None) if is_full else _symbols(
+        sparse_info, sparse_info_indptr, A.device, "flashomni_gemm", A.shape[0], A.shape[1],
+        num_qo_heads, num_text_tokens, sparse_q_size)
     if not is_full and info is None:
         raise RuntimeError("flashomni_gemm: sparse_info is required unless is_full=True")
     L = _lib.lib()
@@ -149,7 +170,11 @@ def flashomni_gemm_reduction(
             kind = _lib.FO_BIAS_MATRIX
             bias_code = _lib.dtype_code(bias.dtype)
         bias = bias.contiguous()
-    info, indptr = _symbols(sparse_info, sparse_info_indptr, A.device)
+    if num_qo_heads <= 0 or num_text_tokens < 0 or sparse_q_size <= 0:
+        raise RuntimeError("flashomni_gemm_reduction: num_qo_heads > 0, num_text_tokens >= 0 and "
+                           "sparse_q_size > 0 are required")
+    info, indptr = _symbols(sparse_info, sparse_info_indptr, A.device, "flashomni_gemm_reduction",
+                            Bsz, M, num_qo_heads, num_text_tokens, sparse_q_size)
     L = _lib.lib()
     workspace, ws_bytes = None, 0  # the reduction visits every token block: no tile list
     _lib.check(L.fo_gemm_o(

@@ -2,7 +2,7 @@
 
 The reference shows the procedure as a script (benchmark/test_attn_score.py:93-160: torch sort,
 cumsum and searchsorted, then Triton kernels that clear the selected entries of uint8 maps, which
-benchmark/test_flashomni_attention.py:254-257 transposes and packs).  Here one HIP launch pair goes
+benchmark/test_flashomni_attention.py:254-257 transposes and packs).  Here one HIP launch goes
 from the scores to the packed bits.
 """
 from typing import Optional, Tuple, Union

@@ -163,6 +163,35 @@ def test_dtype_mismatch_and_missing_symbols_raise(dev):
         w.run(q, q, q, is_full=True, out=torch.zeros(64, 1, 128, device=dev, dtype=torch.bfloat16))
 
 
+def test_undersized_tensors_raise(dev):
+    """Tensors smaller than the planned batch are refused on the host: the kernels index by the
+    planned token counts and symbol layout."""
+    import flashomni_amd as fo
+    w = fo.BatchFlashOmniFAWithRaggedKVWrapper(torch.empty(128 << 20, dtype=torch.uint8, device=dev))
+    qo = torch.tensor([0, 300, 556], dtype=torch.int32, device=dev)      # 3 + 2 q blocks
+    kv = torch.tensor([0, 256, 700], dtype=torch.int32, device=dev)      # 2 + 4 kv blocks
+    w.plan(qo, kv, 4, 4, 128, q_data_type=torch.bfloat16)
+    q = torch.zeros(556, 4, 128, device=dev, dtype=torch.bfloat16)
+    k = torch.zeros(700, 4, 128, device=dev, dtype=torch.bfloat16)
+    info = torch.zeros(2 + 1, dtype=torch.uint8, device=dev)             # ceil(12/8) + ceil(8/8)
+    keep = torch.zeros(3 + 4, dtype=torch.uint8, device=dev)             # ceil(24/8) + ceil(32/8)
+    ip = torch.tensor([0, 2, 3], dtype=torch.int32, device=dev)
+    kp = torch.tensor([0, 3, 7], dtype=torch.int32, device=dev)
+    w.run(q, k, k, info, keep, ip, kp)
+    with pytest.raises(ValueError, match="tokens; the planned"):
+        w.run(q[:500], k, k, info, keep, ip, kp)
+    with pytest.raises(ValueError, match="tokens; the planned"):
+        w.run(q, k[:600], k[:600], info, keep, ip, kp)
+    with pytest.raises(ValueError, match="sparse_info holds 2 bytes"):
+        w.run(q, k, k, info[:2], keep, ip, kp)
+    with pytest.raises(ValueError, match="sparse_kv_info holds 6 bytes"):
+        w.run(q, k, k, info, keep[:6], ip, kp)
+    with pytest.raises(ValueError, match="must have 3 entries"):
+        w.run(q, k, k, info, keep, ip[:2], kp)
+    with pytest.raises(ValueError, match="3-dimensional"):
+        w.run(q[:, 0], k, k, info, keep, ip, kp)
+
+
 # ------------------------------------------------------------------------------------------------
 # fp8 (e4m3fn) Q.K^T path.  The reference has no fp8 matrix product (it up-casts fp8 storage to
 # fp16) and no absmax quantiser: parity unpinned against it.  Two checks:

@@ -77,6 +77,26 @@ def test_gemm_q_shape_errors(dev):
         fo.flashomni_gemm(x.to(dev), w.to(dev), 1, is_full=True)
 
 
+def test_undersized_symbols_raise(dev):
+    """Packed flags shorter than the last bit the kernels would read are refused on the host."""
+    import flashomni_amd as fo
+    x, w, b = _operands(2, 512, 256, 256, torch.bfloat16, seed=2)
+    x, w = x.to(dev), w.to(dev)
+    # (512 text + 512 tokens) / 128 = 8 blocks x 2 heads = 16 bits = 2 bytes per request
+    info = torch.zeros(4, dtype=torch.uint8, device=dev)
+    ip = torch.tensor([0, 2, 4], dtype=torch.int32, device=dev)
+    fo.flashomni_gemm(x, w, 2, info, ip, 512)
+    fo.flashomni_gemm_reduction(x, w, 2, info, ip, 512)
+    with pytest.raises(RuntimeError, match="a request needs 2"):
+        fo.flashomni_gemm(x, w, 2, info[:1], ip, 512)
+    with pytest.raises(RuntimeError, match="a request needs 2"):
+        fo.flashomni_gemm_reduction(x, w, 2, info[:1], ip, 512)
+    with pytest.raises(RuntimeError, match="batch \\+ 1 = 3 entries"):
+        fo.flashomni_gemm(x, w, 2, info, ip[:2], 512)
+    with pytest.raises(RuntimeError, match="needs sparse_info_indptr"):
+        fo.flashomni_gemm(x, w, 2, info, None, 512)
+
+
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
 @pytest.mark.parametrize("use_bias", [False, True])
 @pytest.mark.parametrize("shape", [(1, 512, 384, 3, 0), (2, 256, 256, 2, 0), (1, 300, 512, 4, 0)])
