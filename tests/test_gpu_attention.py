@@ -441,3 +441,38 @@ def test_video_shapes_sampled_rows(dev, config):
         den += float((b ** 2).sum())
     assert worst_abs <= MAX_ABS
     assert math.sqrt(num / den) <= REL_L2
+
+
+def test_two_wrappers_on_two_streams(dev):
+    """Two planned wrappers (own workspaces, own work lists) launched back to back on two streams
+    without synchronising in between: the library keeps no state that the launches could share."""
+    import flashomni_amd as fo
+    cases = []
+    for seed, (ql, kl, heads) in enumerate([([700, 260], [900, 300], 8), ([1536], [2048], 16)]):
+        m = make_ragged_masks(ql, kl, heads, 0.7, 0.5, seed=50 + seed)
+        g = torch.Generator().manual_seed(60 + seed)
+        nq, nk = int(m["qo_indptr"][-1]), int(m["kv_indptr"][-1])
+        q = torch.randn(nq, heads, 128, generator=g).to(torch.bfloat16)
+        k = torch.randn(nk, heads, 128, generator=g).to(torch.bfloat16)
+        v = torch.randn(nk, heads, 128, generator=g).to(torch.bfloat16)
+        t = lambda a: torch.from_numpy(a).to(dev)
+        w = fo.BatchFlashOmniFAWithRaggedKVWrapper(torch.empty(64 << 20, dtype=torch.uint8, device=dev))
+        w.plan(t(m["qo_indptr"]), t(m["kv_indptr"]), heads, heads, 128, q_data_type=torch.bfloat16)
+        dev_args = (q.to(dev), k.to(dev), v.to(dev), t(m["packed_info"]), t(m["packed_keep"]),
+                    t(m["info_indptr"]), t(m["keep_indptr"]))
+        out0 = sentinel_like((nq, heads, 128), torch.bfloat16)
+        exp = oracle.sparse_attention(q, k, v, m["packed_info"], m["packed_keep"], m["info_indptr"],
+                                      m["keep_indptr"], m["qo_indptr"], m["kv_indptr"], out=out0.clone())
+        cases.append((w, dev_args, out0, exp, m, heads, torch.cuda.Stream(device=dev)))
+    torch.cuda.synchronize()
+    outs = []
+    for rep in range(3):
+        outs = []
+        for w, dev_args, out0, exp, m, heads, stream in cases:
+            with torch.cuda.stream(stream):
+                out = out0.clone().to(dev, non_blocking=False)
+                w.run(*dev_args, out=out)
+                outs.append(out)
+    torch.cuda.synchronize()
+    for out, (w, dev_args, out0, exp, m, heads, stream) in zip(outs, cases):
+        _check(out.cpu(), exp, out0, m, heads)
