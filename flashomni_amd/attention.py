@@ -52,8 +52,9 @@ class DecodedWorkList:
     """Device buffers holding one decoded work list (canonical order).
 
     ``row_req/row_qb/row_head[n_rows]``, ``kv_row_ptr[n_rows+1]``, ``kv_idx[nnz]``, all int32;
-    ``counts = [n_rows, nnz, 0, 0]``; ``order[n_rows]`` / ``sched[256]`` are the execution order
-    and queue words the attention kernel schedules from.  The sizes live on the device;
+    ``counts = [n_rows, nnz, 0, 0]``; ``order[n_rows]`` / ``sched[1024]`` are the execution order
+    and queue words the attention kernel schedules from, ``shares`` the table of even shares it
+    uses instead when there are only a few rows per CU.  The sizes live on the device;
     ``sizes()`` copies them back (one synchronisation) for tests and reports."""
 
     def __init__(self, max_rows: int, max_nnz: int, num_heads: int, device):
@@ -66,7 +67,8 @@ class DecodedWorkList:
         self.kv_idx = torch.empty(max(max_nnz, 1), dtype=torch.int32, device=device)
         self.counts = torch.zeros(4, dtype=torch.int32, device=device)
         self.order = torch.empty(n, dtype=torch.int32, device=device)
-        self.sched = torch.zeros(256, dtype=torch.int32, device=device)
+        self.sched = torch.zeros(1024, dtype=torch.int32, device=device)
+        self.shares = torch.zeros(512 + n + 1, dtype=torch.int32, device=device)
         self.scratch = torch.empty(2 * n + 8192, dtype=torch.int32, device=device)
 
     def sizes(self) -> Tuple[int, int]:
@@ -371,7 +373,8 @@ class BatchFlashOmniFAWithRaggedKVWrapper:
             self._n_q_blk, self._num_qo_heads, self._sparse_block_size_for_kv, int(bool(is_full)),
             _lib.ptr(wl.row_req), _lib.ptr(wl.row_qb), _lib.ptr(wl.row_head), _lib.ptr(wl.kv_row_ptr),
             _lib.ptr(wl.kv_idx), _lib.ptr(wl.counts), _lib.ptr(wl.order), _lib.ptr(wl.sched),
-            _lib.ptr(wl.scratch), int(self._split_ws_ok()), _lib.current_stream(self.device)))
+            _lib.ptr(wl.scratch), _lib.ptr(wl.shares if self._split_ws_ok() else None),
+            _lib.current_stream(self.device)))
         # the memo holds the tensors alive so a recycled address cannot alias the key
         self._decode_key = None if capturing else key
         self._decode_refs = (tensors, sparse_info, sparse_kv_info, sparse_info_indptr,
@@ -473,6 +476,7 @@ class BatchFlashOmniFAWithRaggedKVWrapper:
             _lib.ptr(wl.sched), self._max_rows, q.size(1), self._num_kv_heads, q.size(2),
             self._sparse_block_size_for_q,
             self._sparse_block_size_for_kv, float(sm_scale),
+            _lib.ptr(wl.shares if self._split_ws_ok() else None),
             _lib.ptr(self._float_workspace_buffer) if self._split_ws_ok() else None,
             self._float_ws_bytes(), _lib.current_stream(self.device)))
         return (out, lse) if return_lse else out

@@ -9,13 +9,13 @@
 // Besides the canonical list the decoder emits an execution order for the attention kernel:
 // `order` lists row positions grouped by head, heads dealt to the 8 XCDs round-robin (head % 8), so
 // that the workgroups of one XCD (which share an L2) walk the rows of the same few heads and find
-// that head's K/V in their L2.  Inside a head the rows go longest first (up to 32 length classes relative
-// to the longest row of the launch), which evens out the workgroups' finishing times when there are
-// only a few rows per CU.  sched[0..8] delimit the 8 per-XCD queues inside `order`, sched[16..23]
-// are the queue cursors, sched[24] a completion counter (all cleared here) and sched[25] the
-// longest row's kv count.  sched[32..55] describe, per queue, the rows at its end that the attention
-// kernel shares between workgroups, and sched[64..191] are their arrival counters (cleared here).  The order inside a length class is not deterministic (atomic cursors);
-// results do not depend on it.
+// that head's K/V in their L2.  Inside a head the rows go longest first (up to 32 length classes
+// relative to the longest row of the launch), which evens out the workgroups' finishing times.
+// sched[0..8] delimit the 8 per-XCD queues inside `order`, sched[16..23] are the queue cursors,
+// sched[24] a completion counter (all cleared here) and sched[25] the longest row's kv count.  The
+// order inside a length class is not deterministic (atomic cursors); results do not depend on it.
+// With at most three rows per workgroup of the attention kernel (and a share table to fill) the
+// layout is different, "even shares": see the scan kernel.
 // Integer work, bounded by HBM traffic and launch latency; bit-exact by construction.
 //
 // Symbol semantics (reference: include/flashomni/attention/prefill.cuh:1284-1294, 1380-1403,
@@ -31,9 +31,15 @@ constexpr int kScanThreads = 1024;
 constexpr int kMaxHeads = 1024;
 constexpr int kXcds = 8;
 constexpr int kHistSlots = 8192;  // (head, length class) counters of the order layout
-// split rows (see the attention kernel): words of `sched` and limits
-constexpr int kSchedSplitStart = 32, kSchedSplitParts = 40, kSchedSplitSlot = 48, kSchedArrived = 64;
-constexpr int kMaxSplitSlots = 128, kMaxSplitParts = 4, kSplitMaxRounds = 1;
+// even shares (see the attention kernel): words of `sched` and limits
+constexpr int kSchedEven = 26, kSchedShare = 27, kSchedTotal = 28, kSchedShares = 29, kSchedRows = 30,
+              kSchedArrived = 64;
+constexpr int kMaxShares = 512;      // arrival counters in `sched`, first-row entries in `shares`
+constexpr int kMaxSplitParts = 4;    // a row is cut into at most this many parts
+constexpr int kEvenMaxRounds = 3;    // even shares when there are at most this many rows per workgroup
+                                     // (measured: from ~5 rows per workgroup on, the queues balance as well
+                                     // and adapt to the workgroups' actual speeds, which fixed shares cannot)
+constexpr int kRowOverhead = 3;      // fixed cost of a row (prologue, epilogue) in units of one kv block
 
 // number of length classes for num_heads heads (32 up to 256 heads)
 __host__ __device__ __forceinline__ int len_classes(int32_t num_heads) {
@@ -120,7 +126,8 @@ __global__ void __launch_bounds__(kCountThreads) decode_count_kernel(
 __global__ void __launch_bounds__(kScanThreads) decode_scan_kernel(
     int64_t n_cand, int32_t num_heads, int32_t* __restrict__ act, int32_t* __restrict__ cnt,
     int32_t* __restrict__ kv_row_ptr, int32_t* __restrict__ counts,
-    int32_t* __restrict__ head_cursor, int32_t* __restrict__ sched, int32_t cus_per_xcd) {
+    int32_t* __restrict__ head_cursor, int32_t* __restrict__ sched, int32_t* __restrict__ order,
+    int32_t* __restrict__ shares, int32_t n_shares) {
   __shared__ int32_t s_rows[kScanThreads];
   __shared__ int32_t s_kv[kScanThreads];
   __shared__ int32_t s_hist[kHistSlots];
@@ -166,18 +173,110 @@ __global__ void __launch_bounds__(kScanThreads) decode_scan_kernel(
     row_pos += a;
     kv_pos += n;
   }
+  const int32_t n_rows = s_rows[kScanThreads - 1], nnz = s_kv[kScanThreads - 1];
   if (tid == kScanThreads - 1) {
-    const int32_t n_rows = s_rows[tid], nnz = s_kv[tid];
     counts[0] = n_rows;
     counts[1] = nnz;
     counts[2] = 0;
     counts[3] = 0;
     kv_row_ptr[n_rows] = nnz;
   }
+  __threadfence_block();
+  __syncthreads();  // s_rows / s_kv are free again; act / cnt hold positions now
+
+  // Even shares.  With only a few rows per workgroup, whole rows cannot be dealt evenly (at 2.5 rows
+  // per workgroup the last one to finish has three while others have two).  The rows are then laid
+  // out head by head (q blocks ascending inside a head: a fixed order), every row costs
+  // kRowOverhead + its kv blocks, and workgroup j of the attention kernel gets the cost range
+  // [j * share, (j + 1) * share): rows that straddle a boundary are computed in parts by the
+  // neighbouring workgroups and combined by whoever finishes last.  Nothing depends on timing, so
+  // results repeat from launch to launch.
+  const bool even = shares != nullptr && n_shares > 0 && n_shares <= kMaxShares && n_rows > 0 &&
+                    n_rows <= kEvenMaxRounds * n_shares && num_heads <= kScanThreads;
+  if (even) {
+    const int32_t nq = static_cast<int32_t>(n_cand / num_heads);
+    const int segs = kScanThreads / num_heads;  // threads per head, each a run of q blocks
+    const int per = (nq + segs - 1) / segs;
+    const int h = tid / segs, seg = tid - h * segs;
+    const bool mine = h < num_heads;
+    const int t0 = mine ? min(seg * per, nq) : 0, t1 = mine ? min(t0 + per, nq) : 0;
+    auto kv_count = [&](int64_t c) { return (c + 1 < n_cand ? cnt[c + 1] : nnz) - cnt[c]; };
+    int32_t my_rows = 0, my_cost = 0;
+    for (int t = t0; t < t1; ++t) {
+      const int64_t c = static_cast<int64_t>(t) * num_heads + h;
+      if (act[c] >= 0) {
+        ++my_rows;
+        my_cost += kRowOverhead + kv_count(c);
+      }
+    }
+    s_rows[tid] = my_rows;
+    s_kv[tid] = my_cost;
+    __syncthreads();
+    for (int off = 1; off < kScanThreads; off <<= 1) {
+      int32_t r = 0, k = 0;
+      if (tid >= off) {
+        r = s_rows[tid - off];
+        k = s_kv[tid - off];
+      }
+      __syncthreads();
+      s_rows[tid] += r;
+      s_kv[tid] += k;
+      __syncthreads();
+    }
+    const int32_t total = s_kv[kScanThreads - 1];
+    // a row of n blocks touches at most ceil(n / share) + 1 ranges: share >= n / 3 keeps that within
+    // kMaxSplitParts
+    static_assert(kMaxSplitParts == 4, "the share's lower bound assumes four parts");
+    const int32_t share = max(max((total + n_shares - 1) / n_shares, (max_n + 2) / 3), 1);
+    int32_t pos = s_rows[tid] - my_rows, cost = s_kv[tid] - my_cost;
+    int32_t* first_row = shares;           // [kMaxShares]
+    int32_t* row_start = shares + kMaxShares;  // [n_rows + 1]: cost at which a row's kv blocks begin
+    for (int t = t0; t < t1; ++t) {
+      const int64_t c = static_cast<int64_t>(t) * num_heads + h;
+      if (act[c] >= 0) {
+        order[pos] = act[c];
+        row_start[pos] = cost + kRowOverhead;
+        ++pos;
+        cost += kRowOverhead + kv_count(c);
+      }
+    }
+    if (tid == 0) {
+      row_start[n_rows] = total + kRowOverhead;
+      for (int i = 0; i < 32; ++i) sched[i] = 0;
+      // (the queues stay usable: eight equal runs of the same order, for a launch without shares)
+      for (int x = 0; x <= kXcds; ++x) sched[x] = static_cast<int32_t>(static_cast<int64_t>(n_rows) * x / kXcds);
+      sched[25] = max_n;
+      sched[kSchedEven] = 1;
+      sched[kSchedShare] = share;
+      sched[kSchedTotal] = total;
+      sched[kSchedShares] = n_shares;
+      sched[kSchedRows] = n_rows;
+    }
+    for (int i = tid; i < kMaxShares; i += kScanThreads) sched[kSchedArrived + i] = 0;
+    __threadfence_block();
+    __syncthreads();  // row_start is complete
+    // first row of every share: the first one whose kv blocks end behind the share's lower bound (a
+    // row without kv blocks stands for the last unit of its own overhead)
+    for (int j = tid; j < n_shares; j += kScanThreads) {
+      const int32_t a = j * share;
+      int lo = 0, hi = n_rows;  // first i in [0, n_rows] with end(i) > a; end is increasing
+      while (lo < hi) {
+        const int mid = (lo + hi) >> 1;
+        const int32_t e = row_start[mid + 1] - kRowOverhead;
+        if (e > a) {
+          hi = mid;
+        } else {
+          lo = mid + 1;
+        }
+      }
+      first_row[j] = lo;
+    }
+    return;
+  }
+
   // execution order layout: queue x holds heads x, x+8, x+16, ... back to back, each head's length
   // classes in order.  Exclusive prefix sum of the histogram taken in that order: every thread owns
   // a run of consecutive entries, wavefront scan by lane shifts, then the sixteen wavefront totals.
-  __syncthreads();  // s_rows / s_kv are free again
   {
     const int n_ent = num_heads * n_classes;
     const int per = (n_ent + kScanThreads - 1) / kScanThreads;
@@ -223,29 +322,7 @@ __global__ void __launch_bounds__(kScanThreads) decode_scan_kernel(
       sched[kXcds] = total;
       for (int i = kXcds + 1; i < 32; ++i) sched[i] = 0;
       sched[25] = max_n;
-      // A queue's rows go to the cus_per_xcd workgroups of its XCD.  When there are so few rows that
-      // at most half of the workgroups would get one, every row is cut into 2..4 parts (consecutive
-      // ranges of its kv blocks) so that they all get work.  (With one or more full rounds of rows
-      // the parts' extra prologues and the merge cost what the better balance gains: measured.)
-      int32_t slot = 0;
-      for (int x = 0; x < kXcds; ++x) {
-        const int32_t len = sched[x + 1] - sched[x];
-        int32_t rest = 0, parts = 1;
-        if (cus_per_xcd > 1) {
-          const int32_t rounds = len / cus_per_xcd, rem = len - rounds * cus_per_xcd;
-          if (rounds < kSplitMaxRounds && rem > 0 && 2 * rem <= cus_per_xcd &&
-              slot + rem <= kMaxSplitSlots) {
-            rest = rem;
-            parts = min(kMaxSplitParts, cus_per_xcd / rem);
-          }
-        }
-        sched[kSchedSplitStart + x] = sched[x + 1] - rest;
-        sched[kSchedSplitParts + x] = parts;
-        sched[kSchedSplitSlot + x] = slot;
-        slot += rest;
-      }
     }
-    for (int i = tid; i < kMaxSplitSlots; i += kScanThreads) sched[kSchedArrived + i] = 0;
   }
 }
 
@@ -275,7 +352,8 @@ __global__ void __launch_bounds__(kCountThreads) decode_fill_kernel(
     kv_row_ptr[pos] = out;
     const int32_t listed = (c + 1 < n_cand ? kv_pos[c + 1] : counts[1]) - out;  // kv blocks of this row
     const int n_classes = len_classes(num_heads);
-    order[atomicAdd(&head_cursor[cd.head * n_classes + len_class(listed, sched[25], n_classes)], 1)] = pos;
+    if (!sched[kSchedEven])  // (with even shares the scan kernel has written the order)
+      order[atomicAdd(&head_cursor[cd.head * n_classes + len_class(listed, sched[25], n_classes)], 1)] = pos;
   }
   if (cd.nkv <= 0) return;
   if (is_full) {
@@ -312,7 +390,7 @@ extern "C" int fo_decode_sparse(const uint8_t* sparse_info, const uint8_t* spars
                                 int32_t num_heads, int32_t block_kv, int is_full,
                                 int32_t* row_req, int32_t* row_qb, int32_t* row_head,
                                 int32_t* kv_row_ptr, int32_t* kv_idx, int32_t* counts,
-                                int32_t* order, int32_t* sched, int32_t* scratch, int split_rows,
+                                int32_t* order, int32_t* sched, int32_t* scratch, int32_t* shares,
                                 void* stream) {
   FO_REQUIRE(n_blk >= 0 && num_heads > 0 && num_heads <= kMaxHeads && block_kv > 0,
              "decode: bad sizes");
@@ -337,9 +415,9 @@ extern "C" int fo_decode_sparse(const uint8_t* sparse_info, const uint8_t* spars
         kv_indptr, n_cand, num_heads, block_kv, is_full, act, cnt);
     FO_CHECK_LAUNCH();
   }
-  const int32_t cus_per_xcd = split_rows ? fo_num_cu() / kXcds : 0;
+  const int32_t n_shares = shares ? fo_num_cu() : 0;  // one share per workgroup of the attention kernel
   decode_scan_kernel<<<1, kScanThreads, 0, s>>>(n_cand, num_heads, act, cnt, kv_row_ptr, counts,
-                                                head_cursor, sched, cus_per_xcd);
+                                                head_cursor, sched, order, shares, n_shares);
   FO_CHECK_LAUNCH();
   if (n_cand > 0) {
     const int per_wg = kCountThreads / kWave;

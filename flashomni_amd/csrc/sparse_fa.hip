@@ -117,6 +117,7 @@ struct FaParams {
   const int32_t* order;
   int32_t* sched;
   float* split_ws;  // partial results of rows whose kv list is split over workgroups (or null)
+  const int32_t* shares;  // even shares: first row of every share, then the rows' cost offsets (or null)
   int32_t num_heads;
   int32_t kv_group;  // q heads per kv head (grouped-query attention); 1 = one kv head per q head
   int32_t n_q_blocks, n_kv_blocks;  // row lengths of q_scale / k_scale
@@ -195,12 +196,18 @@ __device__ __forceinline__ float max_across_halves(float x) {
 }
 
 // words of `sched` (written by the decoder): [0..8] queue bounds inside `order`, [16..23] queue
-// cursors, [24] completion counter, [32..39] first split position of each queue, [40..47] number
-// of parts its split rows are cut into, [48..55] first split slot of the queue, [64..191] arrival
-// counters of the split slots
-constexpr int kSchedSplitStart = 32, kSchedSplitParts = 40, kSchedSplitSlot = 48, kSchedArrived = 64;
-constexpr int kMaxSplitSlots = 128, kMaxSplitParts = 4;
+// cursors, [24] completion counter; [26] even shares in use, [27] cost share of a workgroup, [28]
+// total cost, [29] number of shares, [30] number of rows; [64..575] arrival counters of the rows cut at share boundaries
+constexpr int kSchedEven = 26, kSchedArrived = 64;
+constexpr int kMaxShares = 512, kMaxSplitParts = 4, kRowOverhead = 3;
+constexpr int kItemBatch = 16;  // item records of a share gathered at a time
 constexpr int kSplitPartFloats = 128 * 128 + 2 * 256;  // O (fp32) + (max, sum) per lane of kv group 0
+// Partial results live in 2 * kMaxShares areas of the workspace: share j writes the part of a row
+// that began in an earlier share to area 2j and the first part of a row that continues into the
+// next share to area 2j + 1 (a share holds at most one of each).
+__device__ __forceinline__ int part_area(int first_share, int part) {
+  return part == 0 ? 2 * first_share + 1 : 2 * (first_share + part);
+}
 
 // Partial results cross workgroups (and XCDs, whose L2s are not coherent with each other) through
 // device-scope accesses that bypass the local L2 instead of through fences, which would write back
@@ -216,35 +223,24 @@ __device__ __forceinline__ void load_pair_device(const float* p, float& a, float
   b = __uint_as_float(static_cast<uint32_t>(v >> 32));
 }
 
-struct Item {
-  int row;   // position in the canonical row list, -1 = queues are empty
-  int meta;  // part | parts << 4 | slot << 8
-};
-
-// Pop the next work item for this workgroup: own XCD queue first, then the neighbours'.  The last
-// rows of a queue may be cut into `parts` items that cover consecutive ranges of the row's kv
-// blocks: position ss + v of the queue then stands for part v % parts of row order[ss + v / parts].
-// `first` is the first queue that may still hold items: a queue found empty stays empty for the rest
-// of the launch, so it is not asked again.  `q` is the launch's copy of the queue words
-// (q[x] = bounds, q[9 + x] = split start, q[17 + x] = parts, q[25 + x] = first slot): the pop itself
-// is one atomic and one load.
-__device__ __forceinline__ Item pop_row(const FaParams& p, int xcd, const int* q, int* first) {
+// Pop the next row for this workgroup from the queues: own XCD queue first, then the neighbours'.
+// `first` is the first queue that may still hold rows: a queue found empty stays empty for the rest
+// of the launch, so it is not asked again.  `q` is the launch's copy of the queue bounds: the pop
+// itself is one atomic and one load.  Returns the row's position in the canonical list or -1.
+__device__ __forceinline__ int pop_row(const FaParams& p, int xcd, const int* q, int* first) {
   for (int a = *first; a < kXcds; ++a) {
     const int x = (xcd + a) & (kXcds - 1);
-    const int beg = q[x], end = q[x + 1], ss = q[9 + x], parts = q[17 + x];
-    const int vend = end + (end - ss) * (parts - 1);
-    if (beg < vend) {
+    const int beg = q[x], end = q[x + 1];
+    if (beg < end) {
       const int pos = beg + atomicAdd(&p.sched[16 + x], 1);
-      if (pos < vend) {
+      if (pos < end) {
         *first = a;
-        if (pos < ss) return Item{p.order[pos], 1 << 4};
-        const int v = pos - ss, r = v / parts;
-        return Item{p.order[ss + r], (v - r * parts) | parts << 4 | (q[25 + x] + r) << 8};
+        return p.order[pos];
       }
     }
   }
   *first = kXcds;
-  return Item{-1, 0};
+  return -1;
 }
 
 // T: element type of V, P and O (and of Q, K unless kFp8).  kFp8: Q and K are e4m3fn bytes with one
@@ -267,7 +263,9 @@ __global__ void __launch_bounds__(kThreads) sparse_fa_kernel(const FaParams p) {
   };
   __shared__ RowInfo s_next_row[2];
   __shared__ int s_arrived;
-  __shared__ int s_queue[40];  // the queue words of `sched`, read once
+  __shared__ int s_queue[16];  // queue bounds and even-share words of `sched`, read once
+  __shared__ int s_share[1];   // even shares: items of this workgroup's share handed out so far
+  __shared__ RowInfo s_items[kItemBatch];  // even shares: records of the share's next items
   __shared__ uint16_t s_blk2[2][kMaxRowBlocks];  // kv block list of this row / the next one
 
   const int tid = threadIdx.x, lane = tid & 63;
@@ -312,26 +310,84 @@ __global__ void __launch_bounds__(kThreads) sparse_fa_kernel(const FaParams p) {
   // The next row is popped by kv group 1 while kv group 0 combines and stores the current one
   // (group 1 has nothing else to do then), so the queue atomics are off the critical path.
   if (tid < 9) s_queue[tid] = p.sched[tid];
-  if (tid >= 64 && tid < 64 + 24)
-    s_queue[9 + tid - 64] = p.sched[kSchedSplitStart + tid - 64];  // split start, parts, first slot
+  if (tid >= 64 && tid < 64 + 5) s_queue[9 + tid - 64] = p.sched[kSchedEven + tid - 64];
   __syncthreads();
+  // Even shares: the decoder has laid the rows out head by head and given every row a cost
+  // (kRowOverhead + its kv blocks); share j is the cost range [j * share, (j + 1) * share), and a
+  // row that straddles share boundaries is computed in parts by the shares it touches.  Every
+  // workgroup holds one share; they are dealt so that the workgroups of one XCD hold neighbouring
+  // shares (the same heads' K and V).  A share's items are consecutive rows of `order`, known from
+  // the start: their records are gathered sixteen at a time, all in parallel, so that between two
+  // rows only the kv block list has to be fetched.
+  const int ev_share = s_queue[10], ev_total = s_queue[11], ev_n = s_queue[12], ev_rows = s_queue[13];
+  const bool even = s_queue[9] != 0 && p.shares != nullptr && p.split_ws != nullptr &&
+                    static_cast<int>(gridDim.x) == ev_n;
+  const int ev_j = (ev_n & (kXcds - 1)) == 0 ? (blockIdx.x & (kXcds - 1)) * (ev_n / kXcds) + blockIdx.x / kXcds
+                                             : static_cast<int>(blockIdx.x);
+  auto fill_items = [&](int batch_base) {
+    if (lane < kItemBatch) {
+      RowInfo it;
+      it.row = -1;
+      it.ptr0 = 0;
+      it.nb = 0;
+      const int a = ev_j * ev_share, b = min(a + ev_share, ev_total);
+      const int i = p.shares[ev_j] + batch_base + lane;
+      const int32_t* row_start = p.shares + kMaxShares;
+      if (a < ev_total && i < ev_rows) {
+        const int u = row_start[i], e = row_start[i + 1] - kRowOverhead;  // kv blocks cost [u, e)
+        // (a row without kv blocks stands for the last unit of its own overhead)
+        if ((e > u ? u : u - 1) < b) {
+          const int w = p.order[i];
+          it.row = w;
+          it.part = 0;
+          it.parts = 1;
+          it.slot = 0;
+          if (e > u) {
+            const int j_lo = u / ev_share, j_hi = (e - 1) / ev_share;
+            it.part = ev_j - j_lo;
+            it.parts = j_hi - j_lo + 1;
+            it.slot = j_lo;
+          }
+          it.req = p.row_req[w];
+          it.qb = p.row_qb[w];
+          it.head = p.row_head[w];
+          it.q_begin = p.qo_indptr[it.req] + it.qb * kBlockQ;
+          it.q_rows = min(kBlockQ, p.qo_indptr[it.req + 1] - it.q_begin);
+          it.kv_begin = p.kv_indptr[it.req];
+          it.kv_len = p.kv_indptr[it.req + 1] - it.kv_begin;
+          // this share's range of the row's kv blocks
+          const int blk_lo = max(a, u) - u, blk_hi = min(min(b, e) - u, kMaxRowBlocks);
+          it.ptr0 = p.kv_row_ptr[w] + blk_lo;
+          it.nb = max(blk_hi - blk_lo, 0);
+        }
+      }
+      s_items[lane] = it;
+    }
+  };
   int first_queue = 0;  // kept by the popping lane (the first pop is lane 0's, the others lane 256's)
-  // One wavefront: lane 0 pops the next item and gathers its row's metadata (two rounds of loads),
-  // then all lanes copy the row's kv block list; both go to LDS for the whole workgroup.
+  // One wavefront: lane 0 takes the next item (even shares: from the gathered records; otherwise it
+  // pops a row and gathers its metadata, two rounds of loads), then all lanes copy the row's kv
+  // block list; both go to LDS for the whole workgroup.
   auto fetch_next = [&](int slot_idx) {
     RowInfo ri;
     ri.row = -1;
     ri.ptr0 = 0;
     ri.nb = 0;
-    if (lane == 0) {
-      for (;;) {
-        const Item item = pop_row(p, blockIdx.x & (kXcds - 1), s_queue, &first_queue);
-        ri.row = item.row;
-        if (item.row < 0) break;
-        const int w = item.row;
-        ri.part = item.meta & 15;
-        ri.parts = (item.meta >> 4) & 15;
-        ri.slot = item.meta >> 8;
+    if (even) {
+      const int c = s_share[0];  // items handed out so far
+      if (c > 0 && (c & (kItemBatch - 1)) == 0) fill_items(c);
+      if (lane == 0) {
+        ri = s_items[c & (kItemBatch - 1)];
+        s_share[0] = c + 1;
+        s_next_row[slot_idx] = ri;
+      }
+    } else if (lane == 0) {
+      const int w = pop_row(p, blockIdx.x & (kXcds - 1), s_queue, &first_queue);
+      ri.row = w;
+      ri.part = 0;
+      ri.parts = 1;
+      ri.slot = 0;
+      if (w >= 0) {
         ri.req = p.row_req[w];
         ri.qb = p.row_qb[w];
         ri.head = p.row_head[w];
@@ -342,18 +398,6 @@ __global__ void __launch_bounds__(kThreads) sparse_fa_kernel(const FaParams p) {
         ri.q_rows = min(kBlockQ, p.qo_indptr[ri.req + 1] - ri.q_begin);
         ri.kv_begin = p.kv_indptr[ri.req];
         ri.kv_len = p.kv_indptr[ri.req + 1] - ri.kv_begin;
-        if (ri.parts > 1) {
-          if (ri.nb < 2 * ri.parts || p.split_ws == nullptr) {
-            // too short to share (or nowhere to put partial results): part 0 does the whole row
-            if (ri.part > 0) continue;
-            ri.parts = 1;
-          } else {
-            const int b0 = ri.nb * ri.part / ri.parts, b1 = ri.nb * (ri.part + 1) / ri.parts;
-            ri.ptr0 += b0;
-            ri.nb = b1 - b0;
-          }
-        }
-        break;
       }
       s_next_row[slot_idx] = ri;
     }
@@ -362,10 +406,22 @@ __global__ void __launch_bounds__(kThreads) sparse_fa_kernel(const FaParams p) {
       const int list0 = __builtin_amdgcn_readfirstlane(ri.ptr0), n = __builtin_amdgcn_readfirstlane(ri.nb);
       for (int i = lane; i < n; i += 64) s_blk2[slot_idx][i] = static_cast<uint16_t>(p.kv_idx[list0 + i]);
     }
+    // (everything fetched has been used; said explicitly so that the compiler does not carry these
+    // loads as pending to the top of the row loop and wait there, behind the previous row's stores)
+    __builtin_amdgcn_s_waitcnt(0x0f70);
   };
-  if (wv == 0) fetch_next(0);
+  if (wv == 0) {
+    if (even) {
+      if (lane == 0) s_share[0] = 0;
+      fill_items(0);
+    }
+    fetch_next(0);
+  }
   for (int row_it = 0;; ++row_it) {
-    __syncthreads();  // s_next_row is published; everyone is done with the previous row's LDS data
+    // s_next_row is published; everyone is done with the previous row's LDS data.  (Not
+    // __syncthreads(): its fence would also wait for the row just stored to be acknowledged by
+    // memory, a few microseconds that nothing here depends on.)
+    asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
     const RowInfo& ri = s_next_row[row_it & 1];
     const int w = __builtin_amdgcn_readfirstlane(ri.row);  // uniform values, kept in scalar registers
     if (w < 0) break;
@@ -578,10 +634,14 @@ __global__ void __launch_bounds__(kThreads) sparse_fa_kernel(const FaParams p) {
     // Q from LDS while the first tile copies are in flight: rows (qs % 2) * 32 + l32 of the tile that
     // kv group qs / 2 copied, addressed like a K operand
     if constexpr (!kFp8) {
+      // (the lane terms are made opaque here: otherwise the eight read addresses are worked out once
+      // per kernel, live across the main loop, and their reloads wait for every copy in flight)
+      int q_rd_base = k_rd_base, q_rd_x = k_rd_x;
+      asm volatile("" : "+v"(q_rd_base), "+v"(q_rd_x));
       const uint8_t* qt = smem + (qs >> 1) * kGroupBytes + kStageBytes + kKBytes + (qs & 1) * 32 * kRowBytes +
-                          k_rd_base;
+                          q_rd_base;
 #pragma unroll
-      for (int ks = 0; ks < 8; ++ks) qreg[ks] = *reinterpret_cast<const x8*>(qt + (k_rd_x ^ (ks << 5)));
+      for (int ks = 0; ks < 8; ++ks) qreg[ks] = *reinterpret_cast<const x8*>(qt + (q_rd_x ^ (ks << 5)));
       // the softmax scale (log2 domain) is folded into Q, so S^T needs no multiply
 #pragma unroll
       for (int ks = 0; ks < 8; ++ks)
@@ -880,72 +940,103 @@ __global__ void __launch_bounds__(kThreads) sparse_fa_kernel(const FaParams p) {
         if (row_ok && p.lse && g == 0)
           p.lse[q_tok * p.num_heads + head] = __builtin_amdgcn_logf(d_tot) + m;
       } else {
-        // one part of a split row: fold kv group 1 in without normalising and publish the partial
-        // result (same lane layout as the LDS merge area)
-        float* part_ws = p.split_ws +
-                         static_cast<int64_t>(split_slot * kMaxSplitParts + part) * kSplitPartFloats;
-        // (opaque lane index: see the row store below)
-        int ln = lane;
-        asm volatile("" : "+v"(ln));
-        float* lane_ws = part_ws + (qs * 16 * 2 * 64 + ln) * 2;
+        // one part of a row cut at share boundaries: fold kv group 1 in without normalising; the
+        // accumulators then hold this workgroup's partial result (reference point m, sum d_tot)
         f32x4 t4[16];
 #pragma unroll
         for (int e = 0; e < 16; ++e) t4[e] = mo[(qs * 16 + e) * 64 + lane];
         __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
-        for (int e = 0; e < 16; ++e) {
-          float u[4];
+        for (int e = 0; e < 16; ++e)
 #pragma unroll
-          for (int j = 0; j < 4; ++j) u[j] = o_acc[e >> 2][(e & 3) * 4 + j] * a0 + t4[e][j] * a1;
-          // two planes of 8-byte pairs: each store instruction covers 512 contiguous bytes
-          store_pair_device(lane_ws + e * 256, u[0], u[1]);
-          store_pair_device(lane_ws + e * 256 + 128, u[2], u[3]);
-        }
-        store_pair_device(part_ws + 128 * 128 + (qs * 64 + ln) * 2, m, d_tot);
+          for (int j = 0; j < 4; ++j)
+            o_acc[e >> 2][(e & 3) * 4 + j] = o_acc[e >> 2][(e & 3) * 4 + j] * a0 + t4[e][j] * a1;
+        m_all = m;
+        d_all = d_tot;
       }
     }
     if (parts > 1) {
-      // whoever arrives last at the row's slot combines the parts and writes the row
-      __builtin_amdgcn_s_waitcnt(0x0f70);  // vmcnt(0): this lane's partial results have left
+      // Whoever comes last combines the parts and writes the row.  A workgroup that finds every
+      // other part arrived already need not publish its own; otherwise it publishes, then counts
+      // itself in, and may still turn out to be the last.
+      if (tid == 0)
+        s_arrived = __hip_atomic_load(&p.sched[kSchedArrived + split_slot], __ATOMIC_RELAXED,
+                                      __HIP_MEMORY_SCOPE_AGENT);
       __syncthreads();
-      if (tid == 0) s_arrived = atomicAdd(&p.sched[kSchedArrived + split_slot], 1);
-      __syncthreads();
-      if (s_arrived == parts - 1) {
+      bool last = s_arrived == parts - 1;
+      if (!last) {
         if (kg == 0) {
-          // every part is read back, this workgroup's own included, and added in part order: the
-          // row does not depend on which part arrived last
-          const float* slot_ws = p.split_ws + static_cast<int64_t>(split_slot * kMaxSplitParts) * kSplitPartFloats;
+          // same lane layout as the LDS merge area; two planes of 8-byte pairs, so that each store
+          // instruction covers 512 contiguous bytes
+          float* part_ws = p.split_ws + static_cast<int64_t>(part_area(split_slot, part)) * kSplitPartFloats;
+          // (opaque lane index: see the row store below)
+          int ln = lane;
+          asm volatile("" : "+v"(ln));
+          float* lane_ws = part_ws + (qs * 16 * 2 * 64 + ln) * 2;
+#pragma unroll
+          for (int e = 0; e < 16; ++e) {
+            store_pair_device(lane_ws + e * 256, o_acc[e >> 2][(e & 3) * 4 + 0], o_acc[e >> 2][(e & 3) * 4 + 1]);
+            store_pair_device(lane_ws + e * 256 + 128, o_acc[e >> 2][(e & 3) * 4 + 2], o_acc[e >> 2][(e & 3) * 4 + 3]);
+          }
+          store_pair_device(part_ws + 128 * 128 + (qs * 64 + ln) * 2, m_all, d_all);
+        }
+        __builtin_amdgcn_s_waitcnt(0x0f70);  // vmcnt(0): this lane's partial results have left
+        __syncthreads();
+        if (tid == 0) s_arrived = atomicAdd(&p.sched[kSchedArrived + split_slot], 1);
+        __syncthreads();
+        last = s_arrived == parts - 1;
+      }
+      if (last) {
+        if (kg == 0) {
+          // The parts are added in part order, this workgroup's own from its registers (the same
+          // values it would have published), the others read back: the row does not depend on
+          // which part came last.
+          auto part_base = [&](int i) {
+            return p.split_ws + static_cast<int64_t>(part_area(split_slot, i)) * kSplitPartFloats;
+          };
           float m_p[kMaxSplitParts], d_p[kMaxSplitParts];
+          const float m_own = m_all, d_own = d_all;
           m_all = kNegInf;
           for (int i = 0; i < parts; ++i) {
-            load_pair_device(slot_ws + i * kSplitPartFloats + 128 * 128 + (qs * 64 + lane) * 2, m_p[i], d_p[i]);
+            if (i == part) {
+              m_p[i] = m_own;
+              d_p[i] = d_own;
+            } else {
+              load_pair_device(part_base(i) + 128 * 128 + (qs * 64 + lane) * 2, m_p[i], d_p[i]);
+            }
             m_all = fmaxf(m_all, m_p[i]);
           }
           d_all = 0.f;
+          f32x16 acc[4];
 #pragma unroll
           for (int dt = 0; dt < 4; ++dt)
 #pragma unroll
-            for (int e = 0; e < 16; ++e) o_acc[dt][e] = 0.f;
+            for (int e = 0; e < 16; ++e) acc[dt][e] = 0.f;
           int ln = lane;
           asm volatile("" : "+v"(ln));
           for (int i = 0; i < parts; ++i) {
-            const float* lane_ws = slot_ws + i * kSplitPartFloats + (qs * 16 * 2 * 64 + ln) * 2;
             const float a = __builtin_amdgcn_exp2f(m_p[i] - m_all);
-            d_all += d_p[i] * a;
-            // half of the part's values at a time, all loads of a half in flight together
+            d_all = __builtin_fmaf(d_p[i], a, d_all);
+            if (i == part) {
 #pragma unroll
-            for (int half = 0; half < 2; ++half) {
-              float u[8][4];
+              for (int dt = 0; dt < 4; ++dt)
 #pragma unroll
-              for (int e = 0; e < 8; ++e) {
-                load_pair_device(lane_ws + (half * 8 + e) * 256, u[e][0], u[e][1]);
-                load_pair_device(lane_ws + (half * 8 + e) * 256 + 128, u[e][2], u[e][3]);
+                for (int e = 0; e < 16; ++e) acc[dt][e] = __builtin_fmaf(o_acc[dt][e], a, acc[dt][e]);
+            } else {
+              const float* lane_ws = part_base(i) + (qs * 16 * 2 * 64 + ln) * 2;
+              // all loads of the part in flight together
+              float u[16][4];
+#pragma unroll
+              for (int e = 0; e < 16; ++e) {
+                load_pair_device(lane_ws + e * 256, u[e][0], u[e][1]);
+                load_pair_device(lane_ws + e * 256 + 128, u[e][2], u[e][3]);
               }
               __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
-              for (int e = 0; e < 8; ++e)
+              for (int e = 0; e < 16; ++e)
 #pragma unroll
-                for (int j = 0; j < 4; ++j) o_acc[half * 2 + (e >> 2)][(e & 3) * 4 + j] += u[e][j] * a;
+                for (int j = 0; j < 4; ++j)
+                  acc[e >> 2][(e & 3) * 4 + j] = __builtin_fmaf(u[e][j], a, acc[e >> 2][(e & 3) * 4 + j]);
             }
           }
           const float inv = __builtin_amdgcn_rcpf(d_all);
@@ -955,7 +1046,7 @@ __global__ void __launch_bounds__(kThreads) sparse_fa_kernel(const FaParams p) {
             for (int i4 = 0; i4 < 4; ++i4) {
               x4 out;
 #pragma unroll
-              for (int j = 0; j < 4; ++j) out[j] = static_cast<T>(o_acc[dt][i4 * 4 + j] * inv);
+              for (int j = 0; j < 4; ++j) out[j] = static_cast<T>(acc[dt][i4 * 4 + j] * inv);
               *reinterpret_cast<x4*>(out_row + (dt * 32 + i4 * 8 + g * 4) * sizeof(T)) = out;
             }
           if (row_ok && p.lse && g == 0)
@@ -964,6 +1055,9 @@ __global__ void __launch_bounds__(kThreads) sparse_fa_kernel(const FaParams p) {
         if (tid == 0) p.sched[kSchedArrived + split_slot] = 0;  // re-armed for the next launch
         store_row = true;
       }
+      // (nothing may be in flight into registers where this path joins the one that stores a row:
+      // the compiler would wait there for everything, the row's stores included)
+      __builtin_amdgcn_s_waitcnt(0x0f70);
     }
     if (store_row) {
       __syncthreads();  // the row is complete in the LDS tile
@@ -1007,8 +1101,8 @@ int launch(const FaParams& p, int64_t max_rows, hipStream_t stream) {
   int num_cu = fo_num_cu();
   if (num_cu <= 0) return fo::fail(FO_ERR_HIP, "sparse_fa: no device");
   int64_t grid = num_cu;  // one persistent workgroup per CU (LDS bound)
-  const int64_t max_items = p.split_ws ? max_rows * kMaxSplitParts : max_rows;
-  if (grid > max_items) grid = max_items;
+  // (with even shares every workgroup may hold a part of a row; otherwise at most one row each)
+  if (!(p.split_ws && p.shares) && grid > max_rows) grid = max_rows;
   sparse_fa_kernel<T, kFp8><<<static_cast<unsigned>(grid), kThreads, kSmemBytes, stream>>>(p);
   FO_CHECK_LAUNCH();
   return FO_OK;
@@ -1017,7 +1111,8 @@ int launch(const FaParams& p, int64_t max_rows, hipStream_t stream) {
 }  // namespace
 
 extern "C" int64_t fo_sparse_fa_split_workspace_bytes(void) {
-  return static_cast<int64_t>(kMaxSplitSlots) * kMaxSplitParts * kSplitPartFloats * sizeof(float);
+  // two areas per share, one share per workgroup = per CU
+  return static_cast<int64_t>(2) * fo_num_cu() * kSplitPartFloats * sizeof(float);
 }
 
 extern "C" int fo_sparse_fa_run(const void* q, const void* k, const void* v, void* o, float* lse,
@@ -1032,8 +1127,8 @@ extern "C" int fo_sparse_fa_run(const void* q, const void* k, const void* v, voi
                                 const int32_t* kv_row_ptr, const int32_t* kv_idx,
                                 const int32_t* order, int32_t* sched, int64_t max_rows,
                                 int32_t num_heads, int32_t num_kv_heads, int32_t head_dim, int32_t block_q,
-                                int32_t block_kv, float sm_scale, void* split_workspace,
-                                int64_t split_workspace_bytes, void* stream) {
+                                int32_t block_kv, float sm_scale, const int32_t* shares,
+                                void* split_workspace, int64_t split_workspace_bytes, void* stream) {
   FO_REQUIRE(head_dim == kHeadDim, "sparse_fa: head_dim %d is not supported (only 128)", head_dim);
   FO_REQUIRE(block_q == kBlockQ && block_kv == kBlockKV,
              "sparse_fa: sparse block sizes (%d, %d) are not supported (only 128, 128)", block_q,
@@ -1071,12 +1166,18 @@ extern "C" int fo_sparse_fa_run(const void* q, const void* k, const void* v, voi
   p.q_blk_base = q_blk_base; p.kv_blk_base = kv_blk_base;
   p.row_req = row_req; p.row_qb = row_qb; p.row_head = row_head;
   p.kv_row_ptr = kv_row_ptr; p.kv_idx = kv_idx; p.order = order; p.sched = sched;
-  // without room for partial results every split row is computed whole by its first part
+  // even shares need both the decoder's share table and room for partial results (without them
+  // the rows are taken whole from the queues, which the decoder fills either way)
   p.split_ws = nullptr;
-  if (split_workspace != nullptr && split_workspace_bytes >= fo_sparse_fa_split_workspace_bytes()) {
+  p.shares = nullptr;
+  if (shares != nullptr) {
+    FO_REQUIRE(split_workspace != nullptr && split_workspace_bytes >= fo_sparse_fa_split_workspace_bytes(),
+               "sparse_fa: the work list was decoded for even shares, which need a split workspace of "
+               "fo_sparse_fa_split_workspace_bytes() bytes");
     FO_REQUIRE((reinterpret_cast<uintptr_t>(split_workspace) & 15) == 0,
                "sparse_fa: split_workspace must be 16-byte aligned");
     p.split_ws = static_cast<float*>(split_workspace);
+    p.shares = shares;
   }
   p.num_heads = num_heads; p.kv_group = num_heads / num_kv_heads; p.n_q_blocks = n_q_blocks; p.n_kv_blocks = n_kv_blocks;
   p.sm_scale_log2 = sm_scale * 1.44269504088896340736f;

@@ -90,16 +90,20 @@ int fo_prefill_plan(void* float_ws, size_t float_ws_bytes, void* int_ws_dev, voi
  *   order [n_rows]   execution order for the attention kernel: canonical row positions grouped by
  *                    head, heads dealt round-robin to 8 queues (head % 8, one queue per XCD);
  *                    inside one head longer rows first (up to 32 length classes), otherwise unspecified
- *   sched [256]      sched[0..8] = queue boundaries inside `order`, sched[16..23] = queue cursors
+ *   sched [1024]     sched[0..8] = queue boundaries inside `order`, sched[16..23] = queue cursors
  *                    and sched[24] = completion counter, both cleared to 0; sched[25] = kv count of
- *                    the longest row; sched[32..39] = first split position of each queue,
- *                    sched[40..47] = parts per split row, sched[48..55] = first split slot,
- *                    sched[64..191] = arrival counters of the split slots (cleared to 0)
- * split_rows != 0: when a queue holds so few rows that at most half of the workgroups of its XCD
- * would get one, the attention kernel cuts each row into 2..4 parts (consecutive ranges of its kv
- * blocks) that different workgroups compute
- * (the counterpart of the reference's split-kv plan, scheduler.cuh:35-64, decided on the device
- * from the decoded row count).  The canonical lists do not change.
+ *                    the longest row; sched[26..30] = even shares: in use, cost share of a
+ *                    workgroup, total cost, number of shares, number of rows;
+ *                    sched[64..575] = arrival counters of rows cut at share boundaries (cleared)
+ * shares (optional, [512 + n_blk*H + 1] int32): when given and the list holds at most 3 rows per
+ * CU, the decoder lays out even shares instead: `order` then lists the rows head by head (q blocks
+ * ascending: a fixed order), a row costs 3 + its kv blocks, shares[512 + i] is the cost at which the
+ * kv blocks of row order[i] begin, share j is the cost range [j*sched[27], (j+1)*sched[27]) and
+ * shares[j] its first row.  The attention kernel gives every workgroup one share and computes a
+ * row that straddles a boundary in parts (consecutive ranges of its kv blocks, at most 4), one per
+ * share it touches (the counterpart of the reference's split-kv plan, scheduler.cuh:35-64, decided
+ * on the device from the decoded list).  The queues stay valid (eight equal runs of `order`), and
+ * the canonical lists do not change.
  * is_full != 0 ignores the symbol tensors (which may be NULL) and lists everything
  * (csrc/batch_sparseFA.cu:123-128).
  * `scratch` needs 2*n_blk*H + 8192 int32.
@@ -116,7 +120,7 @@ int fo_decode_sparse(const uint8_t* sparse_info, const uint8_t* sparse_kv_info,
                      int32_t n_blk, int32_t num_heads, int32_t block_kv, int is_full,
                      int32_t* row_req, int32_t* row_qb, int32_t* row_head, int32_t* kv_row_ptr,
                      int32_t* kv_idx, int32_t* counts, int32_t* order, int32_t* sched,
-                     int32_t* scratch, int split_rows, void* stream);
+                     int32_t* scratch, int32_t* shares, void* stream);
 
 /* ---------------------------------------------------------------------------------------------
  * Ragged block-sparse FlashAttention prefill over a decoded work list.
@@ -136,11 +140,13 @@ int fo_decode_sparse(const uint8_t* sparse_info, const uint8_t* sparse_kv_info,
  * Rows are taken from the queues described by `order` / `sched` (see fo_decode_sparse); the
  * kernel leaves the queue cursors rewound, so one decoded list can be run any number of times,
  * but two launches sharing one `sched` must not overlap in time.
- * split_workspace: device memory of fo_sparse_fa_split_workspace_bytes() bytes, 16-byte aligned,
- * for the unnormalised partial results (fp32 O, row maximum, row sum) of split rows: the part that
- * arrives last combines them (replaces the reference's float workspace + merge kernels,
- * scheduler.cuh:322-328, cascade.cuh:346-437).  NULL or too small: every split row is computed
- * whole by the workgroup that pops its first part.  Launches sharing it must not overlap in time.
+ * shares: the table fo_decode_sparse filled for this list, or NULL.  With it (and when the decoder
+ * chose even shares) every workgroup computes one share; split_workspace, device memory of
+ * fo_sparse_fa_split_workspace_bytes() bytes (two areas per CU), 16-byte aligned, is then required
+ * and receives the unnormalised partial results (fp32 O, row maximum, row sum) of rows cut at share
+ * boundaries: the part that arrives last combines them in part order (replaces the reference's
+ * float workspace + merge kernels, scheduler.cuh:322-328, cascade.cuh:346-437).  Without shares
+ * the rows are taken whole from the queues.  Launches sharing a workspace must not overlap in time.
  * Supported: D = 128, block_q = 128, block_kv = 128.  max_rows bounds the number of rows.
  * ------------------------------------------------------------------------------------------- */
 int64_t fo_sparse_fa_split_workspace_bytes(void);
@@ -153,8 +159,8 @@ int fo_sparse_fa_run(const void* q, const void* k, const void* v, void* o, float
                      int32_t n_kv_blocks, const int32_t* row_req, const int32_t* row_qb, const int32_t* row_head,
                      const int32_t* kv_row_ptr, const int32_t* kv_idx, const int32_t* order,
                      int32_t* sched, int64_t max_rows, int32_t num_heads, int32_t num_kv_heads, int32_t head_dim,
-                     int32_t block_q, int32_t block_kv, float sm_scale, void* split_workspace,
-                     int64_t split_workspace_bytes, void* stream);
+                     int32_t block_q, int32_t block_kv, float sm_scale, const int32_t* shares,
+                     void* split_workspace, int64_t split_workspace_bytes, void* stream);
 
 /* ---------------------------------------------------------------------------------------------
  * GEMM-Q: y[b, tile] = x[b] . w^T + bias for every (128-row, 128-column) tile whose symbol bit

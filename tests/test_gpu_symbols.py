@@ -119,6 +119,7 @@ def test_decoder_execution_order(dev, case):
     m = make_ragged_masks(ql, kl, heads, pa, pk, seed=7)
     ws = torch.empty(128 << 20, dtype=torch.uint8, device=dev)
     w = fo.BatchFlashOmniFAWithRaggedKVWrapper(ws)
+    w._share_rows = False                       # whole rows from the queues
     w.plan(torch.from_numpy(m["qo_indptr"]), torch.from_numpy(m["kv_indptr"]), heads, heads, 128,
            q_data_type=torch.bfloat16)
     t = lambda a: torch.from_numpy(a).to(dev)
@@ -130,7 +131,7 @@ def test_decoder_execution_order(dev, case):
     ptr = wl.kv_row_ptr[:n_rows + 1].cpu().numpy()
     lens = ptr[1:] - ptr[:-1]
     assert sorted(order.tolist()) == list(range(n_rows))
-    assert sched[0] == 0 and sched[8] == n_rows and (sched[16:25] == 0).all()
+    assert sched[0] == 0 and sched[8] == n_rows and (sched[16:25] == 0).all() and sched[26] == 0
     max_n = int(lens.max()) if n_rows else 0
     assert sched[25] == max_n
     n_classes = min(32, 8192 // heads)
@@ -142,3 +143,44 @@ def test_decoder_execution_order(dev, case):
         cls = (max_n - lens[seg]).astype(np.int64) * n_classes // (max_n + 1)
         same_head = np.diff(h) == 0
         assert (np.diff(cls)[same_head] >= 0).all()   # longest class first inside a head
+
+
+@pytest.mark.parametrize("case", CASES)
+def test_decoder_even_shares(dev, case):
+    """Few rows per CU: `order` lists the rows head by head in canonical order, a row costs
+    3 + its kv blocks, and the share table cuts the cost line into one range per CU."""
+    import flashomni_amd as fo
+    ql, kl, heads, pa, pk = case
+    m = make_ragged_masks(ql, kl, heads, pa, pk, seed=7)
+    w = fo.BatchFlashOmniFAWithRaggedKVWrapper(torch.empty(128 << 20, dtype=torch.uint8, device=dev))
+    w.plan(torch.from_numpy(m["qo_indptr"]), torch.from_numpy(m["kv_indptr"]), heads, heads, 128,
+           q_data_type=torch.bfloat16)
+    t = lambda a: torch.from_numpy(a).to(dev)
+    wl = w.decode(t(m["packed_info"]), t(m["packed_keep"]), t(m["info_indptr"]), t(m["keep_indptr"]))
+    n_rows, _ = wl.sizes()
+    n_cu = torch.cuda.get_device_properties(dev).multi_processor_count
+    assert 0 < n_rows <= 3 * n_cu
+    sched = wl.sched.cpu().numpy()
+    order = wl.order[:n_rows].cpu().numpy()
+    shares = wl.shares.cpu().numpy()
+    row_head = wl.row_head[:n_rows].cpu().numpy()
+    ptr = wl.kv_row_ptr[:n_rows + 1].cpu().numpy()
+    lens = (ptr[1:] - ptr[:-1]).astype(np.int64)
+    exp_order = np.argsort(row_head, kind="stable")
+    assert (order == exp_order).all()
+    cost = 3 + lens[exp_order]
+    start = np.concatenate([[0], np.cumsum(cost)])[:-1] + 3
+    total = int(cost.sum())
+    assert (shares[512:512 + n_rows] == start).all() and shares[512 + n_rows] == total + 3
+    max_n = int(lens.max())
+    share = max(-(-total // n_cu), (max_n + 2) // 3, 1)
+    assert list(sched[25:31]) == [max_n, 1, share, total, n_cu, n_rows]
+    assert (sched[16:25] == 0).all() and (sched[64:576] == 0).all()
+    assert [int(sched[x]) for x in range(9)] == [n_rows * x // 8 for x in range(9)]
+    end = start + lens[exp_order]
+    for j in range(n_cu):
+        first = int(np.searchsorted(end, j * share, side="right"))   # first row with end > j * share
+        assert shares[j] == first, j
+    # a row touches at most four shares
+    touched = (end - 1) // share - np.minimum(start, end - 1) // share + 1
+    assert touched.max() <= 4
