@@ -260,6 +260,18 @@ __global__ void __launch_bounds__(kThreads) sparse_fa_kernel(const FaParams p) {
   // while the rest of the workgroup finishes the current row
   struct RowInfo {
     int row, part, parts, slot, req, qb, head, q_begin, q_rows, kv_begin, kv_len, ptr0, nb;
+    float q_scale;  // fp8: dequantisation scale of the row's q block
+    int k_scale0;   // fp8: position of the request's first kv block in k_scale (the kv head's row)
+  };
+  // (fetched with the rest of the record: read in the row's prologue, they would wait behind every
+  // tile copy in flight)
+  auto fill_scales = [&](RowInfo& it) {
+    it.q_scale = 1.f;
+    it.k_scale0 = 0;
+    if constexpr (kFp8) {
+      it.q_scale = p.q_scale[static_cast<int64_t>(it.head) * p.n_q_blocks + p.q_blk_base[it.req] + it.qb];
+      it.k_scale0 = (it.head / p.kv_group) * p.n_kv_blocks + p.kv_blk_base[it.req];
+    }
   };
   __shared__ RowInfo s_next_row[2];
   __shared__ int s_arrived;
@@ -267,6 +279,9 @@ __global__ void __launch_bounds__(kThreads) sparse_fa_kernel(const FaParams p) {
   __shared__ int s_share[1];   // even shares: items of this workgroup's share handed out so far
   __shared__ RowInfo s_items[kItemBatch];  // even shares: records of the share's next items
   __shared__ uint16_t s_blk2[2][kMaxRowBlocks];  // kv block list of this row / the next one
+  // fp8: the k dequantisation scales of the listed blocks (read per tile: from global memory the
+  // compiler would wait for every tile copy in flight along with them)
+  __shared__ float s_ksc2[2][kFp8 ? kMaxRowBlocks : 1];
 
   const int tid = threadIdx.x, lane = tid & 63;
   const int wv = __builtin_amdgcn_readfirstlane(tid >> 6);  // wavefront index, kept scalar
@@ -359,6 +374,7 @@ __global__ void __launch_bounds__(kThreads) sparse_fa_kernel(const FaParams p) {
           const int blk_lo = max(a, u) - u, blk_hi = min(min(b, e) - u, kMaxRowBlocks);
           it.ptr0 = p.kv_row_ptr[w] + blk_lo;
           it.nb = max(blk_hi - blk_lo, 0);
+          fill_scales(it);
         }
       }
       s_items[lane] = it;
@@ -398,13 +414,19 @@ __global__ void __launch_bounds__(kThreads) sparse_fa_kernel(const FaParams p) {
         ri.q_rows = min(kBlockQ, p.qo_indptr[ri.req + 1] - ri.q_begin);
         ri.kv_begin = p.kv_indptr[ri.req];
         ri.kv_len = p.kv_indptr[ri.req + 1] - ri.kv_begin;
+        fill_scales(ri);
       }
       s_next_row[slot_idx] = ri;
     }
     const int row = __builtin_amdgcn_readfirstlane(ri.row);
     if (row >= 0) {
       const int list0 = __builtin_amdgcn_readfirstlane(ri.ptr0), n = __builtin_amdgcn_readfirstlane(ri.nb);
-      for (int i = lane; i < n; i += 64) s_blk2[slot_idx][i] = static_cast<uint16_t>(p.kv_idx[list0 + i]);
+      const int ks0 = __builtin_amdgcn_readfirstlane(ri.k_scale0);
+      for (int i = lane; i < n; i += 64) {
+        const int blk = p.kv_idx[list0 + i];
+        s_blk2[slot_idx][i] = static_cast<uint16_t>(blk);
+        if constexpr (kFp8) s_ksc2[slot_idx][i] = p.k_scale[ks0 + blk];
+      }
     }
     // (everything fetched has been used; said explicitly so that the compiler does not carry these
     // loads as pending to the top of the row loop and wait there, behind the previous row's stores)
@@ -492,10 +514,9 @@ __global__ void __launch_bounds__(kThreads) sparse_fa_kernel(const FaParams p) {
     // softmax scale in the log2 domain; with fp8 operands the per-block dequantisation scales of
     // q (one per row of the list) and k (one per kv block) are folded in tile by tile
     float cq = c;
-    if constexpr (kFp8) cq *= p.q_scale[static_cast<int64_t>(head) * p.n_q_blocks + p.q_blk_base[req] + qb];
-    const float* ksc = nullptr;
+    if constexpr (kFp8) cq *= __builtin_bit_cast(float, __builtin_amdgcn_readfirstlane(__builtin_bit_cast(int, ri.q_scale)));
     const int kv_head = head / p.kv_group;
-    if constexpr (kFp8) ksc = p.k_scale + static_cast<int64_t>(kv_head) * p.n_kv_blocks + p.kv_blk_base[req];
+    const float* const s_ksc = s_ksc2[row_it & 1];
 
     f32x16 o_acc[4];
 #pragma unroll
@@ -717,7 +738,7 @@ __global__ void __launch_bounds__(kThreads) sparse_fa_kernel(const FaParams p) {
       if (it + 2 < my_tiles) copy_k(it + 2);
       const int valid = tile_valid(it);
       float cs = cq;
-      if constexpr (kFp8) cs = cq * ksc[s_blk[it]];
+      if constexpr (kFp8) cs = cq * s_ksc[it];
       const uint8_t* vs_base = group_smem + (it & 1) * kStageBytes + kKBytes;
 #pragma unroll
       for (int kk = 0; kk < 4; ++kk) {
