@@ -580,17 +580,24 @@ __global__ void __launch_bounds__(kThreads) gemm_kernel(const GemmParams p) {
       if constexpr (!kReduce) {
         if (p.y8) {
           if (p.bias_kind == FO_BIAS_VECTOR) {
+            // all sixteen pieces requested before the first is used (taken one by one, each load
+            // waits for the one before it and for the trailing tile copies)
+            x4 bvs[NT * 4];
 #pragma unroll
             for (int nt = 0; nt < NT; ++nt)
 #pragma unroll
-              for (int i4 = 0; i4 < 4; ++i4) {
-                const x4 bv = *reinterpret_cast<const x4*>(static_cast<const T*>(p.bias) + n0 + nt * 32 +
-                                                           i4 * 8 + wg * 4);
+              for (int i4 = 0; i4 < 4; ++i4)
+                bvs[nt * 4 + i4] = *reinterpret_cast<const x4*>(static_cast<const T*>(p.bias) + n0 + nt * 32 +
+                                                                i4 * 8 + wg * 4);
+            __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+            for (int nt = 0; nt < NT; ++nt)
+#pragma unroll
+              for (int i4 = 0; i4 < 4; ++i4)
 #pragma unroll
                 for (int mt = 0; mt < MT; ++mt)
 #pragma unroll
-                  for (int j = 0; j < 4; ++j) acc[nt][mt][i4 * 4 + j] += static_cast<float>(bv[j]);
-              }
+                  for (int j = 0; j < 4; ++j) acc[nt][mt][i4 * 4 + j] += static_cast<float>(bvs[nt * 4 + i4][j]);
             bias_added = true;
           }
           float amax = 0.f;
