@@ -653,12 +653,23 @@ __global__ void __launch_bounds__(kThreads) gemm_kernel(const GemmParams p) {
             bm[i] = *reinterpret_cast<const BiasVec*>(static_cast<const BiasT*>(p.bias) + off);
           }
         }
+        // four rows are read back and biased before the first of them is stored (row by row, every
+        // read waited for the stores before it: one memory counter for loads and stores)
+        f32x4 vals[4];
 #pragma unroll
         for (int i = 0; i < 16; ++i) {
           const int row = i * 2 + rsub;
-          f32x4 v = *reinterpret_cast<const f32x4*>(region + row * 512 + ((col4 ^ row) << 4));
+          if ((i & 3) == 0) {  // four rows at a time
 #pragma unroll
-          for (int j = 0; j < 4; ++j) v[j] += has_matrix ? static_cast<float>(bm[i][j]) : bvec[j];
+            for (int k = 0; k < 4; ++k) {
+              const int rk = (i + k) * 2 + rsub;
+              vals[k] = *reinterpret_cast<const f32x4*>(region + rk * 512 + ((col4 ^ rk) << 4));
+#pragma unroll
+              for (int j = 0; j < 4; ++j) vals[k][j] += has_matrix ? static_cast<float>(bm[i + k][j]) : bvec[j];
+            }
+            __builtin_amdgcn_sched_barrier(0);
+          }
+          const f32x4 v = vals[i & 3];
           const int grow = row_base + row;
           if (grow < p.m) {
             const int64_t off = y_batch + static_cast<int64_t>(grow) * p.n + n0 + col4 * 4;
