@@ -14,7 +14,7 @@
 // sched[0..8] delimit the 8 per-XCD queues inside `order`, sched[16..23] are the queue cursors,
 // sched[24] a completion counter (all cleared here) and sched[25] the longest row's kv count.  The
 // order inside a length class is not deterministic (atomic cursors); results do not depend on it.
-// With at most three rows per workgroup of the attention kernel (and a share table to fill) the
+// With at most two rows per workgroup of the attention kernel (and a share table to fill) the
 // layout is different, "even shares": see the scan kernel.
 // Integer work, bounded by HBM traffic and launch latency; bit-exact by construction.
 //
@@ -36,9 +36,10 @@ constexpr int kSchedEven = 26, kSchedShare = 27, kSchedTotal = 28, kSchedShares 
               kSchedArrived = 64;
 constexpr int kMaxShares = 512;      // arrival counters in `sched`, first-row entries in `shares`
 constexpr int kMaxSplitParts = 4;    // a row is cut into at most this many parts
-constexpr int kEvenMaxRounds = 3;    // even shares when there are at most this many rows per workgroup
-                                     // (measured: from ~5 rows per workgroup on, the queues balance as well
-                                     // and adapt to the workgroups' actual speeds, which fixed shares cannot)
+constexpr int kEvenMaxRounds = 2;    // even shares when there are at most this many rows per workgroup.
+// (Measured: at 2.5 rows per workgroup even shares are 2 % ahead of the queues but miss the L2 3.7 times as
+// often, three heads' K and V being live in every XCD at once; from ~5 rows on the queues balance as well and
+// adapt to the workgroups' actual speeds, which fixed shares cannot.)
 constexpr int kRowOverhead = 3;      // fixed cost of a row (prologue, epilogue) in units of one kv block
 
 // number of length classes for num_heads heads (32 up to 256 heads)

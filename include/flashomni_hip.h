@@ -95,7 +95,7 @@ int fo_prefill_plan(void* float_ws, size_t float_ws_bytes, void* int_ws_dev, voi
  *                    the longest row; sched[26..30] = even shares: in use, cost share of a
  *                    workgroup, total cost, number of shares, number of rows;
  *                    sched[64..575] = arrival counters of rows cut at share boundaries (cleared)
- * shares (optional, [512 + n_blk*H + 1] int32): when given and the list holds at most 3 rows per
+ * shares (optional, [512 + n_blk*H + 1] int32): when given and the list holds at most 2 rows per
  * CU, the decoder lays out even shares instead: `order` then lists the rows head by head (q blocks
  * ascending: a fixed order), a row costs 3 + its kv blocks, shares[512 + i] is the cost at which the
  * kv blocks of row order[i] begin, share j is the cost range [j*sched[27], (j+1)*sched[27]) and

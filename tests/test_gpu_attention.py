@@ -320,7 +320,7 @@ def _split_case(dev, ql, kl, heads, seed, share, dtype=torch.bfloat16, pk=0.6):
     ([1024], [4096], 2),             # 16 rows of ~19 blocks: every row cut in up to four parts
     ([1536], [2048 + 77], 8),        # 96 rows, ragged kv tail in a last part
     ([128 * 9], [128 * 9], 1),       # 9 short rows in one head
-    ([2304, 1000], [2304, 1500], 24),  # 2.6 rows per CU: most workgroups end in a shared row
+    ([1536, 640], [2304, 1500], 24),   # 1.6 rows per CU: most workgroups end in a shared row
 ])
 def test_rows_shared_between_workgroups(dev, case):
     """Few rows per CU: the decoder lays out even shares, rows that straddle a share boundary are
