@@ -53,8 +53,8 @@ class DecodedWorkList:
 
     ``row_req/row_qb/row_head[n_rows]``, ``kv_row_ptr[n_rows+1]``, ``kv_idx[nnz]``, all int32;
     ``counts = [n_rows, nnz, 0, 0]``; ``order[n_rows]`` / ``sched[1024]`` are the execution order
-    and queue words the attention kernel schedules from, ``shares`` the table of even shares it
-    uses instead when there are only a few rows per CU.  The sizes live on the device;
+    and queue words the attention kernel schedules from; ``shares`` holds one record per queue
+    entry or, when there are only a few rows per CU, the table of even shares used instead.  The sizes live on the device;
     ``sizes()`` copies them back (one synchronisation) for tests and reports."""
 
     def __init__(self, max_rows: int, max_nnz: int, num_heads: int, device):
@@ -68,7 +68,7 @@ class DecodedWorkList:
         self.counts = torch.zeros(4, dtype=torch.int32, device=device)
         self.order = torch.empty(n, dtype=torch.int32, device=device)
         self.sched = torch.zeros(1024, dtype=torch.int32, device=device)
-        self.shares = torch.zeros(512 + n + 1, dtype=torch.int32, device=device)
+        self.shares = torch.zeros(512 + 8 * (n + 1), dtype=torch.int32, device=device)
         self.scratch = torch.empty(2 * n + 8192, dtype=torch.int32, device=device)
 
     def sizes(self) -> Tuple[int, int]:

@@ -33,7 +33,8 @@ constexpr int kXcds = 8;
 constexpr int kHistSlots = 8192;  // (head, length class) counters of the order layout
 // even shares (see the attention kernel): words of `sched` and limits
 constexpr int kSchedEven = 26, kSchedShare = 27, kSchedTotal = 28, kSchedShares = 29, kSchedRows = 30,
-              kSchedArrived = 64;
+              kSchedRecords = 31, kSchedArrived = 64;
+constexpr int kRecordInts = 8;  // queue entry: row, request, q block, head, first kv slot, kv count, pad, pad
 constexpr int kMaxShares = 512;      // arrival counters in `sched`, first-row entries in `shares`
 constexpr int kMaxSplitParts = 4;    // a row is cut into at most this many parts
 constexpr int kEvenMaxRounds = 2;    // even shares when there are at most this many rows per workgroup.
@@ -323,6 +324,9 @@ __global__ void __launch_bounds__(kScanThreads) decode_scan_kernel(
       sched[kXcds] = total;
       for (int i = kXcds + 1; i < 32; ++i) sched[i] = 0;
       sched[25] = max_n;
+      // with a share table the fill kernel also leaves one record per queue entry there (what the
+      // attention kernel needs to start a row: one load after the pop instead of three rounds)
+      sched[kSchedRecords] = shares != nullptr ? 1 : 0;
     }
   }
 }
@@ -337,7 +341,8 @@ __global__ void __launch_bounds__(kCountThreads) decode_fill_kernel(
     int32_t* __restrict__ row_qb, int32_t* __restrict__ row_head,
     int32_t* __restrict__ kv_row_ptr, int32_t* __restrict__ kv_idx,
     int32_t* __restrict__ head_cursor, int32_t* __restrict__ order,
-    const int32_t* __restrict__ counts, const int32_t* __restrict__ sched) {
+    const int32_t* __restrict__ counts, const int32_t* __restrict__ sched,
+    int32_t* __restrict__ shares) {
   const int lane = threadIdx.x % kWave;
   const int64_t c = static_cast<int64_t>(blockIdx.x) * (kCountThreads / kWave) + threadIdx.x / kWave;
   if (c >= n_cand) return;
@@ -353,8 +358,16 @@ __global__ void __launch_bounds__(kCountThreads) decode_fill_kernel(
     kv_row_ptr[pos] = out;
     const int32_t listed = (c + 1 < n_cand ? kv_pos[c + 1] : counts[1]) - out;  // kv blocks of this row
     const int n_classes = len_classes(num_heads);
-    if (!sched[kSchedEven])  // (with even shares the scan kernel has written the order)
-      order[atomicAdd(&head_cursor[cd.head * n_classes + len_class(listed, sched[25], n_classes)], 1)] = pos;
+    if (!sched[kSchedEven]) {  // (with even shares the scan kernel has written the order)
+      const int32_t at = atomicAdd(&head_cursor[cd.head * n_classes + len_class(listed, sched[25], n_classes)], 1);
+      order[at] = pos;
+      if (shares) {
+        typedef __attribute__((ext_vector_type(4))) int i32x4;
+        i32x4* rec = reinterpret_cast<i32x4*>(shares + kMaxShares + kRecordInts * static_cast<int64_t>(at));
+        rec[0] = i32x4{pos, cd.req, cd.qb, cd.head};
+        rec[1] = i32x4{out, listed, 0, 0};
+      }
+    }
   }
   if (cd.nkv <= 0) return;
   if (is_full) {
@@ -401,6 +414,7 @@ extern "C" int fo_decode_sparse(const uint8_t* sparse_info, const uint8_t* spars
                "decode: sparse_info, sparse_kv_info and their indptrs are required unless is_full");
   }
   FO_REQUIRE(blk_req && blk_qb && kv_indptr && scratch, "decode: null table");
+  FO_REQUIRE((reinterpret_cast<uintptr_t>(shares) & 15) == 0, "decode: shares must be 16-byte aligned");
   const int64_t n_cand = static_cast<int64_t>(n_blk) * num_heads;
   FO_REQUIRE(n_cand < (int64_t(1) << 31), "decode: too many (q-block, head) pairs");
   hipStream_t s = static_cast<hipStream_t>(stream);
@@ -426,7 +440,7 @@ extern "C" int fo_decode_sparse(const uint8_t* sparse_info, const uint8_t* spars
     decode_fill_kernel<<<grid, kCountThreads, 0, s>>>(
         sparse_info, sparse_kv_info, sparse_info_indptr, sparse_kv_info_indptr, blk_req, blk_qb,
         kv_indptr, n_cand, num_heads, block_kv, is_full, act, cnt, row_req, row_qb, row_head,
-        kv_row_ptr, kv_idx, head_cursor, order, counts, sched);
+        kv_row_ptr, kv_idx, head_cursor, order, counts, sched, shares);
     FO_CHECK_LAUNCH();
   }
   return FO_OK;

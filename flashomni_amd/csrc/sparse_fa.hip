@@ -197,8 +197,10 @@ __device__ __forceinline__ float max_across_halves(float x) {
 
 // words of `sched` (written by the decoder): [0..8] queue bounds inside `order`, [16..23] queue
 // cursors, [24] completion counter; [26] even shares in use, [27] cost share of a workgroup, [28]
-// total cost, [29] number of shares, [30] number of rows; [64..575] arrival counters of the rows cut at share boundaries
+// total cost, [29] number of shares, [30] number of rows, [31] the share table holds one record per
+// queue entry; [64..575] arrival counters of the rows cut at share boundaries
 constexpr int kSchedEven = 26, kSchedArrived = 64;
+constexpr int kRecordInts = 8;  // queue entry record: row, request, q block, head, first kv slot, kv count
 constexpr int kMaxShares = 512, kMaxSplitParts = 4, kRowOverhead = 3;
 constexpr int kItemBatch = 16;  // item records of a share gathered at a time
 constexpr int kSplitPartFloats = 128 * 128 + 2 * 256;  // O (fp32) + (max, sum) per lane of kv group 0
@@ -226,7 +228,7 @@ __device__ __forceinline__ void load_pair_device(const float* p, float& a, float
 // Pop the next row for this workgroup from the queues: own XCD queue first, then the neighbours'.
 // `first` is the first queue that may still hold rows: a queue found empty stays empty for the rest
 // of the launch, so it is not asked again.  `q` is the launch's copy of the queue bounds: the pop
-// itself is one atomic and one load.  Returns the row's position in the canonical list or -1.
+// itself is one atomic.  Returns the entry's position in `order` or -1.
 __device__ __forceinline__ int pop_row(const FaParams& p, int xcd, const int* q, int* first) {
   for (int a = *first; a < kXcds; ++a) {
     const int x = (xcd + a) & (kXcds - 1);
@@ -235,7 +237,7 @@ __device__ __forceinline__ int pop_row(const FaParams& p, int xcd, const int* q,
       const int pos = beg + atomicAdd(&p.sched[16 + x], 1);
       if (pos < end) {
         *first = a;
-        return p.order[pos];
+        return pos;
       }
     }
   }
@@ -325,7 +327,7 @@ __global__ void __launch_bounds__(kThreads) sparse_fa_kernel(const FaParams p) {
   // The next row is popped by kv group 1 while kv group 0 combines and stores the current one
   // (group 1 has nothing else to do then), so the queue atomics are off the critical path.
   if (tid < 9) s_queue[tid] = p.sched[tid];
-  if (tid >= 64 && tid < 64 + 5) s_queue[9 + tid - 64] = p.sched[kSchedEven + tid - 64];
+  if (tid >= 64 && tid < 64 + 6) s_queue[9 + tid - 64] = p.sched[kSchedEven + tid - 64];
   __syncthreads();
   // Even shares: the decoder has laid the rows out head by head and given every row a cost
   // (kRowOverhead + its kv blocks); share j is the cost range [j * share, (j + 1) * share), and a
@@ -380,6 +382,7 @@ __global__ void __launch_bounds__(kThreads) sparse_fa_kernel(const FaParams p) {
       s_items[lane] = it;
     }
   };
+  const bool have_records = s_queue[14] != 0 && p.shares != nullptr;
   int first_queue = 0;  // kept by the popping lane (the first pop is lane 0's, the others lane 256's)
   // One wavefront: lane 0 takes the next item (even shares: from the gathered records; otherwise it
   // pops a row and gathers its metadata, two rounds of loads), then all lanes copy the row's kv
@@ -398,18 +401,31 @@ __global__ void __launch_bounds__(kThreads) sparse_fa_kernel(const FaParams p) {
         s_next_row[slot_idx] = ri;
       }
     } else if (lane == 0) {
-      const int w = pop_row(p, blockIdx.x & (kXcds - 1), s_queue, &first_queue);
-      ri.row = w;
+      const int at = pop_row(p, blockIdx.x & (kXcds - 1), s_queue, &first_queue);
       ri.part = 0;
       ri.parts = 1;
       ri.slot = 0;
-      if (w >= 0) {
-        ri.req = p.row_req[w];
-        ri.qb = p.row_qb[w];
-        ri.head = p.row_head[w];
-        ri.ptr0 = p.kv_row_ptr[w];
-        // (a row longer than the LDS list is cut; the host side refuses such requests at plan time)
-        ri.nb = min(p.kv_row_ptr[w + 1] - ri.ptr0, kMaxRowBlocks);
+      if (at >= 0) {
+        if (have_records) {
+          // one record per queue entry, left by the decoder: one round of loads after the pop
+          const i32x4* rec = reinterpret_cast<const i32x4*>(p.shares + kMaxShares + kRecordInts * static_cast<int64_t>(at));
+          const i32x4 r0 = rec[0], r1 = rec[1];
+          ri.row = r0[0];
+          ri.req = r0[1];
+          ri.qb = r0[2];
+          ri.head = r0[3];
+          ri.ptr0 = r1[0];
+          ri.nb = min(r1[1], kMaxRowBlocks);
+        } else {
+          const int w = p.order[at];
+          ri.row = w;
+          ri.req = p.row_req[w];
+          ri.qb = p.row_qb[w];
+          ri.head = p.row_head[w];
+          ri.ptr0 = p.kv_row_ptr[w];
+          // (a row longer than the LDS list is cut; the host side refuses such requests at plan time)
+          ri.nb = min(p.kv_row_ptr[w + 1] - ri.ptr0, kMaxRowBlocks);
+        }
         ri.q_begin = p.qo_indptr[ri.req] + ri.qb * kBlockQ;
         ri.q_rows = min(kBlockQ, p.qo_indptr[ri.req + 1] - ri.q_begin);
         ri.kv_begin = p.kv_indptr[ri.req];

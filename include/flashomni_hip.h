@@ -93,17 +93,22 @@ int fo_prefill_plan(void* float_ws, size_t float_ws_bytes, void* int_ws_dev, voi
  *   sched [1024]     sched[0..8] = queue boundaries inside `order`, sched[16..23] = queue cursors
  *                    and sched[24] = completion counter, both cleared to 0; sched[25] = kv count of
  *                    the longest row; sched[26..30] = even shares: in use, cost share of a
- *                    workgroup, total cost, number of shares, number of rows;
+ *                    workgroup, total cost, number of shares, number of rows; sched[31] = the
+ *                    share table holds queue-entry records;
  *                    sched[64..575] = arrival counters of rows cut at share boundaries (cleared)
- * shares (optional, [512 + n_blk*H + 1] int32): when given and the list holds at most 2 rows per
- * CU, the decoder lays out even shares instead: `order` then lists the rows head by head (q blocks
- * ascending: a fixed order), a row costs 3 + its kv blocks, shares[512 + i] is the cost at which the
- * kv blocks of row order[i] begin, share j is the cost range [j*sched[27], (j+1)*sched[27]) and
- * shares[j] its first row.  The attention kernel gives every workgroup one share and computes a
- * row that straddles a boundary in parts (consecutive ranges of its kv blocks, at most 4), one per
- * share it touches (the counterpart of the reference's split-kv plan, scheduler.cuh:35-64, decided
- * on the device from the decoded list).  The queues stay valid (eight equal runs of `order`), and
- * the canonical lists do not change.
+ * shares (optional, [512 + 8*(n_blk*H + 1)] int32, 16-byte aligned): scheduling table for the
+ * attention kernel, to be passed to fo_sparse_fa_run with the list.  Normally (sched[31] = 1) it
+ * receives one 8-int record per entry of `order`, at shares[512 + 8*i]: row, request, q block,
+ * head, first kv_idx slot, kv block count, 0, 0, so that a popped entry costs the attention kernel
+ * one load instead of three dependent rounds.  When the list holds at most 2 rows per CU the
+ * decoder lays out even shares instead (sched[26] = 1): `order` then lists the rows head by head
+ * (q blocks ascending: a fixed order), a row costs 3 + its kv blocks, shares[512 + i] is the cost
+ * at which the kv blocks of row order[i] begin, share j is the cost range
+ * [j*sched[27], (j+1)*sched[27]) and shares[j] its first row.  The attention kernel gives every
+ * workgroup one share and computes a row that straddles a boundary in parts (consecutive ranges
+ * of its kv blocks, at most 4), one per share it touches (the counterpart of the reference's
+ * split-kv plan, scheduler.cuh:35-64, decided on the device from the decoded list).  The queues
+ * stay valid (eight equal runs of `order`), and the canonical lists do not change.
  * is_full != 0 ignores the symbol tensors (which may be NULL) and lists everything
  * (csrc/batch_sparseFA.cu:123-128).
  * `scratch` needs 2*n_blk*H + 8192 int32.
@@ -140,8 +145,8 @@ int fo_decode_sparse(const uint8_t* sparse_info, const uint8_t* sparse_kv_info,
  * Rows are taken from the queues described by `order` / `sched` (see fo_decode_sparse); the
  * kernel leaves the queue cursors rewound, so one decoded list can be run any number of times,
  * but two launches sharing one `sched` must not overlap in time.
- * shares: the table fo_decode_sparse filled for this list, or NULL.  With it (and when the decoder
- * chose even shares) every workgroup computes one share; split_workspace, device memory of
+ * shares: the table fo_decode_sparse filled for this list, or NULL.  With it a popped queue entry
+ * is read as one record; when the decoder chose even shares every workgroup computes one share; split_workspace, device memory of
  * fo_sparse_fa_split_workspace_bytes() bytes (two areas per CU), 16-byte aligned, is then required
  * and receives the unnormalised partial results (fp32 O, row maximum, row sum) of rows cut at share
  * boundaries: the part that arrives last combines them in part order (replaces the reference's

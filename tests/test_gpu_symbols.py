@@ -184,3 +184,30 @@ def test_decoder_even_shares(dev, case):
     # a row touches at most four shares
     touched = (end - 1) // share - np.minimum(start, end - 1) // share + 1
     assert touched.max() <= 4
+
+
+def test_decoder_queue_records(dev):
+    """More than two rows per CU and a share table: the queues are laid out as without one, and the
+    table holds one record per queue entry (row, request, q block, head, first kv slot, kv count)."""
+    import flashomni_amd as fo
+    ql, kl, heads, pa, pk = [4608, 1000], [4608, 700], 24, 0.75, 0.5
+    m = make_ragged_masks(ql, kl, heads, pa, pk, seed=7)
+    w = fo.BatchFlashOmniFAWithRaggedKVWrapper(torch.empty(128 << 20, dtype=torch.uint8, device=dev))
+    w.plan(torch.from_numpy(m["qo_indptr"]), torch.from_numpy(m["kv_indptr"]), heads, heads, 128,
+           q_data_type=torch.bfloat16)
+    t = lambda a: torch.from_numpy(a).to(dev)
+    wl = w.decode(t(m["packed_info"]), t(m["packed_keep"]), t(m["info_indptr"]), t(m["keep_indptr"]))
+    n_rows, _ = wl.sizes()
+    n_cu = torch.cuda.get_device_properties(dev).multi_processor_count
+    assert n_rows > 2 * n_cu
+    sched = wl.sched.cpu().numpy()
+    assert sched[26] == 0 and sched[31] == 1 and sched[8] == n_rows
+    order = wl.order[:n_rows].cpu().numpy()
+    rec = wl.shares.cpu().numpy()[512:512 + 8 * n_rows].reshape(n_rows, 8)
+    ptr = wl.kv_row_ptr[:n_rows + 1].cpu().numpy()
+    assert sorted(order.tolist()) == list(range(n_rows))
+    assert (rec[:, 0] == order).all()
+    assert (rec[:, 1] == wl.row_req[:n_rows].cpu().numpy()[order]).all()
+    assert (rec[:, 2] == wl.row_qb[:n_rows].cpu().numpy()[order]).all()
+    assert (rec[:, 3] == wl.row_head[:n_rows].cpu().numpy()[order]).all()
+    assert (rec[:, 4] == ptr[order]).all() and (rec[:, 5] == ptr[order + 1] - ptr[order]).all()
