@@ -67,6 +67,7 @@ constexpr int kMaxHeads = 256;
 constexpr int kMaxSteps = 2048;  // GEMM-O: k steps of one work item (K <= 65536)
 constexpr int kXcds = 8;
 constexpr int kListThreads = 1024;
+constexpr int kInlineCells = 512;  // up to this many cells the GEMM-Q kernel lists its quads itself
 constexpr int kWindow = 16;   // token blocks per scheduling window
 constexpr int kQuadInts = 8;  // b, r0, r1, c0, c1, valid mask, pad, pad
 
@@ -100,6 +101,8 @@ struct GemmParams {
                          // quads are enumerated arithmetically (GEMM-O, GEMM-Q with is_full)
   const int32_t* qoff;   // qoff[0..8] queue boundaries inside `quads`
   int32_t n_row_tiles, n_col_tiles, n_cp;  // geometry for the arithmetic enumeration
+  int32_t n_win;         // windows of 16 token blocks per batch
+  int32_t inline_cells;  // > 0: GEMM-Q builds its quad list itself from the flags of this many cells
   int32_t batch, m, n, k;
   int32_t sparse_q_size, num_heads, head_dim, num_text_tokens;
   int32_t flag;       // GEMM-Q: is_full.  GEMM-O: is_for_cached
@@ -126,7 +129,7 @@ __device__ __forceinline__ bool flag_bit(const uint8_t* info, uint32_t bit) {
 // Quad list.  A cell = (batch, window of 16 token blocks, column pair); cells are ordered batch,
 // window, column pair.  One workgroup counts the quads of every cell (flagged-row masks of its two
 // columns), scans the counts, emits every cell's quads at its offset, and cuts the list into eight
-// contiguous, equally long queues.
+// contiguous, equally long queues.  (Up to kInlineCells cells the GEMM-Q kernel does the same itself.)
 // ---------------------------------------------------------------------------------------------
 struct ListGeom {
   int32_t batch, n_row_tiles, n_col_tiles, n_win, n_cp;  // windows per batch, column pairs
@@ -289,6 +292,12 @@ __global__ void __launch_bounds__(kThreads) gemm_kernel(const GemmParams p) {
   // GEMM-O: per k step, k offset | (row0 selects) << 16 | (row1 selects) << 17; four entries past
   // the end repeat the last step
   __shared__ int32_t s_step[kReduce ? kMaxSteps + 4 : 1];
+  // GEMM-Q listing its own quads (short launches: saves the list kernel's launch): quad count
+  // prefix and flagged-row masks of every cell, and the entry picked for the current work item
+  __shared__ int32_t s_cell_pref[kReduce ? 1 : kInlineCells + 1];
+  __shared__ uint32_t s_cell_mask[kReduce ? 1 : 2 * kInlineCells];
+  __shared__ int32_t s_cell_wave[kThreads / 64];
+  __shared__ int32_t s_entry[8];
 
   const int tid = threadIdx.x, lane = tid & 63;
   const int wv = __builtin_amdgcn_readfirstlane(tid >> 6);  // wavefront index, kept scalar
@@ -321,7 +330,49 @@ __global__ void __launch_bounds__(kThreads) gemm_kernel(const GemmParams p) {
   const int last_q = (last_rows + 1) / 2;
   const int quads_per_batch = (full_w * (kWindow / 2) + last_q) * p.n_cp;
   int q_lo, q_len;
-  if (p.quads) {
+  bool inline_list = false;
+  if constexpr (!kReduce) inline_list = p.inline_cells > 0;
+  if (inline_list) {
+    if constexpr (!kReduce) {
+      // thread = cell: masks, quad count, workgroup-wide inclusive scan of the counts
+      ListGeom gm;
+      gm.batch = p.batch;
+      gm.n_row_tiles = p.n_row_tiles;
+      gm.n_col_tiles = p.n_col_tiles;
+      gm.n_win = p.n_win;
+      gm.n_cp = p.n_cp;
+      int32_t cnt = 0;
+      if (tid < p.inline_cells) {
+        int b, row0, cp;
+        uint32_t m0, m1;
+        cell_masks(gm, tid, true, p.sparse_info, p.sparse_info_indptr, p.sparse_q_size, p.num_heads,
+                   p.head_dim, p.num_text_tokens, &b, &row0, &cp, &m0, &m1);
+        for_each_quad(m0, m1, [&](int, int, int) { ++cnt; });
+        s_cell_mask[2 * tid] = m0;
+        s_cell_mask[2 * tid + 1] = m1;
+      }
+      int32_t incl = cnt;
+#pragma unroll
+      for (int d = 1; d < 64; d <<= 1) {
+        const int32_t up = __shfl_up(incl, d, 64);
+        if (lane >= d) incl += up;
+      }
+      if (lane == 63) s_cell_wave[wv] = incl;
+      __syncthreads();
+      int32_t base = 0, total = 0;
+#pragma unroll
+      for (int w = 0; w < kThreads / 64; ++w) {
+        const int32_t t = s_cell_wave[w];
+        if (w < wv) base += t;
+        total += t;
+      }
+      if (tid < kInlineCells) s_cell_pref[tid + 1] = base + incl;
+      if (tid == 0) s_cell_pref[0] = 0;
+      q_lo = static_cast<int>(static_cast<int64_t>(total) * xcd / kXcds);
+      q_len = static_cast<int>(static_cast<int64_t>(total) * (xcd + 1) / kXcds) - q_lo;
+      __syncthreads();
+    }
+  } else if (p.quads) {
     q_lo = p.qoff[xcd];
     q_len = p.qoff[xcd + 1] - q_lo;
   } else {
@@ -332,7 +383,35 @@ __global__ void __launch_bounds__(kThreads) gemm_kernel(const GemmParams p) {
 
   for (int work = slot; work < q_len; work += per_xcd) {
     int bz, valid, r[2], c[2];
-    if (p.quads) {
+    if (inline_list) {
+      if constexpr (!kReduce) {
+        // the thread whose cell holds quad q_lo + work walks the cell's quads up to it
+        const int q = q_lo + work;
+        if (tid < p.inline_cells && s_cell_pref[tid] <= q && q < s_cell_pref[tid + 1]) {
+          const int cp = tid % p.n_cp, t = tid / p.n_cp;
+          const int w = t % p.n_win, b = t / p.n_win;
+          int k = q - s_cell_pref[tid];
+          for_each_quad(s_cell_mask[2 * tid], s_cell_mask[2 * tid + 1], [&](int r0, int r1, int v) {
+            if (k == 0) {
+              s_entry[0] = b;
+              s_entry[1] = w * kWindow + r0;
+              s_entry[2] = w * kWindow + (r1 < 0 ? r0 : r1);
+              s_entry[3] = (v & 0x5) ? 2 * cp : 2 * cp + 1;
+              s_entry[4] = (v & 0xA) ? 2 * cp + 1 : 2 * cp;
+              s_entry[5] = v;
+            }
+            --k;
+          });
+        }
+        __syncthreads();
+        bz = s_entry[0];
+        r[0] = s_entry[1];
+        r[1] = s_entry[2];
+        c[0] = s_entry[3];
+        c[1] = s_entry[4];
+        valid = s_entry[5];
+      }
+    } else if (p.quads) {
       const int32_t* e = p.quads + kQuadInts * static_cast<int64_t>(q_lo + work);
       bz = e[0];
       r[0] = e[1];
@@ -736,6 +815,8 @@ int launch(GemmParams& p, const ListGeom& gm, bool use_flags, void* workspace, h
   p.n_row_tiles = gm.n_row_tiles;
   p.n_col_tiles = gm.n_col_tiles;
   p.n_cp = gm.n_cp;
+  p.n_win = gm.n_win;
+  p.inline_cells = 0;
   int num_cu = fo_num_cu();
   if (num_cu <= 0) return fo::fail(FO_ERR_HIP, "gemm: no device");
   int64_t grid = (num_cu + kXcds - 1) / kXcds * kXcds;  // one persistent workgroup per CU
@@ -746,6 +827,16 @@ int launch(GemmParams& p, const ListGeom& gm, bool use_flags, void* workspace, h
     // every unit is computed: no list, the kernel enumerates the quads itself
     p.quads = nullptr;
     p.qoff = nullptr;
+    gemm_kernel<T, kReduce><<<static_cast<unsigned>(grid), kThreads, kSmemBytes, stream>>>(p);
+    FO_CHECK_LAUNCH();
+    return FO_OK;
+  }
+  const int64_t n_cells = static_cast<int64_t>(gm.batch) * gm.n_win * gm.n_cp;
+  if (!kReduce && n_cells <= kInlineCells) {
+    // short launch: the kernel lists its quads itself (one launch less)
+    p.quads = nullptr;
+    p.qoff = nullptr;
+    p.inline_cells = static_cast<int32_t>(n_cells);
     gemm_kernel<T, kReduce><<<static_cast<unsigned>(grid), kThreads, kSmemBytes, stream>>>(p);
     FO_CHECK_LAUNCH();
     return FO_OK;
