@@ -476,3 +476,23 @@ def test_two_wrappers_on_two_streams(dev):
     torch.cuda.synchronize()
     for out, (w, dev_args, out0, exp, m, heads, stream) in zip(outs, cases):
         _check(out.cpu(), exp, out0, m, heads)
+
+
+@pytest.mark.parametrize("seed", range(16))
+def test_random_ragged_batches(dev, seed):
+    """Seeded random batches (1-4 requests, ragged lengths down to one token, 1-12 heads, random
+    densities, either dtype, either layout; short lists, so the rows are cut into even shares)
+    against the oracle, lse included."""
+    rng = np.random.default_rng(1000 + seed)
+    n_req = int(rng.integers(1, 5))
+    ql = [int(rng.integers(1, 900)) for _ in range(n_req)]
+    kl = [int(rng.integers(1, 1400)) for _ in range(n_req)]
+    heads = int(rng.choice([1, 2, 3, 5, 8, 12]))
+    pa, pk = float(rng.choice([0.3, 0.7, 1.0])), float(rng.choice([0.1, 0.5, 0.9]))
+    dtype = torch.bfloat16 if seed % 2 == 0 else torch.float16
+    layout = "NHD" if seed % 3 else "HND"
+    out, exp, out0, m, lse, exp_lse = _run_case(dev, ql, kl, heads, dtype, seed=2000 + seed, pa=pa, pk=pk,
+                                                return_lse=True, layout=layout)
+    _check(out, exp, out0, m, heads)
+    ok = ~torch.isnan(exp_lse)
+    assert torch.allclose(lse[ok], exp_lse[ok], atol=2e-3, rtol=1e-3)
