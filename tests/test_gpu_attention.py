@@ -496,3 +496,34 @@ def test_random_ragged_batches(dev, seed):
     _check(out, exp, out0, m, heads)
     ok = ~torch.isnan(exp_lse)
     assert torch.allclose(lse[ok], exp_lse[ok], atol=2e-3, rtol=1e-3)
+
+
+def test_share_with_many_short_rows(dev):
+    """One long row (150 kv blocks, cut into parts) beside 80 rows without any kv block: the
+    long row sets the share size, so single shares hold more than sixteen of the short rows (their
+    records are gathered in batches of sixteen)."""
+    import flashomni_amd as fo
+    heads, ql, kl = 1, [128, 80 * 128], [150 * 128, 128]
+    info = [np.ones((1, 1), dtype=bool), np.ones((80, 1), dtype=bool)]
+    keep = [np.ones((1, 1, 150), dtype=bool), np.zeros((80, 1, 1), dtype=bool)]
+    pack = lambda parts: (np.concatenate([np.packbits(p.reshape(-1), bitorder="little") for p in parts]),
+                          np.cumsum([0] + [(p.size + 7) // 8 for p in parts]).astype(np.int32))
+    pinfo, info_ip = pack(info)
+    pkeep, keep_ip = pack(keep)
+    qo, kv = np.array([0, 128, 128 + 80 * 128], dtype=np.int32), np.array([0, 150 * 128, 151 * 128], dtype=np.int32)
+    g = torch.Generator().manual_seed(9)
+    q = torch.randn(int(qo[-1]), heads, 128, generator=g).to(torch.bfloat16)
+    k = torch.randn(int(kv[-1]), heads, 128, generator=g).to(torch.bfloat16)
+    v = torch.randn(int(kv[-1]), heads, 128, generator=g).to(torch.bfloat16)
+    t = lambda a: torch.from_numpy(a).to(dev)
+    w = fo.BatchFlashOmniFAWithRaggedKVWrapper(torch.empty(128 << 20, dtype=torch.uint8, device=dev))
+    w.plan(t(qo), t(kv), heads, heads, 128, q_data_type=torch.bfloat16)
+    out0 = sentinel_like(q.shape, torch.bfloat16)
+    out = out0.clone().to(dev)
+    w.run(q.to(dev), k.to(dev), v.to(dev), t(pinfo), t(pkeep), t(info_ip), t(keep_ip), out=out)
+    sched = w._worklist.sched.cpu().numpy()
+    assert sched[26] == 1 and sched[27] == 50 and sched[30] == 81   # share = ceil((150 + 2) / 3)
+    exp = oracle.sparse_attention(q, k, v, pinfo, pkeep, info_ip, keep_ip, qo, kv, out=out0.clone())
+    out = out.cpu()
+    assert float(out[128:].abs().max()) == 0.0 and float(exp[128:].abs().max()) == 0.0
+    assert max_abs(out[:128], exp[:128]) <= MAX_ABS and rel_l2(out[:128], exp[:128]) <= REL_L2
