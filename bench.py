@@ -26,7 +26,7 @@ import torch
 ROOT = os.path.dirname(os.path.abspath(__file__))
 sys.path.insert(0, ROOT)
 
-FA_C0_HBM_BYTES = 176.4e6  # measured, see the roofline entry
+FA_C0_HBM_BYTES = 184.8e6  # measured, see the roofline entry
 PEAK_BF16 = 2516.6   # TFLOP/s dense
 PEAK_FP8 = 5033.2
 PEAK_HBM = 8000.0    # GB/s
@@ -428,8 +428,8 @@ def main():
         "kernel": "sparse_fa_kernel<bf16> (config 0, FLUX shape)", "bound": "mfma",
         "achieved": round(fa_flops / (fa_ms * 1e-3) / 1e12, 2), "peak": PEAK_BF16, "unit": "TFLOP/s",
         "frac": round(fa_flops / (fa_ms * 1e-3) / 1e12 / PEAK_BF16, 4),
-        # HBM bytes per launch from two rocprofv3 --pmc runs of this command (FETCH_SIZE 68020.6 KiB x 2.0,
-        # the factor a 256 MiB copy kernel gives for that counter, + WRITE_SIZE 36182.5 KiB x 1.0);
+        # HBM bytes per launch from two rocprofv3 --pmc runs of this command (FETCH_SIZE 69946.3 KiB x 2.0,
+        # the factor a 256 MiB copy kernel gives for that counter, + WRITE_SIZE 40532.7 KiB x 1.0);
         # the algorithmic bytes of the launch are 98.6e6 (the excess is K/V re-fetched after falling out
         # of an XCD's L2, which three heads share)
         "traffic": FA_C0_HBM_BYTES if 0 in configs else None, "traffic_unit": "bytes/launch",
