@@ -804,11 +804,14 @@ int64_t workspace_ints(const ListGeom& gm, int64_t* max_quads_out) {
 
 template <typename T, bool kReduce>
 int launch(GemmParams& p, const ListGeom& gm, bool use_flags, void* workspace, hipStream_t stream) {
-  static bool attr_set = false;
-  if (!attr_set) {
+  // (the attribute belongs to the kernel's code object on one device: set once per device)
+  static bool attr_set[64] = {};
+  int dev = 0;
+  FO_HIP_CALL(hipGetDevice(&dev));
+  if (dev < 0 || dev >= 64 || !attr_set[dev]) {
     FO_HIP_CALL(hipFuncSetAttribute(reinterpret_cast<const void*>(&gemm_kernel<T, kReduce>),
                                     hipFuncAttributeMaxDynamicSharedMemorySize, kSmemBytes));
-    attr_set = true;
+    if (dev >= 0 && dev < 64) attr_set[dev] = true;
   }
   int64_t max_quads = 0;
   workspace_ints(gm, &max_quads);

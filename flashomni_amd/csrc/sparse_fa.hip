@@ -1129,11 +1129,14 @@ __global__ void __launch_bounds__(kThreads) sparse_fa_kernel(const FaParams p) {
 template <typename T, bool kFp8>
 int launch(const FaParams& p, int64_t max_rows, hipStream_t stream) {
   constexpr int kSmemBytes = Geom<kFp8>::kSmemBytes;
-  static bool attr_set = false;
-  if (!attr_set) {
+  // (the attribute belongs to the kernel's code object on one device: set once per device)
+  static bool attr_set[64] = {};
+  int dev = 0;
+  FO_HIP_CALL(hipGetDevice(&dev));
+  if (dev < 0 || dev >= 64 || !attr_set[dev]) {
     FO_HIP_CALL(hipFuncSetAttribute(reinterpret_cast<const void*>(&sparse_fa_kernel<T, kFp8>),
                                     hipFuncAttributeMaxDynamicSharedMemorySize, kSmemBytes));
-    attr_set = true;
+    if (dev >= 0 && dev < 64) attr_set[dev] = true;
   }
   int num_cu = fo_num_cu();
   if (num_cu <= 0) return fo::fail(FO_ERR_HIP, "sparse_fa: no device");
