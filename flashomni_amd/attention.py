@@ -112,7 +112,10 @@ class BatchFlashOmniFAWithRaggedKVWrapper:
         _check_kv_layout(kv_layout)
         self._kv_layout = kv_layout
         self._float_workspace_buffer = float_workspace_buffer
-        self._share_rows = True   # let short work lists cut rows into parts (needs the float workspace)
+        # give the decoder a share table (queue-entry records; even shares for short lists); needs a
+        # float workspace of fo_sparse_fa_split_workspace_bytes().  Read at plan() time.
+        self._share_rows = True
+        self._split_ok = False
         self.device = float_workspace_buffer.device
         if self.device.type != "cuda":
             raise ValueError("float_workspace_buffer must live on the GPU; there is no CPU path")
@@ -295,6 +298,7 @@ class BatchFlashOmniFAWithRaggedKVWrapper:
             self._worklist = DecodedWorkList(max_rows, max_nnz, num_qo_heads, self.device)
         self._max_rows = max_rows
         self._decode_key = None
+        self._split_ok = self._split_ws_ok()
 
         self._num_qo_heads = num_qo_heads
         self._num_kv_heads = num_kv_heads
@@ -373,7 +377,7 @@ class BatchFlashOmniFAWithRaggedKVWrapper:
             self._n_q_blk, self._num_qo_heads, self._sparse_block_size_for_kv, int(bool(is_full)),
             _lib.ptr(wl.row_req), _lib.ptr(wl.row_qb), _lib.ptr(wl.row_head), _lib.ptr(wl.kv_row_ptr),
             _lib.ptr(wl.kv_idx), _lib.ptr(wl.counts), _lib.ptr(wl.order), _lib.ptr(wl.sched),
-            _lib.ptr(wl.scratch), _lib.ptr(wl.shares if self._split_ws_ok() else None),
+            _lib.ptr(wl.scratch), _lib.ptr(wl.shares if self._split_ok else None),
             _lib.current_stream(self.device)))
         # the memo holds the tensors alive so a recycled address cannot alias the key
         self._decode_key = None if capturing else key
@@ -476,8 +480,8 @@ class BatchFlashOmniFAWithRaggedKVWrapper:
             _lib.ptr(wl.sched), self._max_rows, q.size(1), self._num_kv_heads, q.size(2),
             self._sparse_block_size_for_q,
             self._sparse_block_size_for_kv, float(sm_scale),
-            _lib.ptr(wl.shares if self._split_ws_ok() else None),
-            _lib.ptr(self._float_workspace_buffer) if self._split_ws_ok() else None,
+            _lib.ptr(wl.shares if self._split_ok else None),
+            _lib.ptr(self._float_workspace_buffer) if self._split_ok else None,
             self._float_ws_bytes(), _lib.current_stream(self.device)))
         return (out, lse) if return_lse else out
 
