@@ -32,6 +32,46 @@ def test_library_exports_every_declared_symbol():
     assert L.lib().fo_abi_version() == 1
 
 
+_C_SCALARS = {"int": ctypes.c_int, "int32_t": ctypes.c_int32, "uint32_t": ctypes.c_uint32,
+              "int64_t": ctypes.c_int64, "uint64_t": ctypes.c_uint64, "size_t": ctypes.c_size_t,
+              "float": ctypes.c_float, "double": ctypes.c_double}
+
+
+def test_ctypes_signatures_follow_the_header():
+    """Every parameter the header declares has a ctypes argument of the same kind and width in the
+    same position (a pointer or array -> a pointer-sized argument), and the return types agree: a
+    changed entry point cannot drift from its binding unnoticed."""
+    header = open(os.path.join(ROOT, "include", "flashomni_hip.h")).read()
+    header = re.sub(r"/\*.*?\*/", "", header, flags=re.S)
+    header = re.sub(r"//[^\n]*", "", header)
+    L = _lib()
+    seen = 0
+    for m in re.finditer(r"([A-Za-z_][A-Za-z0-9_ ]*?[\s\*]+)(fo_[a-z0-9_]+)\s*\(([^)]*)\)\s*;", header):
+        ret, name, args = m.group(1).strip(), m.group(2), m.group(3).strip()
+        params = [] if args in ("", "void") else [a.strip() for a in args.split(",")]
+        argtypes, restype = L.SIGNATURES[name]
+        assert len(params) == len(argtypes), name
+        for i, (decl, ct) in enumerate(zip(params, argtypes)):
+            if "*" in decl or "[" in decl:
+                assert ctypes.sizeof(ct) == ctypes.sizeof(ctypes.c_void_p) and ct in (
+                    ctypes.c_void_p, ctypes.c_char_p), (name, i, decl)
+                continue
+            words = [w for w in decl.split() if w not in ("const", "unsigned", "signed")]
+            want = _C_SCALARS[words[-2]]
+            assert ctypes.sizeof(ct) == ctypes.sizeof(want), (name, i, decl)
+            assert (ct in (ctypes.c_float, ctypes.c_double)) == (want in (ctypes.c_float, ctypes.c_double)), \
+                (name, i, decl)
+        ret_words = [w for w in ret.replace("*", " * ").split() if w not in ("const", "extern", "FO_API")]
+        if "*" in ret_words:
+            assert restype in (ctypes.c_char_p, ctypes.c_void_p), name
+        elif ret_words[-1] == "void":
+            assert restype is None, name
+        else:
+            assert ctypes.sizeof(restype) == ctypes.sizeof(_C_SCALARS[ret_words[-1]]), name
+        seen += 1
+    assert seen == len(L.SIGNATURES)
+
+
 def _plan(qo, kv, hq, hkv, d, num_cu=256, int_ws=8 << 20, float_ws=128 << 20, graph=False, total=None):
     L = _lib()
     qo_t, kv_t = torch.tensor(qo, dtype=torch.int32), torch.tensor(kv, dtype=torch.int32)
