@@ -26,7 +26,8 @@ import torch
 ROOT = os.path.dirname(os.path.abspath(__file__))
 sys.path.insert(0, ROOT)
 
-FA_C0_HBM_BYTES = 184.8e6  # measured, see the roofline entry
+TRAFFIC_PROFILE = os.path.join(ROOT, "profiles", "hbm_traffic_flux_layer_c0_c1_c2.txt")
+SETTLE_MS = 150.0    # load applied before any timing: an idle device's clocks take ~100 ms to ramp
 PEAK_BF16 = 2516.6   # TFLOP/s dense
 PEAK_FP8 = 5033.2
 PEAK_HBM = 8000.0    # GB/s
@@ -34,6 +35,18 @@ PEAK_HBM = 8000.0    # GB/s
 
 def log(*a):
     print(*a, file=sys.stderr, flush=True)
+
+
+def traffic_from_profile():
+    """HBM bytes per sparse-FA launch at config 0, as recorded in the committed rocprofv3 summary
+    (line ``traffic_bytes_per_launch <kernel> = <bytes>``); None when the summary has no such line."""
+    try:
+        for line in open(TRAFFIC_PROFILE):
+            if line.startswith("traffic_bytes_per_launch sparse_fa_kernel<bf16>"):
+                return float(line.split("=")[1].split()[0])
+    except OSError:
+        pass
+    return None
 
 
 def time_gpu(fn, iters, warmup):
@@ -89,14 +102,12 @@ class FluxLayer:
                                       out=self.out_q)
 
     def decode(self):
-        self.wrapper._decode_key = None
         return self.wrapper.decode(self.info, self.kv_info, self.info_ip, self.kv_ip)
 
     def attention(self, fresh_decode=True):
-        if fresh_decode:
-            self.wrapper._decode_key = None
+        """fresh_decode=False: run the list the last decode() left (ordered after it across streams)."""
         return self.wrapper.run(self.q, self.k, self.v, self.info, self.kv_info, self.info_ip,
-                                self.kv_ip, out=self.out_fa)
+                                self.kv_ip, out=self.out_fa, reuse_decoded=not fresh_decode)
 
     def gemm_o_cache(self):
         return self.fo.flashomni_gemm_reduction(self.a, self.wo, 24, self.info, self.info_ip, 0,
@@ -139,17 +150,13 @@ def bench_big_attention(dev, index, iters, warmup):
     args = [t.to(dev) for t in (wl.packed_info, wl.packed_kv_info, wl.info_indptr, wl.kv_info_indptr)]
     out = torch.zeros_like(q)
 
-    def dec():
-        w._decode_key = None
-        w.decode(*args)
-
     res = {}
-    ms = time_gpu(dec, iters, warmup)
+    ms = time_gpu(lambda: w.decode(*args), iters, warmup)
     rows, nnz = w._worklist.sizes()
     dec_bytes = wl.packed_info.numel() + wl.packed_kv_info.numel() + 4 * (4 * rows + 1 + nnz)
     res["decode"] = entry(ms, nbytes=dec_bytes)
     res["decode"]["rows"], res["decode"]["kv_blocks"] = rows, nnz
-    ms = time_gpu(lambda: w.run(q, k, v, *args, out=out), iters, warmup)
+    ms = time_gpu(lambda: w.run(q, k, v, *args, out=out, reuse_decoded=True), iters, warmup)
     res["sparse_fa_bf16"] = entry(ms, flops=wl.attention_flops())
     res["sparse_fa_bf16"]["computed_blocks"] = wl.computed_blocks
     if index == 4:
@@ -162,7 +169,9 @@ def bench_big_attention(dev, index, iters, warmup):
         w8 = fo.BatchFlashOmniFAWithRaggedKVWrapper(ws)
         w8.plan(wl.qo_indptr, wl.kv_indptr, s.heads, s.heads, 128, q_data_type=torch.float8_e4m3fn)
         out8 = torch.zeros_like(q)
-        ms8 = time_gpu(lambda: w8.run(q8, k8, v, *args, out=out8, q_scale=qs, k_scale=ks), iters, warmup)
+        w8.decode(*args)
+        ms8 = time_gpu(lambda: w8.run(q8, k8, v, *args, out=out8, q_scale=qs, k_scale=ks, reuse_decoded=True),
+                       iters, warmup)
         # QK^T half at the fp8 peak, PV half at the bf16 peak
         res["sparse_fa_fp8qk"] = entry(ms8, flops=wl.attention_flops(), peak=2.0 / (1 / PEAK_FP8 + 1 / PEAK_BF16))
         res["sparse_fa_fp8qk"]["frac_of_bf16_peak"] = round(res["sparse_fa_fp8qk"]["tflops"] / PEAK_BF16, 4)
@@ -246,14 +255,12 @@ def bench_wan_chain(dev, iters, warmup):
     def chain_fp8():
         fo.flashomni_gemm(x, wq, s.heads, info, ip, 0, bq, out=False, quant_out=(q8, q8s))
         k8, ks = fo.quant_fp8_block(k, wl.kv_indptr, blocks=blocks)
-        w8._decode_key = None
         w8.run(q8.view(s.seq, s.heads, 128), k8, v, info, kv_info, ip, kv_ip, out=o, q_scale=q8s, k_scale=ks)
         return fo.flashomni_gemm_reduction(o.view(1, s.seq, s.hidden), wo, s.heads, info, ip, 0, bias=cache,
                                            is_for_cache=False)
 
     def chain_bf16():
         fo.flashomni_gemm(x, wq, s.heads, info, ip, 0, bq, out=q16)
-        w16._decode_key = None
         w16.run(q16.view(s.seq, s.heads, 128), k, v, info, kv_info, ip, kv_ip, out=o)
         return fo.flashomni_gemm_reduction(o.view(1, s.seq, s.hidden), wo, s.heads, info, ip, 0, bias=cache,
                                            is_for_cache=False)
@@ -354,7 +361,13 @@ def main():
         "two-stream step differs from the sequential chain"
     del ref_q, ref_fa, ref_o, got_o
 
-    # ---- the timed region: K steps of the chain ----
+    # ---- clock settle (fixed, whatever --warmup says), W warm-up steps, then the timed region ----
+    t_settle = time.perf_counter()
+    while (time.perf_counter() - t_settle) * 1e3 < SETTLE_MS:
+        for _ in range(20):
+            layer.step()
+        torch.cuda.synchronize()
+    settle_ms = (time.perf_counter() - t_settle) * 1e3
     for _ in range(W):
         layer.step()
     torch.cuda.synchronize()
@@ -423,16 +436,19 @@ def main():
             kernels[SHAPES[idx].name] = res
             log("[bench]", SHAPES[idx].name, json.dumps(res))
 
+    # what the step costs beyond its three kernels (the decode runs beside GEMM-Q on a second stream)
+    kernel_sum_ms = (kernels[layer.w1.shape.name]["gemm_q"]["ms"] + fa_ms
+                     + kernels[layer.w2.shape.name]["gemm_o_final"]["ms"])
     fa_flops = w0.attention_flops()
     roofline = {
         "kernel": "sparse_fa_kernel<bf16> (config 0, FLUX shape)", "bound": "mfma",
         "achieved": round(fa_flops / (fa_ms * 1e-3) / 1e12, 2), "peak": PEAK_BF16, "unit": "TFLOP/s",
         "frac": round(fa_flops / (fa_ms * 1e-3) / 1e12 / PEAK_BF16, 4),
-        # HBM bytes per launch from two rocprofv3 --pmc runs of this command (FETCH_SIZE 69946.3 KiB x 2.0,
-        # the factor a 256 MiB copy kernel gives for that counter, + WRITE_SIZE 40532.7 KiB x 1.0);
-        # the algorithmic bytes of the launch are 98.6e6 (the excess is K/V re-fetched after falling out
-        # of an XCD's L2, which three heads share)
-        "traffic": FA_C0_HBM_BYTES if 0 in configs else None, "traffic_unit": "bytes/launch",
+        # HBM bytes per launch: read from the committed summary of two rocprofv3 --pmc runs of this
+        # command (FETCH_SIZE and WRITE_SIZE, each scaled by what a 256 MiB copy kernel reads on the same
+        # counter); the algorithmic bytes of the launch are 98.6e6
+        "traffic": traffic_from_profile(), "traffic_unit": "bytes/launch",
+        "traffic_source": "profiles/" + os.path.basename(TRAFFIC_PROFILE),
         "launch_ms": round(fa_ms, 5), "algorithmic_flop_per_launch": fa_flops,
     }
     cpu = None
@@ -444,7 +460,8 @@ def main():
         "metric": "sparse-FA + GEMM-Q/O effective TFLOP/s on computed blocks, FLUX-shaped sparse layer "
                   "(GEMM-Q c1 -> decode + sparse FA c0 -> GEMM-O final c2), 1 GPU",
         "value": round(value, 2), "unit": "TFLOP/s", "n_gpus": 1, "steps": K, "warmup": W,
-        "ms_per_step": round(ms_per_step, 5), "higher_is_better": True, "scaling": "weak",
+        "ms_per_step": round(ms_per_step, 5), "settle_ms": round(settle_ms, 1),
+        "host_gap_ms": round(ms_per_step - kernel_sum_ms, 5), "higher_is_better": True, "scaling": "weak",
         "vs_baseline": None, "dtype": "bf16", "data": "synthetic",
         "config": {"workload": "FLUX layer: c1_flux_gemm_q + c0_flux_sparse_fa + c2_flux_gemm_o(final)",
                    "seq": 4608, "heads": 24, "head_dim": 128, "hidden": 3072, "block": 128,

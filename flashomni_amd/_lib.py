@@ -83,6 +83,26 @@ def dtype_code(dtype):
     return table[dtype]
 
 
+class _NoGuard:
+    def __enter__(self):
+        return None
+
+    def __exit__(self, *exc):
+        return False
+
+
+_NO_GUARD = _NoGuard()
+
+
+def device_guard(device):
+    """Context that makes ``device`` the current one for the library call inside it (the library
+    launches on, and asks the properties of, the current device).  Costs nothing when it already is."""
+    import torch
+    if device.index is None or torch.cuda.current_device() == device.index:
+        return _NO_GUARD
+    return torch.cuda.device(device)
+
+
 def current_stream(device):
     import torch
     return torch.cuda.current_stream(device).cuda_stream

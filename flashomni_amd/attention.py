@@ -7,8 +7,9 @@ The public surface (constructor, ``plan``, ``run``, ``run_return_lse``, the depr
 * ``plan()`` runs the host planner (fo_prefill_plan) into the wrapper's integer workspace, builds
   the q-block table and sizes the work-list buffers;
 * ``run()`` first decodes the bit-packed symbols into a compacted work list on the GPU
-  (fo_decode_sparse; skipped when the same symbol tensors were decoded by the previous call) and
-  then launches the sparse FlashAttention kernel over that list (fo_sparse_fa_run).
+  (fo_decode_sparse, every call: the symbol buffers may have been rewritten in place by writers
+  torch does not see; ``reuse_decoded=True`` skips it on the caller's word) and then launches the
+  sparse FlashAttention kernel over that list (fo_sparse_fa_run).
 
 Only what the reference's shipped build supports is implemented: no causal / custom mask, no
 positional encoding, no logits soft cap, fp32 logits (reference: setup.py:98-111).
@@ -81,6 +82,183 @@ class DecodedWorkList:
                 self.kv_row_ptr[:n_rows + 1].cpu(), self.kv_idx[:nnz].cpu())
 
 
+class PlannedBatch:
+    """Everything ``plan`` derives from a ragged batch beyond the reference planner's arrays: the
+    decoder's q-block table, the block numbering of the fp8 scales, the sizes ``run`` checks its
+    tensors against and the work-list buffers (sized for the all-ones worst case).  Shared by the
+    wrapper and by the ``torch.ops.flashomni_kernels`` operators, which have no slot for these
+    buffers in the reference's signatures and look the object up by their integer workspace."""
+
+    def __init__(self, float_workspace_buffer, qo_indptr_host, kv_indptr_host, qo_indptr_dev,
+                 kv_indptr_dev, num_qo_heads, num_kv_heads, block_q, block_kv, share_rows=True,
+                 worklist=None):
+        L = _lib.lib()
+        self.device = float_workspace_buffer.device
+        self.float_ws = float_workspace_buffer
+        self.qo_indptr, self.kv_indptr = qo_indptr_dev, kv_indptr_dev
+        self.num_qo_heads, self.num_kv_heads = num_qo_heads, num_kv_heads
+        self.block_q, self.block_kv = block_q, block_kv
+        batch_size = qo_indptr_host.numel() - 1
+        self.batch_size = batch_size
+        n_blk = torch.zeros(3, dtype=torch.int64)
+        _lib.check(L.fo_decode_sizes(_lib.ptr(qo_indptr_host), _lib.ptr(kv_indptr_host), batch_size,
+                                     num_qo_heads, block_q, block_kv,
+                                     n_blk[0:].data_ptr(), n_blk[1:].data_ptr(), n_blk[2:].data_ptr()))
+        n_q_blk, max_rows, max_nnz = (int(v) for v in n_blk)
+        if max_nnz >= 2 ** 31:
+            raise RuntimeError("Failed to plan prefill with error: work list too large")
+        table = torch.empty((2, max(n_q_blk, 1)), dtype=torch.int32)
+        _lib.check(L.fo_sparse_block_table(_lib.ptr(qo_indptr_host), batch_size, block_q,
+                                           table[0].data_ptr(), table[1].data_ptr(), n_q_blk,
+                                           n_blk[0:].data_ptr()))
+        self.blk_table = table.to(self.device)
+        self.n_q_blk = n_q_blk
+        qlen = (qo_indptr_host[1:] - qo_indptr_host[:-1]).to(torch.int64)
+        klen = (kv_indptr_host[1:] - kv_indptr_host[:-1]).to(torch.int64)
+        q_base = torch.zeros(batch_size + 1, dtype=torch.int64)
+        kv_base = torch.zeros(batch_size + 1, dtype=torch.int64)
+        q_base[1:] = torch.cumsum((qlen + block_q - 1) // block_q, 0)
+        kv_base[1:] = torch.cumsum((klen + block_kv - 1) // block_kv, 0)
+        self.q_blk_base = q_base.to(torch.int32).to(self.device)
+        self.kv_blk_base = kv_base.to(torch.int32).to(self.device)
+        self.n_kv_blk = int(kv_base[-1])
+        # sizes the tensors given to run() must have (checked there without reading the device):
+        # token counts, and the packed bytes of the byte-aligned per-request segments
+        self.total_q_rows = int(qo_indptr_host[-1]) if qo_indptr_host.numel() else 0
+        self.total_kv_rows = int(kv_indptr_host[-1]) if kv_indptr_host.numel() else 0
+        nqb = q_base[1:] - q_base[:-1]
+        nkb = kv_base[1:] - kv_base[:-1]
+        self.min_info_bytes = int(((nqb * num_qo_heads + 7) // 8).sum())
+        self.min_kv_info_bytes = int(((nqb * nkb * num_qo_heads + 7) // 8).sum())
+        if worklist is None or worklist.max_rows < max_rows or worklist.max_nnz < max_nnz:
+            worklist = DecodedWorkList(max_rows, max_nnz, num_qo_heads, self.device)
+        self.worklist = worklist
+        self.max_rows = max_rows
+        self.share_rows = share_rows
+        self.split_ok = self._split_ws_ok()
+        self.decoded = None  # (is_full, stream) of the list the work-list buffers hold, or None
+
+    def float_ws_bytes(self) -> int:
+        return self.float_ws.numel() * self.float_ws.element_size()
+
+    def _split_ws_ok(self) -> bool:
+        """Whether the float workspace can hold the partial results of rows whose kv list is shared
+        between workgroups (the reference uses it for its split-kv partials, scheduler.cuh:322-328)."""
+        return (self.share_rows and self.float_ws.data_ptr() % 16 == 0
+                and self.float_ws_bytes() >= _lib.lib().fo_sparse_fa_split_workspace_bytes())
+
+    def decode(self, sparse_info, sparse_kv_info, sparse_info_indptr, sparse_kv_info_indptr,
+               is_full: bool = False) -> DecodedWorkList:
+        """fo_decode_sparse on the current stream into the work-list buffers."""
+        wl = self.worklist
+        if not is_full:
+            if sparse_info is None or sparse_kv_info is None or sparse_info_indptr is None \
+                    or sparse_kv_info_indptr is None:
+                raise ValueError("sparse_info, sparse_kv_info and their indptrs are required unless "
+                                 "is_full=True")
+            tensors = []
+            for name, t, dt in (("sparse_info", sparse_info, torch.uint8),
+                                ("sparse_kv_info", sparse_kv_info, torch.uint8),
+                                ("sparse_info_indptr", sparse_info_indptr, torch.int32),
+                                ("sparse_kv_info_indptr", sparse_kv_info_indptr, torch.int32)):
+                if t.device != self.device:
+                    raise ValueError(f"Invalid device of {name}: expected {self.device}, got {t.device}")
+                if t.dtype != dt or not t.is_contiguous():
+                    t = t.to(dt).contiguous()
+                tensors.append(t)
+            for name, t, need in (("sparse_info", tensors[0], self.min_info_bytes),
+                                  ("sparse_kv_info", tensors[1], self.min_kv_info_bytes)):
+                if t.numel() < need:
+                    raise ValueError(f"{name} holds {t.numel()} bytes; the planned batch needs {need}")
+            for name, t in (("sparse_info_indptr", tensors[2]), ("sparse_kv_info_indptr", tensors[3])):
+                if t.numel() != self.batch_size + 1:
+                    raise ValueError(f"{name} must have {self.batch_size + 1} entries, got {t.numel()}")
+        else:
+            tensors = [None] * 4
+        stream = torch.cuda.current_stream(self.device)
+        with _lib.device_guard(self.device):
+            _lib.check(_lib.lib().fo_decode_sparse(
+                _lib.ptr(tensors[0]), _lib.ptr(tensors[1]), _lib.ptr(tensors[2]), _lib.ptr(tensors[3]),
+                _lib.ptr(self.blk_table[0]), _lib.ptr(self.blk_table[1]), _lib.ptr(self.kv_indptr),
+                self.n_q_blk, self.num_qo_heads, self.block_kv, int(bool(is_full)),
+                _lib.ptr(wl.row_req), _lib.ptr(wl.row_qb), _lib.ptr(wl.row_head), _lib.ptr(wl.kv_row_ptr),
+                _lib.ptr(wl.kv_idx), _lib.ptr(wl.counts), _lib.ptr(wl.order), _lib.ptr(wl.sched),
+                _lib.ptr(wl.scratch), _lib.ptr(wl.shares if self.split_ok else None),
+                stream.cuda_stream))
+        # remembered for reuse_decoded: which stream the list was decoded on (a run on another
+        # stream must be ordered after it)
+        self.decoded = (bool(is_full), stream)
+        return wl
+
+    def reuse_decoded(self, is_full: bool) -> DecodedWorkList:
+        """The work list of the last decode, ordered before the current stream's work."""
+        if self.decoded is None:
+            raise RuntimeError("reuse_decoded=True needs an earlier decode() or run() after plan()")
+        was_full, stream = self.decoded
+        if was_full != bool(is_full):
+            raise RuntimeError("reuse_decoded=True: the last decode was made with is_full=%s" % was_full)
+        cur = torch.cuda.current_stream(self.device)
+        if cur != stream and not torch.cuda.is_current_stream_capturing():
+            ev = torch.cuda.Event()
+            ev.record(stream)
+            cur.wait_event(ev)
+        return self.worklist
+
+    def launch(self, q, k, v, out, lse, kv_layout, sm_scale, q_scale=None, k_scale=None) -> None:
+        """Shape checks against the planned batch, then fo_sparse_fa_run over the decoded list."""
+        if q.dim() != 3 or k.dim() != 3 or v.dim() != 3 or k.size(2) != 128 or v.size(2) != 128:
+            raise ValueError("q, k and v must be 3-dimensional with head_dim 128")
+        fp8 = is_float8(q)
+        if fp8:
+            if q.dtype != torch.float8_e4m3fn or k.dtype != torch.float8_e4m3fn \
+                    or q_scale is None or k_scale is None:
+                raise ValueError("fp8 attention needs float8_e4m3fn q and k with q_scale and k_scale")
+            if v.dtype != torch.bfloat16:
+                raise ValueError("fp8 attention keeps v (and the output) in bfloat16")
+        if q.device != self.device:
+            raise ValueError(f"Invalid device of q: expected {self.device}, got {q.device}")
+        if q.size(1) != self.num_qo_heads or q.size(2) != 128:
+            raise ValueError("q does not match the head count / head_dim given to plan()")
+        kv_head_dim = 1 if kv_layout == "NHD" else 0
+        if k.size(kv_head_dim) != self.num_kv_heads or v.size(kv_head_dim) != self.num_kv_heads:
+            raise ValueError("k / v do not match the kv head count given to plan()")
+        n_kv = min(k.size(1 - kv_head_dim), v.size(1 - kv_head_dim))
+        if q.size(0) < self.total_q_rows or n_kv < self.total_kv_rows:
+            raise ValueError(f"q / k, v hold {q.size(0)} / {n_kv} tokens; the planned "
+                             f"batch has {self.total_q_rows} / {self.total_kv_rows}")
+        if lse is not None and not lse.is_contiguous():
+            raise ValueError("lse must be contiguous")
+        for name, t in (("q", q), ("k", k), ("v", v), ("out", out)):
+            if t.stride(-1) != 1:
+                raise ValueError(f"{name} must have a contiguous last dimension")
+        if kv_layout == "NHD":
+            k_sn, k_sh, v_sn, v_sh = k.stride(0), k.stride(1), v.stride(0), v.stride(1)
+        else:
+            k_sh, k_sn, v_sh, v_sn = k.stride(0), k.stride(1), v.stride(0), v.stride(1)
+        if fp8:
+            q_scale = q_scale.to(torch.float32).contiguous()
+            k_scale = k_scale.to(torch.float32).contiguous()
+            if q_scale.shape != (q.size(1), self.n_q_blk) or \
+                    k_scale.shape != (self.num_kv_heads, self.n_kv_blk):
+                raise ValueError("q_scale / k_scale must be [H, number of 128-token blocks] "
+                                 "(k_scale: one row per kv head)")
+        wl = self.worklist
+        with _lib.device_guard(self.device):
+            _lib.check(_lib.lib().fo_sparse_fa_run(
+                _lib.ptr(q), _lib.ptr(k), _lib.ptr(v), _lib.ptr(out), _lib.ptr(lse),
+                _lib.dtype_code(q.dtype), _lib.ptr(q_scale if fp8 else None),
+                _lib.ptr(k_scale if fp8 else None),
+                q.stride(0), q.stride(1), k_sn, k_sh, v_sn, v_sh, out.stride(0), out.stride(1),
+                _lib.ptr(self.qo_indptr), _lib.ptr(self.kv_indptr), _lib.ptr(self.q_blk_base),
+                _lib.ptr(self.kv_blk_base), self.n_q_blk, self.n_kv_blk, _lib.ptr(wl.row_req),
+                _lib.ptr(wl.row_qb), _lib.ptr(wl.row_head), _lib.ptr(wl.kv_row_ptr), _lib.ptr(wl.kv_idx),
+                _lib.ptr(wl.order), _lib.ptr(wl.sched), self.max_rows, q.size(1), self.num_kv_heads,
+                q.size(2), self.block_q, self.block_kv, float(sm_scale),
+                _lib.ptr(wl.shares if self.split_ok else None),
+                _lib.ptr(self.float_ws) if self.split_ok else None,
+                self.float_ws_bytes(), _lib.current_stream(self.device)))
+
+
 class BatchFlashOmniFAWithRaggedKVWrapper:
     r"""Wrapper class for block-sparse prefill attention over ragged q/k/v tensors.
 
@@ -115,7 +293,6 @@ class BatchFlashOmniFAWithRaggedKVWrapper:
         # give the decoder a share table (queue-entry records; even shares for short lists); needs a
         # float workspace of fo_sparse_fa_split_workspace_bytes().  Read at plan() time.
         self._share_rows = True
-        self._split_ok = False
         self.device = float_workspace_buffer.device
         if self.device.type != "cuda":
             raise ValueError("float_workspace_buffer must live on the GPU; there is no CPU path")
@@ -141,8 +318,7 @@ class BatchFlashOmniFAWithRaggedKVWrapper:
         self._max_total_num_rows = None
         self._backend = backend  # accepted for compatibility; there is one HIP code path
         self._plan_info = None
-        self._worklist = None
-        self._decode_key = None
+        self._planned = None  # PlannedBatch of the last plan()
 
     @property
     def is_cuda_graph_enabled(self) -> bool:
@@ -155,6 +331,12 @@ class BatchFlashOmniFAWithRaggedKVWrapper:
         self._pin_memory_int_workspace_buffer = torch.empty(
             self._int_workspace_buffer.shape, dtype=self._int_workspace_buffer.dtype, device="cpu",
             pin_memory=True)
+        # whether rows may be shared between workgroups depends on the float workspace, and a list
+        # decoded for the old buffers' share table must not be reused
+        if self._planned is not None:
+            self._planned.float_ws = float_workspace_buffer
+            self._planned.split_ok = self._planned._split_ws_ok()
+            self._planned.decoded = None
 
     # ------------------------------------------------------------------------------------------
     def plan(
@@ -262,43 +444,11 @@ class BatchFlashOmniFAWithRaggedKVWrapper:
                 raise RuntimeError("Failed to plan prefill with error: " + str(e)) from None
         self._plan_info = plan_info
 
-        # q-block table + block numbering for the decoder / fp8 scales
-        n_blk = torch.zeros(3, dtype=torch.int64)
-        _lib.check(L.fo_decode_sizes(_lib.ptr(qo_indptr_host), _lib.ptr(kv_indptr_host), batch_size,
-                                     num_qo_heads, sparse_block_size_for_q, sparse_block_size_for_kv,
-                                     n_blk[0:].data_ptr(), n_blk[1:].data_ptr(), n_blk[2:].data_ptr()))
-        n_q_blk, max_rows, max_nnz = (int(v) for v in n_blk)
-        if max_nnz >= 2 ** 31:
-            raise RuntimeError("Failed to plan prefill with error: work list too large")
-        table = torch.empty((2, max(n_q_blk, 1)), dtype=torch.int32)
-        _lib.check(L.fo_sparse_block_table(_lib.ptr(qo_indptr_host), batch_size,
-                                           sparse_block_size_for_q, table[0].data_ptr(),
-                                           table[1].data_ptr(), n_q_blk, n_blk[0:].data_ptr()))
-        self._blk_table = table.to(self.device)
-        self._n_q_blk = n_q_blk
-        qlen = (qo_indptr_host[1:] - qo_indptr_host[:-1]).to(torch.int64)
-        klen = (kv_indptr_host[1:] - kv_indptr_host[:-1]).to(torch.int64)
-        q_base = torch.zeros(batch_size + 1, dtype=torch.int64)
-        kv_base = torch.zeros(batch_size + 1, dtype=torch.int64)
-        q_base[1:] = torch.cumsum((qlen + sparse_block_size_for_q - 1) // sparse_block_size_for_q, 0)
-        kv_base[1:] = torch.cumsum((klen + sparse_block_size_for_kv - 1) // sparse_block_size_for_kv, 0)
-        self._q_blk_base = q_base.to(torch.int32).to(self.device)
-        self._kv_blk_base = kv_base.to(torch.int32).to(self.device)
-        self._n_kv_blk = int(kv_base[-1])
-        # sizes the tensors given to run() must have (checked there without reading the device):
-        # token counts, and the packed bytes of the byte-aligned per-request segments
-        self._total_q_rows = total_num_rows
-        self._total_kv_rows = int(kv_indptr_host[-1]) if kv_indptr_host.numel() else 0
-        nqb = q_base[1:] - q_base[:-1]
-        nkb = kv_base[1:] - kv_base[:-1]
-        self._min_info_bytes = int(((nqb * num_qo_heads + 7) // 8).sum())
-        self._min_kv_info_bytes = int(((nqb * nkb * num_qo_heads + 7) // 8).sum())
-        if (self._worklist is None or self._worklist.max_rows < max_rows
-                or self._worklist.max_nnz < max_nnz):
-            self._worklist = DecodedWorkList(max_rows, max_nnz, num_qo_heads, self.device)
-        self._max_rows = max_rows
-        self._decode_key = None
-        self._split_ok = self._split_ws_ok()
+        self._planned = PlannedBatch(
+            self._float_workspace_buffer, qo_indptr_host, kv_indptr_host, self._qo_indptr_buf,
+            self._kv_indptr_buf, num_qo_heads, num_kv_heads, sparse_block_size_for_q,
+            sparse_block_size_for_kv, share_rows=self._share_rows,
+            worklist=self._planned.worklist if self._planned is not None else None)
 
         self._num_qo_heads = num_qo_heads
         self._num_kv_heads = num_kv_heads
@@ -320,70 +470,25 @@ class BatchFlashOmniFAWithRaggedKVWrapper:
 
     begin_forward = plan
 
-    def _float_ws_bytes(self) -> int:
-        ws = self._float_workspace_buffer
-        return ws.numel() * ws.element_size()
+    # names kept for callers that inspect the wrapper
+    @property
+    def _worklist(self):
+        return None if self._planned is None else self._planned.worklist
 
-    def _split_ws_ok(self) -> bool:
-        """Whether the float workspace can hold the partial results of rows whose kv list is shared
-        between workgroups (the reference uses it for its split-kv partials, scheduler.cuh:322-328)."""
-        ws = self._float_workspace_buffer
-        return (self._share_rows and ws.data_ptr() % 16 == 0
-                and self._float_ws_bytes() >= _lib.lib().fo_sparse_fa_split_workspace_bytes())
+    @property
+    def _split_ok(self):
+        return self._planned is not None and self._planned.split_ok
 
     # ------------------------------------------------------------------------------------------
     def decode(self, sparse_info, sparse_kv_info, sparse_info_indptr, sparse_kv_info_indptr,
                is_full: bool = False) -> DecodedWorkList:
         """Decode the packed symbols into the wrapper's work list (asynchronous, on the current
-        stream) and return it.  ``run`` calls this itself; calling it directly lets a caller decode
-        once and inspect or reuse the list."""
+        stream) and return it.  ``run`` calls this itself on every call; a caller that knows the
+        symbols have not changed can call it once and then pass ``reuse_decoded=True`` to ``run``."""
         if self._plan_info is None:
             raise RuntimeError("plan() must be called before decode()/run()")
-        wl = self._worklist
-        if not is_full:
-            if sparse_info is None or sparse_kv_info is None or sparse_info_indptr is None \
-                    or sparse_kv_info_indptr is None:
-                raise ValueError("sparse_info, sparse_kv_info and their indptrs are required unless "
-                                 "is_full=True")
-            tensors = []
-            for name, t, dt in (("sparse_info", sparse_info, torch.uint8),
-                                ("sparse_kv_info", sparse_kv_info, torch.uint8),
-                                ("sparse_info_indptr", sparse_info_indptr, torch.int32),
-                                ("sparse_kv_info_indptr", sparse_kv_info_indptr, torch.int32)):
-                if t.device != self.device:
-                    raise ValueError(f"Invalid device of {name}: expected {self.device}, got {t.device}")
-                tensors.append(t.to(dt).contiguous())
-            for name, t, need in (("sparse_info", tensors[0], self._min_info_bytes),
-                                  ("sparse_kv_info", tensors[1], self._min_kv_info_bytes)):
-                if t.numel() < need:
-                    raise ValueError(f"{name} holds {t.numel()} bytes; the planned batch needs {need}")
-            n_req = self._qo_indptr_buf.numel() - 1
-            for name, t in (("sparse_info_indptr", tensors[2]), ("sparse_kv_info_indptr", tensors[3])):
-                if t.numel() != n_req + 1:
-                    raise ValueError(f"{name} must have {n_req + 1} entries, got {t.numel()}")
-            key = tuple((t.data_ptr(), t._version, t.numel()) for t in
-                        (sparse_info, sparse_kv_info, sparse_info_indptr, sparse_kv_info_indptr))
-        else:
-            tensors = [None] * 4
-            key = "full"
-        # a stream capture must record the decode: replays see new symbol contents without
-        # passing through this method again
-        capturing = torch.cuda.is_current_stream_capturing()
-        if key == self._decode_key and not capturing:
-            return wl
-        _lib.check(_lib.lib().fo_decode_sparse(
-            _lib.ptr(tensors[0]), _lib.ptr(tensors[1]), _lib.ptr(tensors[2]), _lib.ptr(tensors[3]),
-            _lib.ptr(self._blk_table[0]), _lib.ptr(self._blk_table[1]), _lib.ptr(self._kv_indptr_buf),
-            self._n_q_blk, self._num_qo_heads, self._sparse_block_size_for_kv, int(bool(is_full)),
-            _lib.ptr(wl.row_req), _lib.ptr(wl.row_qb), _lib.ptr(wl.row_head), _lib.ptr(wl.kv_row_ptr),
-            _lib.ptr(wl.kv_idx), _lib.ptr(wl.counts), _lib.ptr(wl.order), _lib.ptr(wl.sched),
-            _lib.ptr(wl.scratch), _lib.ptr(wl.shares if self._split_ok else None),
-            _lib.current_stream(self.device)))
-        # the memo holds the tensors alive so a recycled address cannot alias the key
-        self._decode_key = None if capturing else key
-        self._decode_refs = (tensors, sparse_info, sparse_kv_info, sparse_info_indptr,
-                             sparse_kv_info_indptr)
-        return wl
+        return self._planned.decode(sparse_info, sparse_kv_info, sparse_info_indptr,
+                                    sparse_kv_info_indptr, is_full)
 
     def run(
         self,
@@ -401,6 +506,7 @@ class BatchFlashOmniFAWithRaggedKVWrapper:
         return_lse: bool = False,
         q_scale: Optional[torch.Tensor] = None,
         k_scale: Optional[torch.Tensor] = None,
+        reuse_decoded: bool = False,
     ) -> Union[torch.Tensor, Tuple[torch.Tensor, torch.Tensor]]:
         r"""Compute block-sparse prefill attention.
 
@@ -411,23 +517,21 @@ class BatchFlashOmniFAWithRaggedKVWrapper:
 
         ``q_scale`` / ``k_scale`` (keyword-only extension): fp32 ``[H, n_blocks]`` dequantisation
         scales; with them ``q`` and ``k`` are fp8 e4m3fn, ``v`` and ``out`` are bfloat16.
+
+        ``reuse_decoded`` (keyword-only extension): the symbols are decoded on every call, because
+        a buffer rewritten in place (by a kernel of the caller's, through the C ABI, ...) looks the
+        same from here.  Pass True to skip the decode and run the work list of the previous
+        ``decode``/``run``: the caller then vouches that the four symbol tensors have not changed.
         """
         if self._plan_info is None:
             raise RuntimeError("plan() must be called before run()")
-        if q.dim() != 3 or k.dim() != 3 or v.dim() != 3 or k.size(2) != 128 or v.size(2) != 128:
+        if q.dim() != 3 or v.dim() != 3:
             raise ValueError("q, k and v must be 3-dimensional with head_dim 128")
         _check_cached_qkv_data_type(q, k, self._cached_q_data_type, self._cached_kv_data_type)
         sm_scale = self._sm_scale
         if sm_scale is None:
             sm_scale = 1.0 / math.sqrt(q.size(-1))
-        fp8 = is_float8(q)
-        if fp8:
-            if q.dtype != torch.float8_e4m3fn or k.dtype != torch.float8_e4m3fn \
-                    or q_scale is None or k_scale is None:
-                raise ValueError("fp8 attention needs float8_e4m3fn q and k with q_scale and k_scale")
-            if v.dtype != torch.bfloat16:
-                raise ValueError("fp8 attention keeps v (and the output) in bfloat16")
-        out_dtype = torch.bfloat16 if fp8 else q.dtype
+        out_dtype = torch.bfloat16 if is_float8(q) else q.dtype
         if return_lse:
             if lse is None:
                 lse = torch.empty((q.size(0), q.size(1)), dtype=torch.float32, device=q.device)
@@ -437,52 +541,12 @@ class BatchFlashOmniFAWithRaggedKVWrapper:
             out = torch.zeros(q.shape[:-1] + v.shape[-1:], dtype=out_dtype, device=q.device)
         else:
             _check_shape_dtype_device(out, q.shape[:-1] + v.shape[-1:], out_dtype, q.device, "out")
-        if q.device != self.device:
-            raise ValueError(f"Invalid device of q: expected {self.device}, got {q.device}")
-        if q.size(1) != self._num_qo_heads or q.size(2) != 128:
-            raise ValueError("q does not match the head count / head_dim given to plan()")
-        kv_head_dim = 1 if self._kv_layout == "NHD" else 0
-        if k.size(kv_head_dim) != self._num_kv_heads or v.size(kv_head_dim) != self._num_kv_heads:
-            raise ValueError("k / v do not match the kv head count given to plan()")
-        n_kv = min(k.size(1 - kv_head_dim), v.size(1 - kv_head_dim))
-        if q.size(0) < self._total_q_rows or n_kv < self._total_kv_rows:
-            raise ValueError(f"q / k, v hold {q.size(0)} / {n_kv} tokens; the planned "
-                             f"batch has {self._total_q_rows} / {self._total_kv_rows}")
-        if return_lse and not lse.is_contiguous():
-            raise ValueError("lse must be contiguous")
-        for name, t in (("q", q), ("k", k), ("v", v), ("out", out)):
-            if t.stride(-1) != 1:
-                raise ValueError(f"{name} must have a contiguous last dimension")
-
-        if self._kv_layout == "NHD":
-            k_sn, k_sh, v_sn, v_sh = k.stride(0), k.stride(1), v.stride(0), v.stride(1)
+        pb = self._planned
+        if reuse_decoded:
+            pb.reuse_decoded(is_full)
         else:
-            k_sh, k_sn, v_sh, v_sn = k.stride(0), k.stride(1), v.stride(0), v.stride(1)
-
-        wl = self.decode(sparse_info, sparse_kv_info, sparse_info_indptr, sparse_kv_info_indptr,
-                         is_full)
-        if fp8:
-            q_scale = q_scale.to(torch.float32).contiguous()
-            k_scale = k_scale.to(torch.float32).contiguous()
-            if q_scale.shape != (q.size(1), self._n_q_blk) or \
-                    k_scale.shape != (self._num_kv_heads, self._n_kv_blk):
-                raise ValueError("q_scale / k_scale must be [H, number of 128-token blocks] "
-                                 "(k_scale: one row per kv head)")
-        _lib.check(_lib.lib().fo_sparse_fa_run(
-            _lib.ptr(q), _lib.ptr(k), _lib.ptr(v), _lib.ptr(out), _lib.ptr(lse if return_lse else None),
-            _lib.dtype_code(q.dtype), _lib.ptr(q_scale if fp8 else None),
-            _lib.ptr(k_scale if fp8 else None),
-            q.stride(0), q.stride(1), k_sn, k_sh, v_sn, v_sh, out.stride(0), out.stride(1),
-            _lib.ptr(self._qo_indptr_buf), _lib.ptr(self._kv_indptr_buf), _lib.ptr(self._q_blk_base),
-            _lib.ptr(self._kv_blk_base), self._n_q_blk, self._n_kv_blk, _lib.ptr(wl.row_req),
-            _lib.ptr(wl.row_qb),
-            _lib.ptr(wl.row_head), _lib.ptr(wl.kv_row_ptr), _lib.ptr(wl.kv_idx), _lib.ptr(wl.order),
-            _lib.ptr(wl.sched), self._max_rows, q.size(1), self._num_kv_heads, q.size(2),
-            self._sparse_block_size_for_q,
-            self._sparse_block_size_for_kv, float(sm_scale),
-            _lib.ptr(wl.shares if self._split_ok else None),
-            _lib.ptr(self._float_workspace_buffer) if self._split_ok else None,
-            self._float_ws_bytes(), _lib.current_stream(self.device)))
+            pb.decode(sparse_info, sparse_kv_info, sparse_info_indptr, sparse_kv_info_indptr, is_full)
+        pb.launch(q, k, v, out, lse if return_lse else None, self._kv_layout, sm_scale, q_scale, k_scale)
         return (out, lse) if return_lse else out
 
     run_return_lse = functools.partialmethod(run, return_lse=True)

@@ -9,13 +9,17 @@
 // Besides the canonical list the decoder emits an execution order for the attention kernel:
 // `order` lists row positions grouped by head, heads dealt to the 8 XCDs round-robin (head % 8), so
 // that the workgroups of one XCD (which share an L2) walk the rows of the same few heads and find
-// that head's K/V in their L2.  Inside a head the rows go longest first (up to 32 length classes
-// relative to the longest row of the launch), which evens out the workgroups' finishing times.
+// that head's K/V in their L2.  Inside a head the order depends on how long the list is:
+//   * eight or more rows per workgroup of the attention kernel: q blocks ascending (a fixed order,
+//     laid out by the scan kernel).  Neighbouring q blocks of a head keep overlapping kv blocks
+//     (windowed masks), so the workgroups of an XCD, which pop consecutive entries, share K/V tiles
+//     in that XCD's L2; with that many rows per workgroup the finishing times even out by themselves;
+//   * fewer: longest rows first (up to 32 length classes relative to the longest row of the launch),
+//     which evens out the workgroups' finishing times; the order inside a length class is not
+//     deterministic (atomic cursors), results do not depend on it;
+//   * at most two rows per workgroup (and a share table to fill): "even shares", see the scan kernel.
 // sched[0..8] delimit the 8 per-XCD queues inside `order`, sched[16..23] are the queue cursors,
-// sched[24] a completion counter (all cleared here) and sched[25] the longest row's kv count.  The
-// order inside a length class is not deterministic (atomic cursors); results do not depend on it.
-// With at most two rows per workgroup of the attention kernel (and a share table to fill) the
-// layout is different, "even shares": see the scan kernel.
+// sched[24] a completion counter (all cleared here) and sched[25] the longest row's kv count.
 // Integer work, bounded by HBM traffic and launch latency; bit-exact by construction.
 //
 // Symbol semantics (reference: include/flashomni/attention/prefill.cuh:1284-1294, 1380-1403,
@@ -33,7 +37,8 @@ constexpr int kXcds = 8;
 constexpr int kHistSlots = 8192;  // (head, length class) counters of the order layout
 // even shares (see the attention kernel): words of `sched` and limits
 constexpr int kSchedEven = 26, kSchedShare = 27, kSchedTotal = 28, kSchedShares = 29, kSchedRows = 30,
-              kSchedRecords = 31, kSchedArrived = 64;
+              kSchedRecords = 31, kSchedOrdered = 32, kSchedArrived = 64;
+constexpr int kSchedWords = 40;      // words [0, kSchedWords) are rewritten by every decode
 constexpr int kRecordInts = 8;  // queue entry: row, request, q block, head, first kv slot, kv count, pad, pad
 constexpr int kMaxShares = 512;      // arrival counters in `sched`, first-row entries in `shares`
 constexpr int kMaxSplitParts = 4;    // a row is cut into at most this many parts
@@ -42,6 +47,7 @@ constexpr int kEvenMaxRounds = 2;    // even shares when there are at most this 
 // often, three heads' K and V being live in every XCD at once; from ~5 rows on the queues balance as well and
 // adapt to the workgroups' actual speeds, which fixed shares cannot.)
 constexpr int kRowOverhead = 3;      // fixed cost of a row (prologue, epilogue) in units of one kv block
+constexpr int kOrderedMinRounds = 8; // q blocks ascending inside a head from this many rows per workgroup on
 
 // number of length classes for num_heads heads (32 up to 256 heads)
 __host__ __device__ __forceinline__ int len_classes(int32_t num_heads) {
@@ -129,7 +135,8 @@ __global__ void __launch_bounds__(kScanThreads) decode_scan_kernel(
     int64_t n_cand, int32_t num_heads, int32_t* __restrict__ act, int32_t* __restrict__ cnt,
     int32_t* __restrict__ kv_row_ptr, int32_t* __restrict__ counts,
     int32_t* __restrict__ head_cursor, int32_t* __restrict__ sched, int32_t* __restrict__ order,
-    int32_t* __restrict__ shares, int32_t n_shares) {
+    int32_t* __restrict__ shares, int32_t n_shares, int32_t n_wg, const int32_t* __restrict__ blk_req,
+    const int32_t* __restrict__ blk_qb) {
   __shared__ int32_t s_rows[kScanThreads];
   __shared__ int32_t s_kv[kScanThreads];
   __shared__ int32_t s_hist[kHistSlots];
@@ -244,7 +251,7 @@ __global__ void __launch_bounds__(kScanThreads) decode_scan_kernel(
     }
     if (tid == 0) {
       row_start[n_rows] = total + kRowOverhead;
-      for (int i = 0; i < 32; ++i) sched[i] = 0;
+      for (int i = 0; i < kSchedWords; ++i) sched[i] = 0;
       // (the queues stay usable: eight equal runs of the same order, for a launch without shares)
       for (int x = 0; x <= kXcds; ++x) sched[x] = static_cast<int32_t>(static_cast<int64_t>(n_rows) * x / kXcds);
       sched[25] = max_n;
@@ -276,7 +283,66 @@ __global__ void __launch_bounds__(kScanThreads) decode_scan_kernel(
     return;
   }
 
-  // execution order layout: queue x holds heads x, x+8, x+16, ... back to back, each head's length
+  // Long lists: queue x holds heads x, x+8, x+16, ... back to back, every head's rows with q blocks
+  // ascending.  Each head is cut into runs of q blocks, one per thread; the runs are numbered in queue
+  // order, so one prefix sum over the threads' row counts places every row.
+  if (n_wg > 0 && n_rows >= kOrderedMinRounds * n_wg && num_heads <= kScanThreads) {
+    const int32_t nq = static_cast<int32_t>(n_cand / num_heads);
+    const int segs = kScanThreads / num_heads;
+    const int per = (nq + segs - 1) / segs;
+    const int h = tid / segs, seg = tid - h * segs;
+    const bool mine = h < num_heads;
+    auto heads_of_queue = [&](int x) { return num_heads > x ? (num_heads - x + kXcds - 1) / kXcds : 0; };
+    auto queue_base = [&](int x) {  // heads in the queues before queue x
+      int b = 0;
+      for (int y = 0; y < x; ++y) b += heads_of_queue(y);
+      return b;
+    };
+    const int t0 = mine ? min(seg * per, nq) : 0, t1 = mine ? min(t0 + per, nq) : 0;
+    auto kv_count = [&](int64_t c) { return (c + 1 < n_cand ? cnt[c + 1] : nnz) - cnt[c]; };
+    int32_t my_rows = 0;
+    for (int t = t0; t < t1; ++t) my_rows += act[static_cast<int64_t>(t) * num_heads + h] >= 0 ? 1 : 0;
+    s_rows[tid] = 0;
+    __syncthreads();
+    const int slot = mine ? (queue_base(h % kXcds) + h / kXcds) * segs + seg : 0;
+    if (mine) s_rows[slot] = my_rows;  // (the slots of the heads' runs are a permutation of the first H * segs)
+    __syncthreads();
+    for (int off = 1; off < kScanThreads; off <<= 1) {
+      const int32_t r = tid >= off ? s_rows[tid - off] : 0;
+      __syncthreads();
+      s_rows[tid] += r;
+      __syncthreads();
+    }
+    if (mine) {
+      int32_t pos = s_rows[slot] - my_rows;
+      for (int t = t0; t < t1; ++t) {
+        const int64_t c = static_cast<int64_t>(t) * num_heads + h;
+        if (act[c] >= 0) {
+          order[pos] = act[c];
+          if (shares) {
+            typedef __attribute__((ext_vector_type(4))) int i32x4;
+            i32x4* rec = reinterpret_cast<i32x4*>(shares + kMaxShares + kRecordInts * static_cast<int64_t>(pos));
+            rec[0] = i32x4{act[c], blk_req[t], blk_qb[t], h};
+            rec[1] = i32x4{cnt[c], kv_count(c), 0, 0};
+          }
+          ++pos;
+        }
+      }
+    }
+    if (tid == 0) {
+      for (int i = 0; i < kSchedWords; ++i) sched[i] = 0;
+      for (int x = 0; x <= kXcds; ++x) {
+        const int first = queue_base(x) * segs;  // first run of queue x (x = 8: one past the last)
+        sched[x] = first > 0 ? s_rows[first - 1] : 0;
+      }
+      sched[25] = max_n;
+      sched[kSchedRecords] = shares != nullptr ? 1 : 0;
+      sched[kSchedOrdered] = 1;  // the fill kernel leaves `order` and the records alone
+    }
+    return;
+  }
+
+  // shorter lists: queue x holds heads x, x+8, x+16, ... back to back, each head's length
   // classes in order.  Exclusive prefix sum of the histogram taken in that order: every thread owns
   // a run of consecutive entries, wavefront scan by lane shifts, then the sixteen wavefront totals.
   {
@@ -322,7 +388,7 @@ __global__ void __launch_bounds__(kScanThreads) decode_scan_kernel(
       // queues without heads (fewer than 8 heads) are empty and sit at the end
       for (int x = num_heads; x < kXcds; ++x) sched[x] = total;
       sched[kXcds] = total;
-      for (int i = kXcds + 1; i < 32; ++i) sched[i] = 0;
+      for (int i = kXcds + 1; i < kSchedWords; ++i) sched[i] = 0;
       sched[25] = max_n;
       // with a share table the fill kernel also leaves one record per queue entry there (what the
       // attention kernel needs to start a row: one load after the pop instead of three rounds)
@@ -358,7 +424,7 @@ __global__ void __launch_bounds__(kCountThreads) decode_fill_kernel(
     kv_row_ptr[pos] = out;
     const int32_t listed = (c + 1 < n_cand ? kv_pos[c + 1] : counts[1]) - out;  // kv blocks of this row
     const int n_classes = len_classes(num_heads);
-    if (!sched[kSchedEven]) {  // (with even shares the scan kernel has written the order)
+    if (!sched[kSchedEven] && !sched[kSchedOrdered]) {  // (otherwise the scan kernel has written the order)
       const int32_t at = atomicAdd(&head_cursor[cd.head * n_classes + len_class(listed, sched[25], n_classes)], 1);
       order[at] = pos;
       if (shares) {
@@ -397,15 +463,14 @@ __global__ void __launch_bounds__(kCountThreads) decode_fill_kernel(
 
 }  // namespace
 
-extern "C" int fo_decode_sparse(const uint8_t* sparse_info, const uint8_t* sparse_kv_info,
-                                const int32_t* sparse_info_indptr,
-                                const int32_t* sparse_kv_info_indptr, const int32_t* blk_req,
-                                const int32_t* blk_qb, const int32_t* kv_indptr, int32_t n_blk,
-                                int32_t num_heads, int32_t block_kv, int is_full,
-                                int32_t* row_req, int32_t* row_qb, int32_t* row_head,
-                                int32_t* kv_row_ptr, int32_t* kv_idx, int32_t* counts,
-                                int32_t* order, int32_t* sched, int32_t* scratch, int32_t* shares,
-                                void* stream) {
+namespace {
+
+int decode_impl(const uint8_t* sparse_info, const uint8_t* sparse_kv_info, const int32_t* sparse_info_indptr,
+                const int32_t* sparse_kv_info_indptr, const int32_t* blk_req, const int32_t* blk_qb,
+                const int32_t* kv_indptr, int32_t n_blk, int32_t num_heads, int32_t block_kv, int is_full,
+                int32_t* row_req, int32_t* row_qb, int32_t* row_head, int32_t* kv_row_ptr, int32_t* kv_idx,
+                int32_t* counts, int32_t* order, int32_t* sched, int32_t* scratch_ptr, int32_t* shares,
+                void* stream) {
   FO_REQUIRE(n_blk >= 0 && num_heads > 0 && num_heads <= kMaxHeads && block_kv > 0,
              "decode: bad sizes");
   FO_REQUIRE(counts && kv_row_ptr && order && sched, "decode: null output");
@@ -413,14 +478,14 @@ extern "C" int fo_decode_sparse(const uint8_t* sparse_info, const uint8_t* spars
     FO_REQUIRE(sparse_info && sparse_kv_info && sparse_info_indptr && sparse_kv_info_indptr,
                "decode: sparse_info, sparse_kv_info and their indptrs are required unless is_full");
   }
-  FO_REQUIRE(blk_req && blk_qb && kv_indptr && scratch, "decode: null table");
+  FO_REQUIRE(blk_req && blk_qb && kv_indptr && scratch_ptr, "decode: null table");
   FO_REQUIRE((reinterpret_cast<uintptr_t>(shares) & 15) == 0, "decode: shares must be 16-byte aligned");
   const int64_t n_cand = static_cast<int64_t>(n_blk) * num_heads;
   FO_REQUIRE(n_cand < (int64_t(1) << 31), "decode: too many (q-block, head) pairs");
   hipStream_t s = static_cast<hipStream_t>(stream);
-  int32_t* act = scratch;
-  int32_t* cnt = scratch + n_cand;
-  int32_t* head_cursor = scratch + 2 * n_cand;
+  int32_t* act = scratch_ptr;
+  int32_t* cnt = scratch_ptr + n_cand;
+  int32_t* head_cursor = scratch_ptr + 2 * n_cand;
   if (n_cand > 0) {
     FO_REQUIRE(row_req && row_qb && row_head && kv_idx, "decode: null output");
     const int per_wg = kCountThreads / kWave;
@@ -430,9 +495,11 @@ extern "C" int fo_decode_sparse(const uint8_t* sparse_info, const uint8_t* spars
         kv_indptr, n_cand, num_heads, block_kv, is_full, act, cnt);
     FO_CHECK_LAUNCH();
   }
-  const int32_t n_shares = shares ? fo_num_cu() : 0;  // one share per workgroup of the attention kernel
+  const int32_t n_wg = fo_num_cu();                // workgroups of the attention kernel: one per CU
+  const int32_t n_shares = shares ? n_wg : 0;      // one share per workgroup
   decode_scan_kernel<<<1, kScanThreads, 0, s>>>(n_cand, num_heads, act, cnt, kv_row_ptr, counts,
-                                                head_cursor, sched, order, shares, n_shares);
+                                                head_cursor, sched, order, shares, n_shares, n_wg,
+                                                blk_req, blk_qb);
   FO_CHECK_LAUNCH();
   if (n_cand > 0) {
     const int per_wg = kCountThreads / kWave;
@@ -444,4 +511,20 @@ extern "C" int fo_decode_sparse(const uint8_t* sparse_info, const uint8_t* spars
     FO_CHECK_LAUNCH();
   }
   return FO_OK;
+}
+
+}  // namespace
+
+extern "C" int fo_decode_sparse(const uint8_t* sparse_info, const uint8_t* sparse_kv_info,
+                                const int32_t* sparse_info_indptr,
+                                const int32_t* sparse_kv_info_indptr, const int32_t* blk_req,
+                                const int32_t* blk_qb, const int32_t* kv_indptr, int32_t n_blk,
+                                int32_t num_heads, int32_t block_kv, int is_full,
+                                int32_t* row_req, int32_t* row_qb, int32_t* row_head,
+                                int32_t* kv_row_ptr, int32_t* kv_idx, int32_t* counts,
+                                int32_t* order, int32_t* sched, int32_t* scratch, int32_t* shares,
+                                void* stream) {
+  return decode_impl(sparse_info, sparse_kv_info, sparse_info_indptr, sparse_kv_info_indptr, blk_req, blk_qb,
+                     kv_indptr, n_blk, num_heads, block_kv, is_full, row_req, row_qb, row_head, kv_row_ptr,
+                     kv_idx, counts, order, sched, scratch, shares, stream);
 }

@@ -804,14 +804,15 @@ int64_t workspace_ints(const ListGeom& gm, int64_t* max_quads_out) {
 
 template <typename T, bool kReduce>
 int launch(GemmParams& p, const ListGeom& gm, bool use_flags, void* workspace, hipStream_t stream) {
-  // (the attribute belongs to the kernel's code object on one device: set once per device)
-  static bool attr_set[64] = {};
+  // (the attribute belongs to the kernel's code object on one device: set once per device; the flags
+  // are atomic because host threads may launch concurrently, and setting it twice is harmless)
+  static std::atomic<bool> attr_set[64] = {};
   int dev = 0;
   FO_HIP_CALL(hipGetDevice(&dev));
-  if (dev < 0 || dev >= 64 || !attr_set[dev]) {
+  if (dev < 0 || dev >= 64 || !attr_set[dev].load(std::memory_order_acquire)) {
     FO_HIP_CALL(hipFuncSetAttribute(reinterpret_cast<const void*>(&gemm_kernel<T, kReduce>),
                                     hipFuncAttributeMaxDynamicSharedMemorySize, kSmemBytes));
-    if (dev >= 0 && dev < 64) attr_set[dev] = true;
+    if (dev >= 0 && dev < 64) attr_set[dev].store(true, std::memory_order_release);
   }
   int64_t max_quads = 0;
   workspace_ints(gm, &max_quads);

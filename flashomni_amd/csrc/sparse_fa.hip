@@ -1129,14 +1129,15 @@ __global__ void __launch_bounds__(kThreads) sparse_fa_kernel(const FaParams p) {
 template <typename T, bool kFp8>
 int launch(const FaParams& p, int64_t max_rows, hipStream_t stream) {
   constexpr int kSmemBytes = Geom<kFp8>::kSmemBytes;
-  // (the attribute belongs to the kernel's code object on one device: set once per device)
-  static bool attr_set[64] = {};
+  // (the attribute belongs to the kernel's code object on one device: set once per device; the flags
+  // are atomic because host threads may launch concurrently, and setting it twice is harmless)
+  static std::atomic<bool> attr_set[64] = {};
   int dev = 0;
   FO_HIP_CALL(hipGetDevice(&dev));
-  if (dev < 0 || dev >= 64 || !attr_set[dev]) {
+  if (dev < 0 || dev >= 64 || !attr_set[dev].load(std::memory_order_acquire)) {
     FO_HIP_CALL(hipFuncSetAttribute(reinterpret_cast<const void*>(&sparse_fa_kernel<T, kFp8>),
                                     hipFuncAttributeMaxDynamicSharedMemorySize, kSmemBytes));
-    if (dev >= 0 && dev < 64) attr_set[dev] = true;
+    if (dev >= 0 && dev < 64) attr_set[dev].store(true, std::memory_order_release);
   }
   int num_cu = fo_num_cu();
   if (num_cu <= 0) return fo::fail(FO_ERR_HIP, "sparse_fa: no device");

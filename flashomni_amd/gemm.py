@@ -32,8 +32,11 @@ def _symbols(sparse_info, sparse_info_indptr, device, name, batch, m, num_qo_hea
         return None, None
     if sparse_info_indptr is None:
         raise RuntimeError(f"{name}: sparse_info needs sparse_info_indptr")
-    info = sparse_info.to(device=device, dtype=torch.uint8).contiguous()
-    indptr = sparse_info_indptr.to(device=device, dtype=torch.int32).contiguous()
+    info, indptr = sparse_info, sparse_info_indptr
+    if info.device != device or info.dtype != torch.uint8 or not info.is_contiguous():
+        info = info.to(device=device, dtype=torch.uint8).contiguous()
+    if indptr.device != device or indptr.dtype != torch.int32 or not indptr.is_contiguous():
+        indptr = indptr.to(device=device, dtype=torch.int32).contiguous()
     if indptr.numel() != batch + 1:
         raise RuntimeError(f"{name}: sparse_info_indptr must have batch + 1 = {batch + 1} entries, "
                            f"got {indptr.numel()}")
@@ -44,6 +47,20 @@ def _symbols(sparse_info, sparse_info_indptr, device, name, batch, m, num_qo_hea
             raise RuntimeError(f"{name}: sparse_info holds {info.numel()} bytes, a request needs {need} "
                                f"({last_block + 1} token blocks x {num_qo_heads} heads)")
     return info, indptr
+
+
+# tile-list scratch of GEMM-Q, one buffer per (device, stream): calls on one stream run in order, so
+# they can share it; calls on different streams may overlap and get their own
+_workspaces = {}
+
+
+def _gemm_workspace(device, stream, nbytes):
+    key = (device.index, stream)
+    ws = _workspaces.get(key)
+    if ws is None or ws.numel() < nbytes:
+        ws = torch.empty(max(nbytes, 1), dtype=torch.uint8, device=device)
+        _workspaces[key] = ws
+    return ws
 
 
 def flashomni_gemm(
@@ -57,6 +74,7 @@ def flashomni_gemm(
     out: torch.Tensor = None,
     sparse_q_size: int = 128,
     is_full: bool = False,
+    *,
     quant_out=None,
 ) -> torch.Tensor:
     """``out[b, tile] = A[b] @ B.T + bias`` for every (128-token block, 128-column) tile whose
@@ -96,13 +114,15 @@ def flashomni_gemm(
         raise RuntimeError("flashomni_gemm: sparse_info is required unless is_full=True")
     L = _lib.lib()
     ws_bytes = L.fo_gemm_workspace_bytes(A.shape[0], A.shape[1], B.shape[0])
-    workspace = torch.empty(ws_bytes, dtype=torch.uint8, device=A.device)  # tile-list scratch
+    stream = _lib.current_stream(A.device)
+    workspace = _gemm_workspace(A.device, stream, ws_bytes)
     if quant_out is None:
-        _lib.check(L.fo_gemm_q(
-            _lib.ptr(A), _lib.ptr(B), _lib.ptr(bias), _lib.ptr(out), _lib.dtype_code(A.dtype),
-            A.shape[0], A.shape[1], B.shape[0], A.shape[2], sparse_q_size, num_qo_heads,
-            _lib.ptr(info), _lib.ptr(indptr), num_text_tokens, int(bool(is_full)),
-            _lib.ptr(workspace), ws_bytes, _lib.current_stream(A.device)))
+        with _lib.device_guard(A.device):
+            _lib.check(L.fo_gemm_q(
+                _lib.ptr(A), _lib.ptr(B), _lib.ptr(bias), _lib.ptr(out), _lib.dtype_code(A.dtype),
+                A.shape[0], A.shape[1], B.shape[0], A.shape[2], sparse_q_size, num_qo_heads,
+                _lib.ptr(info), _lib.ptr(indptr), num_text_tokens, int(bool(is_full)),
+                _lib.ptr(workspace), ws_bytes, stream))
         return out
     Bsz, M, N = A.shape[0], A.shape[1], B.shape[0]
     n_blk = Bsz * ((M + 127) // 128)
@@ -118,11 +138,12 @@ def flashomni_gemm(
                 or not scale.is_contiguous() or scale.device != A.device:
             raise RuntimeError("flashomni_gemm: quant_out[1] must be a contiguous [H, B * ceil(M / 128)] "
                                "float32 tensor")
-    _lib.check(L.fo_gemm_q_quant(
-        _lib.ptr(A), _lib.ptr(B), _lib.ptr(bias), _lib.ptr(out), _lib.ptr(q8), _lib.ptr(scale),
-        _lib.dtype_code(A.dtype), Bsz, M, N, A.shape[2], sparse_q_size, num_qo_heads,
-        _lib.ptr(info), _lib.ptr(indptr), num_text_tokens, int(bool(is_full)),
-        _lib.ptr(workspace), ws_bytes, _lib.current_stream(A.device)))
+    with _lib.device_guard(A.device):
+        _lib.check(L.fo_gemm_q_quant(
+            _lib.ptr(A), _lib.ptr(B), _lib.ptr(bias), _lib.ptr(out), _lib.ptr(q8), _lib.ptr(scale),
+            _lib.dtype_code(A.dtype), Bsz, M, N, A.shape[2], sparse_q_size, num_qo_heads,
+            _lib.ptr(info), _lib.ptr(indptr), num_text_tokens, int(bool(is_full)),
+            _lib.ptr(workspace), ws_bytes, stream))
     return out, q8, scale
 
 
@@ -177,9 +198,10 @@ def flashomni_gemm_reduction(
                             Bsz, M, num_qo_heads, num_text_tokens, sparse_q_size)
     L = _lib.lib()
     workspace, ws_bytes = None, 0  # the reduction visits every token block: no tile list
-    _lib.check(L.fo_gemm_o(
-        _lib.ptr(A), _lib.ptr(B), _lib.ptr(bias), _lib.ptr(out), _lib.dtype_code(A.dtype), kind,
-        bias_code, _lib.dtype_code(out_dtype), Bsz, M, N, A.shape[2], sparse_q_size, num_qo_heads,
-        _lib.ptr(info), _lib.ptr(indptr), num_text_tokens, int(bool(is_for_cache)),
-        _lib.ptr(workspace), ws_bytes, _lib.current_stream(A.device)))
+    with _lib.device_guard(A.device):
+        _lib.check(L.fo_gemm_o(
+            _lib.ptr(A), _lib.ptr(B), _lib.ptr(bias), _lib.ptr(out), _lib.dtype_code(A.dtype), kind,
+            bias_code, _lib.dtype_code(out_dtype), Bsz, M, N, A.shape[2], sparse_q_size, num_qo_heads,
+            _lib.ptr(info), _lib.ptr(indptr), num_text_tokens, int(bool(is_for_cache)),
+            _lib.ptr(workspace), ws_bytes, _lib.current_stream(A.device)))
     return out

@@ -36,8 +36,9 @@ def packbits(x: torch.Tensor, bitorder: str = "big") -> torch.Tensor:
     _require_gpu_tensor(x, "x")
     xb = _as_bool_bytes(x.reshape(-1))
     y = torch.empty((xb.size(0) + 7) // 8, dtype=torch.uint8, device=x.device)
-    _lib.check(_lib.lib().fo_packbits(_lib.ptr(xb), xb.size(0), code, _lib.ptr(y),
-                                      _lib.current_stream(x.device)))
+    with _lib.device_guard(x.device):
+        _lib.check(_lib.lib().fo_packbits(_lib.ptr(xb), xb.size(0), code, _lib.ptr(y),
+                                          _lib.current_stream(x.device)))
     return y
 
 
@@ -69,9 +70,10 @@ def segment_packbits(x: torch.Tensor, indptr: torch.Tensor,
     indptr_new = indptr_new.to(device=device, dtype=torch.int32)
     xb = _as_bool_bytes(x.reshape(-1))
     y = torch.empty(output_nnzs, dtype=torch.uint8, device=device)
-    _lib.check(_lib.lib().fo_segment_packbits(_lib.ptr(xb), _lib.ptr(indptr), _lib.ptr(indptr_new),
-                                              len(indptr) - 1, code, _lib.ptr(y),
-                                              _lib.current_stream(device)))
+    with _lib.device_guard(device):
+        _lib.check(_lib.lib().fo_segment_packbits(_lib.ptr(xb), _lib.ptr(indptr), _lib.ptr(indptr_new),
+                                                  len(indptr) - 1, code, _lib.ptr(y),
+                                                  _lib.current_stream(device)))
     return y, indptr_new
 
 
@@ -110,8 +112,9 @@ def quant_fp8_block(x: torch.Tensor, indptr: torch.Tensor, block: int = 128,
     nnz, H, D = x.shape
     x8 = torch.empty((nnz, H, D), dtype=torch.float8_e4m3fn, device=x.device)
     scale = torch.empty((H, tok0.numel()), dtype=torch.float32, device=x.device)
-    _lib.check(_lib.lib().fo_quant_fp8_block(
-        _lib.ptr(x), _lib.dtype_code(x.dtype), x.stride(0), x.stride(1), _lib.ptr(x8),
-        _lib.ptr(scale), _lib.ptr(tok0), _lib.ptr(length), tok0.numel(), H, D,
-        _lib.current_stream(x.device)))
+    with _lib.device_guard(x.device):
+        _lib.check(_lib.lib().fo_quant_fp8_block(
+            _lib.ptr(x), _lib.dtype_code(x.dtype), x.stride(0), x.stride(1), _lib.ptr(x8),
+            _lib.ptr(scale), _lib.ptr(tok0), _lib.ptr(length), tok0.numel(), H, D,
+            _lib.current_stream(x.device)))
     return x8, scale

@@ -58,8 +58,9 @@ def sparse_symbols_from_scores(
     sparse_kv_info = torch.empty(B * kv_bytes, dtype=torch.uint8, device=dev)
     info_indptr = torch.empty(B + 1, dtype=torch.int32, device=dev)
     kv_indptr = torch.empty(B + 1, dtype=torch.int32, device=dev)
-    _lib.check(_lib.lib().fo_symbols_from_scores(
-        _lib.ptr(scores), _lib.dtype_code(scores.dtype), B, H, NQ, NK, t2t, t2t_kv,
-        _lib.ptr(q_thr), _lib.ptr(kv_thr), _lib.ptr(sparse_info), _lib.ptr(info_indptr),
-        _lib.ptr(sparse_kv_info), _lib.ptr(kv_indptr), _lib.current_stream(dev)))
+    with _lib.device_guard(dev):
+        _lib.check(_lib.lib().fo_symbols_from_scores(
+            _lib.ptr(scores), _lib.dtype_code(scores.dtype), B, H, NQ, NK, t2t, t2t_kv,
+            _lib.ptr(q_thr), _lib.ptr(kv_thr), _lib.ptr(sparse_info), _lib.ptr(info_indptr),
+            _lib.ptr(sparse_kv_info), _lib.ptr(kv_indptr), _lib.current_stream(dev)))
     return sparse_info, info_indptr, sparse_kv_info, kv_indptr

@@ -88,13 +88,16 @@ int fo_prefill_plan(void* float_ws, size_t float_ws_bytes, void* int_ws_dev, voi
  *   kv_row_ptr [n_rows+1], kv_idx [nnz]  kept kv blocks of each row, ascending
  *   counts[0] = n_rows, counts[1] = nnz, counts[2..3] = 0
  *   order [n_rows]   execution order for the attention kernel: canonical row positions grouped by
- *                    head, heads dealt round-robin to 8 queues (head % 8, one queue per XCD);
- *                    inside one head longer rows first (up to 32 length classes), otherwise unspecified
+ *                    head, heads dealt round-robin to 8 queues (head % 8, one queue per XCD).  Inside
+ *                    one head: with eight or more rows per CU, ascending (request, q block), a fixed
+ *                    order in which the entries popped together share kv blocks (sched[32] = 1);
+ *                    with fewer, longer rows first (up to 32 length classes), otherwise unspecified
  *   sched [1024]     sched[0..8] = queue boundaries inside `order`, sched[16..23] = queue cursors
  *                    and sched[24] = completion counter, both cleared to 0; sched[25] = kv count of
  *                    the longest row; sched[26..30] = even shares: in use, cost share of a
  *                    workgroup, total cost, number of shares, number of rows; sched[31] = the
- *                    share table holds queue-entry records;
+ *                    share table holds queue-entry records; sched[32] = `order` is the fixed
+ *                    ascending one;
  *                    sched[64..575] = arrival counters of rows cut at share boundaries (cleared)
  * shares (optional, [512 + 8*(n_blk*H + 1)] int32, 16-byte aligned): scheduling table for the
  * attention kernel, to be passed to fo_sparse_fa_run with the list.  Normally (sched[31] = 1) it

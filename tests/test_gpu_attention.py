@@ -398,7 +398,7 @@ def test_grouped_query_attention(dev, heads, layout):
 
 @pytest.mark.parametrize("config", [3, 4])
 def test_video_shapes_sampled_rows(dev, config):
-    """Configs 3 and 4 at full size (H=40, seq 17776 and 76112, ragged last block): the kernel runs
+    """Configs 3 and 4 at full size (H=24, seq 33 280 and H=40, seq 76 112 with a ragged last block): the kernel runs
     the whole work list; every row of the first and last q-block plus 64 seeded random rows are
     checked against the oracle, and skipped (q-block, head) strips keep their bytes."""
     import flashomni_amd as fo

@@ -211,3 +211,43 @@ def test_decoder_queue_records(dev):
     assert (rec[:, 2] == wl.row_qb[:n_rows].cpu().numpy()[order]).all()
     assert (rec[:, 3] == wl.row_head[:n_rows].cpu().numpy()[order]).all()
     assert (rec[:, 4] == ptr[order]).all() and (rec[:, 5] == ptr[order + 1] - ptr[order]).all()
+
+
+@pytest.mark.parametrize("share_table", [True, False])
+def test_decoder_long_list_order(dev, share_table):
+    """Eight or more rows per CU: inside a head the rows are queued with ascending (request, q block),
+    a fixed order; queues by head % 8; with a share table one record per queue entry."""
+    import flashomni_amd as fo
+    n_cu = torch.cuda.get_device_properties(dev).multi_processor_count
+    heads = 12
+    nq = -(-(8 * n_cu) // heads) + 40           # enough q blocks for 8 rows per CU at p = 0.9
+    ql, kl = [nq * 128 - 50, 700], [1500, 300]
+    m = make_ragged_masks(ql, kl, heads, 0.9, 0.5, seed=9)
+    w = fo.BatchFlashOmniFAWithRaggedKVWrapper(torch.empty(128 << 20, dtype=torch.uint8, device=dev))
+    w._share_rows = share_table
+    w.plan(torch.from_numpy(m["qo_indptr"]), torch.from_numpy(m["kv_indptr"]), heads, heads, 128,
+           q_data_type=torch.bfloat16)
+    t = lambda a: torch.from_numpy(a).to(dev)
+    wl = w.decode(t(m["packed_info"]), t(m["packed_keep"]), t(m["info_indptr"]), t(m["keep_indptr"]))
+    n_rows, _ = wl.sizes()
+    assert n_rows >= 8 * n_cu
+    sched = wl.sched.cpu().numpy()
+    order = wl.order[:n_rows].cpu().numpy()
+    row_head = wl.row_head[:n_rows].cpu().numpy()
+    ptr = wl.kv_row_ptr[:n_rows + 1].cpu().numpy()
+    # canonical positions ascend with (request, q block): a head's rows in canonical order
+    exp = np.concatenate([np.nonzero(row_head == h)[0] for x in range(8) for h in range(x, heads, 8)])
+    assert (order == exp).all()
+    bounds = np.concatenate([[0], np.cumsum([sum(int((row_head == h).sum()) for h in range(x, heads, 8))
+                                             for x in range(8)])])
+    assert (sched[:9] == bounds).all()
+    assert (sched[16:25] == 0).all() and sched[25] == int((ptr[1:] - ptr[:-1]).max())
+    assert sched[26] == 0 and sched[31] == int(share_table) and sched[32] == 1
+    if share_table:
+        rec = wl.shares.cpu().numpy()[512:512 + 8 * n_rows].reshape(n_rows, 8)
+        assert (rec[:, 0] == order).all()
+        assert (rec[:, 1] == wl.row_req[:n_rows].cpu().numpy()[order]).all()
+        assert (rec[:, 2] == wl.row_qb[:n_rows].cpu().numpy()[order]).all()
+        assert (rec[:, 3] == row_head[order]).all()
+        assert (rec[:, 4] == ptr[order]).all() and (rec[:, 5] == ptr[order + 1] - ptr[order]).all()
+        assert (rec[:, 6:] == 0).all()
