@@ -25,6 +25,8 @@
 // Symbol semantics (reference: include/flashomni/attention/prefill.cuh:1284-1294, 1380-1403,
 // 1434-1460): bit 1 = compute/keep, little-endian bytes, flag bit index qb*H + h, keep-mask bit
 // index (qb*H + h)*NKV + kvb, per-request byte offsets.
+#include <mutex>
+
 #include "fo_common.h"
 
 namespace {
@@ -463,6 +465,12 @@ __global__ void __launch_bounds__(kCountThreads) decode_fill_kernel(
 
 }  // namespace
 
+// Scratch of the entry point that takes no scratch argument: the per-candidate flags and counts of
+// the count kernel (2 * n_blk * H ints) and the per-(head, length class) cursors (8192 ints).  1 MiB per
+// device, held until the process ends.
+constexpr int64_t kStaticScratchInts = 262144;
+static __device__ __align__(256) int32_t scratch[kStaticScratchInts];
+
 namespace {
 
 int decode_impl(const uint8_t* sparse_info, const uint8_t* sparse_kv_info, const int32_t* sparse_info_indptr,
@@ -513,6 +521,25 @@ int decode_impl(const uint8_t* sparse_info, const uint8_t* sparse_kv_info, const
   return FO_OK;
 }
 
+// device address of `scratch` on the current device (every device holds its own copy of the array
+// at its own address); looked up once per device
+int static_scratch(int32_t** out) {
+  static std::mutex mu;
+  static int32_t* ptrs[64] = {};
+  int dev = 0;
+  FO_HIP_CALL(hipGetDevice(&dev));
+  FO_REQUIRE(dev >= 0 && dev < 64, "decode: device index %d out of range", dev);
+  std::lock_guard<std::mutex> lock(mu);
+  if (ptrs[dev] == nullptr) {
+    void* p = nullptr;
+    FO_HIP_CALL(hipGetSymbolAddress(&p, HIP_SYMBOL(scratch)));
+    FO_REQUIRE(p != nullptr, "decode: the static scratch array has no device address");
+    ptrs[dev] = static_cast<int32_t*>(p);
+  }
+  *out = ptrs[dev];
+  return FO_OK;
+}
+
 }  // namespace
 
 extern "C" int fo_decode_sparse(const uint8_t* sparse_info, const uint8_t* sparse_kv_info,
@@ -527,4 +554,30 @@ extern "C" int fo_decode_sparse(const uint8_t* sparse_info, const uint8_t* spars
   return decode_impl(sparse_info, sparse_kv_info, sparse_info_indptr, sparse_kv_info_indptr, blk_req, blk_qb,
                      kv_indptr, n_blk, num_heads, block_kv, is_full, row_req, row_qb, row_head, kv_row_ptr,
                      kv_idx, counts, order, sched, scratch, shares, stream);
+}
+
+extern "C" int64_t fo_decode_sparse_static_max_pairs(void) { return (kStaticScratchInts - kHistSlots) / 2; }
+
+extern "C" int fo_decode_sparse_static(const uint8_t* sparse_info, const uint8_t* sparse_kv_info,
+                                       const int32_t* sparse_info_indptr,
+                                       const int32_t* sparse_kv_info_indptr, const int32_t* blk_req,
+                                       const int32_t* blk_qb, const int32_t* kv_indptr, int32_t n_blk,
+                                       int32_t num_heads, int32_t block_kv, int is_full,
+                                       int32_t* row_req, int32_t* row_qb, int32_t* row_head,
+                                       int32_t* kv_row_ptr, int32_t* kv_idx, int32_t* counts,
+                                       int32_t* order, int32_t* sched, int32_t* shares, void* stream) {
+  FO_REQUIRE(n_blk >= 0 && num_heads > 0, "decode: bad sizes");
+  const int64_t n_cand = static_cast<int64_t>(n_blk) * num_heads;
+  FO_REQUIRE(n_cand <= fo_decode_sparse_static_max_pairs(),
+             "decode: %lld (q-block, head) pairs exceed the %lld the built-in scratch holds; use "
+             "fo_decode_sparse with a caller-provided scratch",
+             static_cast<long long>(n_cand), static_cast<long long>(fo_decode_sparse_static_max_pairs()));
+  int32_t* ptr = nullptr;
+  const int rc = static_scratch(&ptr);
+  if (rc != FO_OK) return rc;
+  // (nothing in the scratch has to start at zero: the count kernel writes every flag and count the
+  // later kernels read, the scan kernel every cursor)
+  return decode_impl(sparse_info, sparse_kv_info, sparse_info_indptr, sparse_kv_info_indptr, blk_req, blk_qb,
+                     kv_indptr, n_blk, num_heads, block_kv, is_full, row_req, row_qb, row_head, kv_row_ptr,
+                     kv_idx, counts, order, sched, ptr, shares, stream);
 }

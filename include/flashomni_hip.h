@@ -131,6 +131,26 @@ int fo_decode_sparse(const uint8_t* sparse_info, const uint8_t* sparse_kv_info,
                      int32_t* scratch, int32_t* shares, void* stream);
 
 /* ---------------------------------------------------------------------------------------------
+ * fo_decode_sparse without the `scratch` argument, for callers that cannot allocate device memory
+ * for it (code under HIP graph capture, tight serving loops, harnesses that forbid hipMalloc).
+ * No counterpart in the reference.  The decoder's scratch (2*n_blk*H + 8192 int32) lives in a 1 MiB
+ * array built into the library's device code instead (one copy per GPU, held until the process ends),
+ * so n_blk * num_heads may be at most fo_decode_sparse_static_max_pairs() (126 976); larger
+ * inputs are refused with FO_ERR_INVALID.  Same inputs, outputs and results as fo_decode_sparse.
+ * The call allocates nothing (its first call on a device looks up the array's address).  All calls
+ * on one GPU share that array: calls that overlap in time on one GPU (two streams, two threads)
+ * race; calls on one stream are safe.
+ * ------------------------------------------------------------------------------------------- */
+int64_t fo_decode_sparse_static_max_pairs(void);
+int fo_decode_sparse_static(const uint8_t* sparse_info, const uint8_t* sparse_kv_info,
+                            const int32_t* sparse_info_indptr, const int32_t* sparse_kv_info_indptr,
+                            const int32_t* blk_req, const int32_t* blk_qb, const int32_t* kv_indptr,
+                            int32_t n_blk, int32_t num_heads, int32_t block_kv, int is_full,
+                            int32_t* row_req, int32_t* row_qb, int32_t* row_head, int32_t* kv_row_ptr,
+                            int32_t* kv_idx, int32_t* counts, int32_t* order, int32_t* sched,
+                            int32_t* shares, void* stream);
+
+/* ---------------------------------------------------------------------------------------------
  * Ragged block-sparse FlashAttention prefill over a decoded work list.
  * replaces: BatchSparseFAWithRaggedKVRun csrc/batch_sparseFA.cu:67-201 and the kernel
  *           include/flashomni/attention/prefill.cuh:1203-1531 (mask none, no positional
