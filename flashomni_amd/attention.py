@@ -204,7 +204,7 @@ class PlannedBatch:
             cur.wait_event(ev)
         return self.worklist
 
-    def launch(self, q, k, v, out, lse, kv_layout, sm_scale, q_scale=None, k_scale=None) -> None:
+    def launch(self, q, k, v, out, lse, kv_layout, sm_scale, q_scale=None, k_scale=None, q_lo=None) -> None:
         """Shape checks against the planned batch, then fo_sparse_fa_run over the decoded list."""
         if q.dim() != 3 or k.dim() != 3 or v.dim() != 3 or k.size(2) != 128 or v.size(2) != 128:
             raise ValueError("q, k and v must be 3-dimensional with head_dim 128")
@@ -215,6 +215,11 @@ class PlannedBatch:
                 raise ValueError("fp8 attention needs float8_e4m3fn q and k with q_scale and k_scale")
             if v.dtype != torch.bfloat16:
                 raise ValueError("fp8 attention keeps v (and the output) in bfloat16")
+            if q_lo is not None and (q_lo.dtype != q.dtype or q_lo.shape != q.shape
+                                     or q_lo.stride() != q.stride() or q_lo.device != q.device):
+                raise ValueError("q_lo must be a float8_e4m3fn tensor laid out like q")
+        elif q_lo is not None:
+            raise ValueError("q_lo is the second term of an fp8 q")
         if q.device != self.device:
             raise ValueError(f"Invalid device of q: expected {self.device}, got {q.device}")
         if q.size(1) != self.num_qo_heads or q.size(2) != 128:
@@ -246,7 +251,7 @@ class PlannedBatch:
         with _lib.device_guard(self.device):
             _lib.check(_lib.lib().fo_sparse_fa_run(
                 _lib.ptr(q), _lib.ptr(k), _lib.ptr(v), _lib.ptr(out), _lib.ptr(lse),
-                _lib.dtype_code(q.dtype), _lib.ptr(q_scale if fp8 else None),
+                _lib.dtype_code(q.dtype), _lib.ptr(q_lo), _lib.ptr(q_scale if fp8 else None),
                 _lib.ptr(k_scale if fp8 else None),
                 q.stride(0), q.stride(1), k_sn, k_sh, v_sn, v_sh, out.stride(0), out.stride(1),
                 _lib.ptr(self.qo_indptr), _lib.ptr(self.kv_indptr), _lib.ptr(self.q_blk_base),
@@ -506,6 +511,7 @@ class BatchFlashOmniFAWithRaggedKVWrapper:
         return_lse: bool = False,
         q_scale: Optional[torch.Tensor] = None,
         k_scale: Optional[torch.Tensor] = None,
+        q_lo: Optional[torch.Tensor] = None,
         reuse_decoded: bool = False,
     ) -> Union[torch.Tensor, Tuple[torch.Tensor, torch.Tensor]]:
         r"""Compute block-sparse prefill attention.
@@ -517,6 +523,11 @@ class BatchFlashOmniFAWithRaggedKVWrapper:
 
         ``q_scale`` / ``k_scale`` (keyword-only extension): fp32 ``[H, n_blocks]`` dequantisation
         scales; with them ``q`` and ``k`` are fp8 e4m3fn, ``v`` and ``out`` are bfloat16.
+        ``q_lo``: optional second fp8 term of ``q`` (the rounding residual that
+        ``quant_fp8_block(..., residual=True)`` / ``flashomni_gemm(..., quant_out="residual")``
+        return): the logits are computed from ``q + q_lo``, which leaves only the rounding of ``k``
+        in them and brings the output within relative L2 3e-2 of the unquantised result for
+        unit-variance q (two e4m3 operands alone give ~3.9e-2).
 
         ``reuse_decoded`` (keyword-only extension): the symbols are decoded on every call, because
         a buffer rewritten in place (by a kernel of the caller's, through the C ABI, ...) looks the
@@ -546,7 +557,7 @@ class BatchFlashOmniFAWithRaggedKVWrapper:
             pb.reuse_decoded(is_full)
         else:
             pb.decode(sparse_info, sparse_kv_info, sparse_info_indptr, sparse_kv_info_indptr, is_full)
-        pb.launch(q, k, v, out, lse if return_lse else None, self._kv_layout, sm_scale, q_scale, k_scale)
+        pb.launch(q, k, v, out, lse if return_lse else None, self._kv_layout, sm_scale, q_scale, k_scale, q_lo)
         return (out, lse) if return_lse else out
 
     run_return_lse = functools.partialmethod(run, return_lse=True)

@@ -112,6 +112,7 @@ struct GemmParams {
   // GEMM-Q with fused quantisation: e4m3fn bytes [B, M, N] and one scale per (head, token block),
   // y_scale[head * scale_row_len + b * n_row_tiles + token block]; y may then be null
   uint8_t* y8;
+  uint8_t* y8_lo;  // optional second term: the residual result / scale - y8, rounded to e4m3 again
   float* y_scale;
   int32_t scale_row_len;
 };
@@ -769,6 +770,15 @@ __global__ void __launch_bounds__(kThreads) gemm_kernel(const GemmParams p) {
                 w8 = __builtin_amdgcn_cvt_pk_fp8_f32(f[0], f[1], w8, false);
                 w8 = __builtin_amdgcn_cvt_pk_fp8_f32(f[2], f[3], w8, true);
                 *reinterpret_cast<unsigned*>(p.y8 + off) = w8;
+                if (p.y8_lo) {
+                  typedef __attribute__((ext_vector_type(2))) float f32x2;
+                  const f32x2 h0 = __builtin_amdgcn_cvt_pk_f32_fp8(w8, false);
+                  const f32x2 h1 = __builtin_amdgcn_cvt_pk_f32_fp8(w8, true);
+                  unsigned l8 = 0;
+                  l8 = __builtin_amdgcn_cvt_pk_fp8_f32(f[0] - h0[0], f[1] - h0[1], l8, false);
+                  l8 = __builtin_amdgcn_cvt_pk_fp8_f32(f[2] - h1[0], f[3] - h1[1], l8, true);
+                  *reinterpret_cast<unsigned*>(p.y8_lo + off) = l8;
+                }
               }
             }
           }
@@ -895,8 +905,8 @@ extern "C" int64_t fo_gemm_workspace_bytes(int32_t batch, int32_t m, int32_t n) 
 }
 
 namespace {
-int gemm_q_impl(const void* x, const void* w, const void* bias, void* y, uint8_t* y8, float* y_scale,
-                int dtype, int32_t batch, int32_t m, int32_t n, int32_t k, int32_t sparse_q_size,
+int gemm_q_impl(const void* x, const void* w, const void* bias, void* y, uint8_t* y8, uint8_t* y8_lo,
+                float* y_scale, int dtype, int32_t batch, int32_t m, int32_t n, int32_t k, int32_t sparse_q_size,
                 int32_t num_qo_heads, const uint8_t* sparse_info, const int32_t* sparse_info_indptr,
                 int32_t num_text_tokens, int is_full, void* workspace, int64_t workspace_bytes,
                 void* stream) {
@@ -921,7 +931,10 @@ int gemm_q_impl(const void* x, const void* w, const void* bias, void* y, uint8_t
   if (y8) {
     FO_REQUIRE(y_scale, "gemm_q_quant: y_scale is null");
     FO_REQUIRE(p.head_dim == kTile, "gemm_q_quant: head width %d is not supported (only 128)", p.head_dim);
+    FO_REQUIRE((reinterpret_cast<uintptr_t>(y8) & 3) == 0 && (reinterpret_cast<uintptr_t>(y8_lo) & 3) == 0,
+               "gemm_q_quant: y8 and y8_lo must be 4-byte aligned");
     p.y8 = y8;
+    p.y8_lo = y8_lo;
     p.y_scale = y_scale;
     p.scale_row_len = batch * gm.n_row_tiles;
   }
@@ -937,19 +950,19 @@ extern "C" int fo_gemm_q(const void* x, const void* w, const void* bias, void* y
                          const int32_t* sparse_info_indptr, int32_t num_text_tokens, int is_full,
                          void* workspace, int64_t workspace_bytes, void* stream) {
   FO_REQUIRE(y, "gemm: null pointer");
-  return gemm_q_impl(x, w, bias, y, nullptr, nullptr, dtype, batch, m, n, k, sparse_q_size,
+  return gemm_q_impl(x, w, bias, y, nullptr, nullptr, nullptr, dtype, batch, m, n, k, sparse_q_size,
                      num_qo_heads, sparse_info, sparse_info_indptr, num_text_tokens, is_full, workspace,
                      workspace_bytes, stream);
 }
 
 extern "C" int fo_gemm_q_quant(const void* x, const void* w, const void* bias, void* y, uint8_t* y8,
-                               float* y_scale, int dtype, int32_t batch, int32_t m, int32_t n,
+                               uint8_t* y8_lo, float* y_scale, int dtype, int32_t batch, int32_t m, int32_t n,
                                int32_t k, int32_t sparse_q_size, int32_t num_qo_heads,
                                const uint8_t* sparse_info, const int32_t* sparse_info_indptr,
                                int32_t num_text_tokens, int is_full, void* workspace,
                                int64_t workspace_bytes, void* stream) {
   FO_REQUIRE(y8, "gemm_q_quant: y8 is null");
-  return gemm_q_impl(x, w, bias, y, y8, y_scale, dtype, batch, m, n, k, sparse_q_size, num_qo_heads,
+  return gemm_q_impl(x, w, bias, y, y8, y8_lo, y_scale, dtype, batch, m, n, k, sparse_q_size, num_qo_heads,
                      sparse_info, sparse_info_indptr, num_text_tokens, is_full, workspace,
                      workspace_bytes, stream);
 }

@@ -2,6 +2,8 @@
 // One workgroup per (block, head): the 128 x 128 slab is read once into registers (128-bit loads),
 // reduced to its absmax (wave shuffles + LDS), then divided by scale = absmax/448 and converted with
 // the hardware round-to-nearest-even e4m3 conversion; 2 bytes read + 1 byte written per element.
+// Optionally a second e4m3 tensor takes the residual, x/scale - x8 rounded again, so that x8 + x8_lo
+// carries x/scale to about 7 significant bits (a two-term operand for the fp8 matrix cores).
 // The reference has no such kernel (its quantization.cuh only packs bits).
 #include "fo_common.h"
 
@@ -18,7 +20,7 @@ constexpr float kFp8Max = 448.0f;
 template <typename X8>
 __global__ void __launch_bounds__(kThreads) quant_fp8_kernel(
     const void* __restrict__ xv, int64_t sn, int64_t sh, uint8_t* __restrict__ x8,
-    float* __restrict__ scale, const int32_t* __restrict__ blk_tok0,
+    uint8_t* __restrict__ x8_lo, float* __restrict__ scale, const int32_t* __restrict__ blk_tok0,
     const int32_t* __restrict__ blk_len, int32_t n_blk, int32_t num_heads) {
   using T = decltype(X8{}[0]);
   __shared__ float s_red[kThreads / 64];
@@ -67,6 +69,20 @@ __global__ void __launch_bounds__(kThreads) quant_fp8_kernel(
       out[1] = w1;
       const int64_t o = (static_cast<int64_t>(tok0 + r) * num_heads + head) * kBlock + col;
       *reinterpret_cast<u32x2*>(x8 + o) = out;
+      if (x8_lo) {
+        typedef __attribute__((ext_vector_type(2))) float f32x2;
+        const f32x2 h0 = __builtin_amdgcn_cvt_pk_f32_fp8(w0, false), h1 = __builtin_amdgcn_cvt_pk_f32_fp8(w0, true);
+        const f32x2 h2 = __builtin_amdgcn_cvt_pk_f32_fp8(w1, false), h3 = __builtin_amdgcn_cvt_pk_f32_fp8(w1, true);
+        unsigned l0 = 0, l1 = 0;
+        l0 = __builtin_amdgcn_cvt_pk_fp8_f32(f[0] - h0[0], f[1] - h0[1], l0, false);
+        l0 = __builtin_amdgcn_cvt_pk_fp8_f32(f[2] - h1[0], f[3] - h1[1], l0, true);
+        l1 = __builtin_amdgcn_cvt_pk_fp8_f32(f[4] - h2[0], f[5] - h2[1], l1, false);
+        l1 = __builtin_amdgcn_cvt_pk_fp8_f32(f[6] - h3[0], f[7] - h3[1], l1, true);
+        u32x2 lo;
+        lo[0] = l0;
+        lo[1] = l1;
+        *reinterpret_cast<u32x2*>(x8_lo + o) = lo;
+      }
     }
   }
 }
@@ -74,7 +90,7 @@ __global__ void __launch_bounds__(kThreads) quant_fp8_kernel(
 }  // namespace
 
 extern "C" int fo_quant_fp8_block(const void* x, int dtype, int64_t x_stride_n, int64_t x_stride_h,
-                                  uint8_t* x8, float* scale, const int32_t* blk_tok0,
+                                  uint8_t* x8, uint8_t* x8_lo, float* scale, const int32_t* blk_tok0,
                                   const int32_t* blk_len, int32_t n_blk, int32_t num_heads,
                                   int32_t head_dim, void* stream) {
   FO_REQUIRE(dtype == FO_BF16 || dtype == FO_F16, "quant_fp8: input must be bf16 or fp16");
@@ -83,15 +99,16 @@ extern "C" int fo_quant_fp8_block(const void* x, int dtype, int64_t x_stride_n, 
   if (n_blk == 0) return FO_OK;
   FO_REQUIRE(x && x8 && scale && blk_tok0 && blk_len, "quant_fp8: null pointer");
   FO_REQUIRE(x_stride_n % 8 == 0 && x_stride_h % 8 == 0 &&
-                 (reinterpret_cast<uintptr_t>(x) & 15) == 0 && (reinterpret_cast<uintptr_t>(x8) & 7) == 0,
+                 (reinterpret_cast<uintptr_t>(x) & 15) == 0 && (reinterpret_cast<uintptr_t>(x8) & 7) == 0 &&
+                 (reinterpret_cast<uintptr_t>(x8_lo) & 7) == 0,
              "quant_fp8: x must be 16-byte aligned with strides that are multiples of 8");
   dim3 grid(n_blk, num_heads);
   hipStream_t s = static_cast<hipStream_t>(stream);
   if (dtype == FO_BF16) {
-    quant_fp8_kernel<bf16x8><<<grid, kThreads, 0, s>>>(x, x_stride_n, x_stride_h, x8, scale,
+    quant_fp8_kernel<bf16x8><<<grid, kThreads, 0, s>>>(x, x_stride_n, x_stride_h, x8, x8_lo, scale,
                                                       blk_tok0, blk_len, n_blk, num_heads);
   } else {
-    quant_fp8_kernel<f16x8><<<grid, kThreads, 0, s>>>(x, x_stride_n, x_stride_h, x8, scale,
+    quant_fp8_kernel<f16x8><<<grid, kThreads, 0, s>>>(x, x_stride_n, x_stride_h, x8, x8_lo, scale,
                                                      blk_tok0, blk_len, n_blk, num_heads);
   }
   FO_CHECK_LAUNCH();

@@ -102,6 +102,7 @@ struct FaParams {
   const void* v;
   void* o;
   float* lse;
+  const void* q_lo;  // fp8: optional second e4m3 term of q (same layout and scale as q)
   const float* q_scale;
   const float* k_scale;
   int64_t q_sn, q_sh, k_sn, k_sh, v_sn, v_sh, o_sn, o_sh;
@@ -248,9 +249,14 @@ __device__ __forceinline__ int pop_row(const FaParams& p, int xcd, const int* q,
 // T: element type of V, P and O (and of Q, K unless kFp8).  kFp8: Q and K are e4m3fn bytes with one
 // dequantisation scale per (head, 128-token block); S^T then comes from
 // v_mfma_scale_f32_32x32x64_f8f6f4 (64 d per instruction, unit block scale) and the two per-block
-// scales are folded into the softmax scale of the tile.
-template <typename T, bool kFp8>
+// scales are folded into the softmax scale of the tile.  kQLo: q comes as two e4m3 terms, q + q_lo
+// (the second one the rounding residual of the first), and S^T = K.(q + q_lo)^T takes two MFMAs
+// per slab: e4m3 keeps 3 mantissa bits, and with both operands rounded to it the logits are too
+// noisy for the accuracy this path promises; with the two-term q only k's rounding is left.  The
+// fp8 matrix cores run at twice the 16-bit rate, so the two terms cost what a 16-bit S^T costs.
+template <typename T, bool kFp8, bool kQLo>
 __global__ void __launch_bounds__(kThreads) sparse_fa_kernel(const FaParams p) {
+  static_assert(kFp8 || !kQLo, "the two-term q is an fp8 form");
   using TT = Types<T>;
   using x8 = typename TT::x8;
   using x4 = typename TT::x4;
@@ -498,6 +504,7 @@ __global__ void __launch_bounds__(kThreads) sparse_fa_kernel(const FaParams p) {
     // from there.  Requested first so that the latency overlaps the staging below.
     x8 qreg[kFp8 ? 1 : 8];
     i32x8 qreg8[kFp8 ? 2 : 1];
+    i32x8 qlo8[kQLo ? 2 : 1];
     const uint32_t lds_group = static_cast<uint32_t>(reinterpret_cast<uintptr_t>((lds_void*)group_smem));
     if constexpr (kFp8) {
       // (fp8 Q, half the bytes, is still fetched directly: with the LDS detour hipcc arranges the
@@ -508,6 +515,16 @@ __global__ void __launch_bounds__(kThreads) sparse_fa_kernel(const FaParams p) {
         const i32x4 lo = *reinterpret_cast<const i32x4*>(src + sl * 64);
         const i32x4 hi = *reinterpret_cast<const i32x4*>(src + sl * 64 + 16);
         qreg8[sl] = i32x8{lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
+      }
+      if constexpr (kQLo) {
+        const uint8_t* src2 = static_cast<const uint8_t*>(p.q_lo) + q_tok * p.q_sn +
+                              static_cast<int64_t>(head) * p.q_sh + g * 32;
+#pragma unroll
+        for (int sl = 0; sl < 2; ++sl) {
+          const i32x4 lo = *reinterpret_cast<const i32x4*>(src2 + sl * 64);
+          const i32x4 hi = *reinterpret_cast<const i32x4*>(src2 + sl * 64 + 16);
+          qlo8[sl] = i32x8{lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
+        }
       }
     } else {
       const uint8_t* q_head = reinterpret_cast<const uint8_t*>(
@@ -734,6 +751,15 @@ __global__ void __launch_bounds__(kThreads) sparse_fa_kernel(const FaParams p) {
           for (int sl = 0; sl < 2; ++sl)
             s[mt] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(k8[mt][sl], qreg8[sl], s[mt], 0, 0, 0,
                                                                     0x7f7f7f7f, 0, 0x7f7f7f7f);
+        }
+        if constexpr (kQLo) {
+          // (second pass so that the two accumulator chains keep alternating)
+#pragma unroll
+          for (int sl = 0; sl < 2; ++sl)
+#pragma unroll
+            for (int mt = 0; mt < 2; ++mt)
+              s[mt] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(k8[mt][sl], qlo8[sl], s[mt], 0, 0, 0,
+                                                                      0x7f7f7f7f, 0, 0x7f7f7f7f);
         }
       }
     };
@@ -1126,7 +1152,7 @@ __global__ void __launch_bounds__(kThreads) sparse_fa_kernel(const FaParams p) {
   }
 }
 
-template <typename T, bool kFp8>
+template <typename T, bool kFp8, bool kQLo>
 int launch(const FaParams& p, int64_t max_rows, hipStream_t stream) {
   constexpr int kSmemBytes = Geom<kFp8>::kSmemBytes;
   // (the attribute belongs to the kernel's code object on one device: set once per device; the flags
@@ -1135,7 +1161,7 @@ int launch(const FaParams& p, int64_t max_rows, hipStream_t stream) {
   int dev = 0;
   FO_HIP_CALL(hipGetDevice(&dev));
   if (dev < 0 || dev >= 64 || !attr_set[dev].load(std::memory_order_acquire)) {
-    FO_HIP_CALL(hipFuncSetAttribute(reinterpret_cast<const void*>(&sparse_fa_kernel<T, kFp8>),
+    FO_HIP_CALL(hipFuncSetAttribute(reinterpret_cast<const void*>(&sparse_fa_kernel<T, kFp8, kQLo>),
                                     hipFuncAttributeMaxDynamicSharedMemorySize, kSmemBytes));
     if (dev >= 0 && dev < 64) attr_set[dev].store(true, std::memory_order_release);
   }
@@ -1144,7 +1170,7 @@ int launch(const FaParams& p, int64_t max_rows, hipStream_t stream) {
   int64_t grid = num_cu;  // one persistent workgroup per CU (LDS bound)
   // (with even shares every workgroup may hold a part of a row; otherwise at most one row each)
   if (!(p.split_ws && p.shares) && grid > max_rows) grid = max_rows;
-  sparse_fa_kernel<T, kFp8><<<static_cast<unsigned>(grid), kThreads, kSmemBytes, stream>>>(p);
+  sparse_fa_kernel<T, kFp8, kQLo><<<static_cast<unsigned>(grid), kThreads, kSmemBytes, stream>>>(p);
   FO_CHECK_LAUNCH();
   return FO_OK;
 }
@@ -1157,7 +1183,7 @@ extern "C" int64_t fo_sparse_fa_split_workspace_bytes(void) {
 }
 
 extern "C" int fo_sparse_fa_run(const void* q, const void* k, const void* v, void* o, float* lse,
-                                int dtype, const float* q_scale, const float* k_scale,
+                                int dtype, const void* q_lo, const float* q_scale, const float* k_scale,
                                 int64_t q_stride_n, int64_t q_stride_h, int64_t k_stride_n,
                                 int64_t k_stride_h, int64_t v_stride_n, int64_t v_stride_h,
                                 int64_t o_stride_n, int64_t o_stride_h, const int32_t* qo_indptr,
@@ -1194,13 +1220,14 @@ extern "C" int fo_sparse_fa_run(const void* q, const void* k, const void* v, voi
   if (dtype == FO_FP8_E4M3)
     FO_REQUIRE(q_scale && k_scale && q_blk_base && kv_blk_base && n_q_blocks > 0 && n_kv_blocks > 0,
                "sparse_fa: fp8 q/k need q_scale, k_scale, the block numbering and the scale row lengths");
-  for (const void* ptr : {q, k, v, static_cast<const void*>(o)})
+  FO_REQUIRE(q_lo == nullptr || dtype == FO_FP8_E4M3, "sparse_fa: q_lo is the second term of an fp8 q");
+  for (const void* ptr : {q, k, v, static_cast<const void*>(o), q_lo})
     FO_REQUIRE((reinterpret_cast<uintptr_t>(ptr) & 15) == 0,
                "sparse_fa: q/k/v/o must be 16-byte aligned");
 
   FaParams p;
   p.q = q; p.k = k; p.v = v; p.o = o; p.lse = lse;
-  p.q_scale = q_scale; p.k_scale = k_scale;
+  p.q_lo = q_lo; p.q_scale = q_scale; p.k_scale = k_scale;
   p.q_sn = q_stride_n; p.q_sh = q_stride_h; p.k_sn = k_stride_n; p.k_sh = k_stride_h;
   p.v_sn = v_stride_n; p.v_sh = v_stride_h; p.o_sn = o_stride_n; p.o_sh = o_stride_h;
   p.qo_indptr = qo_indptr; p.kv_indptr = kv_indptr;
@@ -1223,7 +1250,8 @@ extern "C" int fo_sparse_fa_run(const void* q, const void* k, const void* v, voi
   p.num_heads = num_heads; p.kv_group = num_heads / num_kv_heads; p.n_q_blocks = n_q_blocks; p.n_kv_blocks = n_kv_blocks;
   p.sm_scale_log2 = sm_scale * 1.44269504088896340736f;
   hipStream_t s = static_cast<hipStream_t>(stream);
-  if (dtype == FO_BF16) return launch<__bf16, false>(p, max_rows, s);
-  if (dtype == FO_F16) return launch<_Float16, false>(p, max_rows, s);
-  return launch<__bf16, true>(p, max_rows, s);
+  if (dtype == FO_BF16) return launch<__bf16, false, false>(p, max_rows, s);
+  if (dtype == FO_F16) return launch<_Float16, false, false>(p, max_rows, s);
+  if (q_lo != nullptr) return launch<__bf16, true, true>(p, max_rows, s);
+  return launch<__bf16, true, false>(p, max_rows, s);
 }

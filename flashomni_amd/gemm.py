@@ -81,14 +81,17 @@ def flashomni_gemm(
     ``sparse_info`` bit is 1; the other tiles of ``out`` are left untouched (a fresh ``out`` is
     ``torch.empty``, as in the reference).
 
-    ``quant_out`` (keyword-only extension, heads of width 128): ``(q8, scale)`` or ``True``.  The
+    ``quant_out`` (keyword-only extension, heads of width 128): ``(q8, scale)``, ``(q8, scale, q8_lo)``,
+    ``True`` or ``"residual"`` (allocate two resp. three outputs).  The
     computed tiles are also written as fp8 e4m3fn with one absmax scale per (head, 128-token block),
     taken from the fp32 results before they are rounded: ``q8`` ``[B, M, N]`` float8_e4m3fn and
     ``scale`` ``[H, B * ceil(M / 128)]`` float32, the operands
     :meth:`BatchFlashOmniFAWithRaggedKVWrapper.run` takes as ``q`` and ``q_scale`` (what
-    :func:`quant_fp8_block` would make of ``out`` in a second pass).  With ``quant_out`` given and
+    :func:`quant_fp8_block` would make of ``out`` in a second pass); ``q8_lo`` is the rounding
+    residual of ``q8`` under the same scale (``q_lo`` of ``run``).  With ``quant_out`` given and
     ``out=False`` the 16-bit result is not written at all.  Returns ``out``, or ``(out, q8, scale)``
-    when ``quant_out`` is given (``out`` is None if it was not written)."""
+    resp. ``(out, q8, scale, q8_lo)`` when ``quant_out`` is given (``out`` is None if it was not
+    written)."""
     _check_gemm_operands(A, B, "flashomni_gemm")
     skip_out = out is False
     if skip_out:
@@ -126,11 +129,21 @@ def flashomni_gemm(
         return out
     Bsz, M, N = A.shape[0], A.shape[1], B.shape[0]
     n_blk = Bsz * ((M + 127) // 128)
-    if quant_out is True:
+    q8_lo = None
+    if quant_out is True or quant_out == "residual":
         q8 = torch.empty((Bsz, M, N), dtype=torch.float8_e4m3fn, device=A.device)
         scale = torch.empty((num_qo_heads, n_blk), dtype=torch.float32, device=A.device)
+        if quant_out == "residual":
+            q8_lo = torch.empty_like(q8)
     else:
-        q8, scale = quant_out
+        if len(quant_out) == 3:
+            q8, scale, q8_lo = quant_out
+            if q8_lo.shape != (Bsz, M, N) or q8_lo.dtype not in (torch.float8_e4m3fn, torch.uint8) \
+                    or not q8_lo.is_contiguous() or q8_lo.device != A.device:
+                raise RuntimeError("flashomni_gemm: quant_out[2] must be a contiguous [B, M, N] float8_e4m3fn "
+                                   "tensor")
+        else:
+            q8, scale = quant_out
         if q8.shape != (Bsz, M, N) or q8.dtype not in (torch.float8_e4m3fn, torch.uint8) \
                 or not q8.is_contiguous() or q8.device != A.device:
             raise RuntimeError("flashomni_gemm: quant_out[0] must be a contiguous [B, M, N] float8_e4m3fn tensor")
@@ -140,11 +153,11 @@ def flashomni_gemm(
                                "float32 tensor")
     with _lib.device_guard(A.device):
         _lib.check(L.fo_gemm_q_quant(
-            _lib.ptr(A), _lib.ptr(B), _lib.ptr(bias), _lib.ptr(out), _lib.ptr(q8), _lib.ptr(scale),
-            _lib.dtype_code(A.dtype), Bsz, M, N, A.shape[2], sparse_q_size, num_qo_heads,
+            _lib.ptr(A), _lib.ptr(B), _lib.ptr(bias), _lib.ptr(out), _lib.ptr(q8), _lib.ptr(q8_lo),
+            _lib.ptr(scale), _lib.dtype_code(A.dtype), Bsz, M, N, A.shape[2], sparse_q_size, num_qo_heads,
             _lib.ptr(info), _lib.ptr(indptr), num_text_tokens, int(bool(is_full)),
             _lib.ptr(workspace), ws_bytes, stream))
-    return out, q8, scale
+    return (out, q8, scale) if q8_lo is None else (out, q8, scale, q8_lo)
 
 
 def flashomni_gemm_reduction(

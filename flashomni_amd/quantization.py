@@ -93,13 +93,16 @@ def token_blocks(indptr: torch.Tensor, block: int = 128):
 
 
 def quant_fp8_block(x: torch.Tensor, indptr: torch.Tensor, block: int = 128,
-                    blocks=None) -> Tuple[torch.Tensor, torch.Tensor]:
+                    blocks=None, residual: bool = False):
     """Quantise ``x`` [nnz, H, D] (bf16/fp16, GPU) to fp8 e4m3fn with one absmax scale per
     (head, ``block``-token block); blocks never straddle the requests delimited by ``indptr``.
 
     Returns ``(x8 [nnz,H,D] float8_e4m3fn, scale [H, n_blocks] float32)`` with
     ``scale = absmax / 448`` (1 for an all-zero block) and ``x ~= x8 * scale``.
-    ``blocks``: optional cached result of :func:`token_blocks` already on the GPU."""
+    ``blocks``: optional cached result of :func:`token_blocks` already on the GPU.
+    ``residual=True`` returns ``(x8, scale, x8_lo)``: ``x8_lo`` is the rounding residual
+    ``x / scale - x8`` as a second float8_e4m3fn tensor, ``x ~= (x8 + x8_lo) * scale`` to about 7
+    significant bits (the ``q_lo`` operand of fp8 attention)."""
     _require_gpu_tensor(x, "x")
     if block != 128:
         raise ValueError("quant_fp8_block: only 128-token blocks are supported")
@@ -111,10 +114,11 @@ def quant_fp8_block(x: torch.Tensor, indptr: torch.Tensor, block: int = 128,
     tok0, length = blocks
     nnz, H, D = x.shape
     x8 = torch.empty((nnz, H, D), dtype=torch.float8_e4m3fn, device=x.device)
+    x8_lo = torch.empty_like(x8) if residual else None
     scale = torch.empty((H, tok0.numel()), dtype=torch.float32, device=x.device)
     with _lib.device_guard(x.device):
         _lib.check(_lib.lib().fo_quant_fp8_block(
             _lib.ptr(x), _lib.dtype_code(x.dtype), x.stride(0), x.stride(1), _lib.ptr(x8),
-            _lib.ptr(scale), _lib.ptr(tok0), _lib.ptr(length), tok0.numel(), H, D,
+            _lib.ptr(x8_lo), _lib.ptr(scale), _lib.ptr(tok0), _lib.ptr(length), tok0.numel(), H, D,
             _lib.current_stream(x.device)))
-    return x8, scale
+    return (x8, scale, x8_lo) if residual else (x8, scale)

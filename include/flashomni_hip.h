@@ -19,7 +19,7 @@
 extern "C" {
 #endif
 
-#define FO_ABI_VERSION 1
+#define FO_ABI_VERSION 2
 
 enum {
   FO_OK = 0,
@@ -161,7 +161,10 @@ int fo_decode_sparse_static(const uint8_t* sparse_info, const uint8_t* sparse_kv
  * h / (H / H_kv) (grouped-query attention, prefill.cuh:410-413); k_scale then has H_kv rows.  dtype FO_BF16 / FO_F16: q,k,v,o share it.  dtype FO_FP8_E4M3: q and k are e4m3fn bytes
  * with dequantisation scales q_scale[H][n_q_blocks], k_scale[H][n_kv_blocks] (fp32, blocks
  * numbered request by request: q_blk_base / kv_blk_base [batch+1] give each request's first
- * block); v and o are bf16.  (The fp8 form has no counterpart in the reference.)
+ * block); v and o are bf16.  q_lo (optional, else NULL): a second e4m3fn tensor laid out like q, the
+ * rounding residual of q under the same scale (fo_quant_fp8_block / fo_gemm_q_quant write it);
+ * the logits are then K.(q + q_lo)^T, two fp8 products at the cost of one 16-bit one, and only k's
+ * rounding error is left in them.  (The fp8 form has no counterpart in the reference.)
  * Rows of the list write every output row of their q-block; q-blocks not in the list are left
  * untouched; a listed row with no kv block writes zeros and lse = -5e4.  lse (optional, fp32
  * [nnz_q,H]) is base 2: log2(sum 2^(s*c - m*c)) + m*c, c = sm_scale*log2(e).
@@ -179,7 +182,7 @@ int fo_decode_sparse_static(const uint8_t* sparse_info, const uint8_t* sparse_kv
  * ------------------------------------------------------------------------------------------- */
 int64_t fo_sparse_fa_split_workspace_bytes(void);
 int fo_sparse_fa_run(const void* q, const void* k, const void* v, void* o, float* lse, int dtype,
-                     const float* q_scale, const float* k_scale, int64_t q_stride_n,
+                     const void* q_lo, const float* q_scale, const float* k_scale, int64_t q_stride_n,
                      int64_t q_stride_h, int64_t k_stride_n, int64_t k_stride_h,
                      int64_t v_stride_n, int64_t v_stride_h, int64_t o_stride_n,
                      int64_t o_stride_h, const int32_t* qo_indptr, const int32_t* kv_indptr,
@@ -236,11 +239,12 @@ int fo_gemm_o(const void* x, const void* w, const void* bias, void* y, int dtype
  * feed the projection straight into fp8 attention.  As fo_gemm_q, plus: y8 [batch, m, n] e4m3fn
  * bytes and y_scale[num_qo_heads][batch * ceil(m / 128)] fp32, written for the computed tiles only:
  * scale = absmax of the (128-token block, head) slab of the fp32 result (bias included) / 448 (1 for
- * an all-zero slab), y8 = rne(result / scale).  y may be NULL (the 16-bit result is then not
- * written).  Needs n / num_qo_heads == 128.
+ * an all-zero slab), y8 = rne(result / scale).  y8_lo (optional, else NULL) [batch, m, n]: the
+ * residual rne(result / scale - y8), the second term of a two-term fp8 operand.  y may be NULL (the
+ * 16-bit result is then not written).  Needs n / num_qo_heads == 128.
  * ------------------------------------------------------------------------------------------- */
 int fo_gemm_q_quant(const void* x, const void* w, const void* bias, void* y, uint8_t* y8,
-                    float* y_scale, int dtype, int32_t batch, int32_t m, int32_t n, int32_t k,
+                    uint8_t* y8_lo, float* y_scale, int dtype, int32_t batch, int32_t m, int32_t n, int32_t k,
                     int32_t sparse_q_size, int32_t num_qo_heads, const uint8_t* sparse_info,
                     const int32_t* sparse_info_indptr, int32_t num_text_tokens, int is_full,
                     void* workspace, int64_t workspace_bytes, void* stream);
@@ -250,10 +254,11 @@ int fo_gemm_q_quant(const void* x, const void* w, const void* bias, void* y, uin
  * No counterpart in the reference (its quantization.cuh only packs bits).
  * x [nnz,H,D] bf16/f16 (strides in elements), x8 [nnz,H,D] bytes contiguous,
  * scale fp32 [H][n_blk]: scale = absmax/448 (1 for an all-zero block), x8 = rne(x/scale).
+ * x8_lo (optional, else NULL), laid out like x8: the residual rne(x/scale - x8).
  * blk_req/blk_tok0/blk_len (int32 [n_blk], device): request, first token and length of each block.
  * ------------------------------------------------------------------------------------------- */
 int fo_quant_fp8_block(const void* x, int dtype, int64_t x_stride_n, int64_t x_stride_h,
-                       uint8_t* x8, float* scale, const int32_t* blk_tok0, const int32_t* blk_len,
+                       uint8_t* x8, uint8_t* x8_lo, float* scale, const int32_t* blk_tok0, const int32_t* blk_len,
                        int32_t n_blk, int32_t num_heads, int32_t head_dim, void* stream);
 
 /* ---------------------------------------------------------------------------------------------

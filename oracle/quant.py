@@ -4,14 +4,16 @@ There is NO counterpart in the reference (its quantization.cuh only packs bits, 
 prefill kernel up-casts fp8 storage to fp16: include/flashomni/attention/prefill.cuh:602-612).
 parity unpinned against the reference; the definition below is the closed form
 scale = absmax / 448 (448 = largest finite e4m3fn), x8 = round_to_nearest_even(x / scale),
-all-zero block -> scale 1."""
+all-zero block -> scale 1.  The optional residual term is the same rounding applied to what the
+first term left: x8_lo = round_to_nearest_even(x / scale - x8)."""
 import torch
 
 FP8_MAX = 448.0
 
 
-def quant_fp8_block(x, indptr, block=128):
-    """x [nnz,H,D] -> (x8 float8_e4m3fn [nnz,H,D], scale fp32 [H, total_blocks]).
+def quant_fp8_block(x, indptr, block=128, residual=False):
+    """x [nnz,H,D] -> (x8 float8_e4m3fn [nnz,H,D], scale fp32 [H, total_blocks]) and, with
+    residual=True, x8_lo = e4m3(x / scale - x8) as a third result.
     Blocks never straddle requests: request r owns ceil(len_r/block) consecutive blocks."""
     nnz, H, D = x.shape
     spans = []
@@ -23,13 +25,16 @@ def quant_fp8_block(x, indptr, block=128):
             t += block
     scale = torch.ones(H, len(spans), dtype=torch.float32)
     x8 = torch.empty(nnz, H, D, dtype=torch.float8_e4m3fn)
+    x8_lo = torch.empty(nnz, H, D, dtype=torch.float8_e4m3fn)
     for j, (a, b) in enumerate(spans):
         blk = x[a:b].float()
         amax = blk.abs().amax(dim=(0, 2))
         s = torch.where(amax > 0, amax / FP8_MAX, torch.ones_like(amax))
         scale[:, j] = s
-        x8[a:b] = (blk / s[None, :, None]).clamp(-FP8_MAX, FP8_MAX).to(torch.float8_e4m3fn)
-    return x8, scale
+        scaled = (blk / s[None, :, None]).clamp(-FP8_MAX, FP8_MAX)
+        x8[a:b] = scaled.to(torch.float8_e4m3fn)
+        x8_lo[a:b] = (scaled - x8[a:b].float()).to(torch.float8_e4m3fn)
+    return (x8, scale, x8_lo) if residual else (x8, scale)
 
 
 def dequant_fp8_block(x8, scale, indptr, block=128):

@@ -205,8 +205,13 @@ def test_undersized_tensors_raise(dev):
 FP8_REL_L2 = 3e-2
 
 
+@pytest.mark.parametrize("two_term", [True, False])
 @pytest.mark.parametrize("case", [([512], [512], 2), ([300, 1, 128, 1000, 129], [77, 513, 128, 1100, 64], 3)])
-def test_fp8_attention(dev, case):
+def test_fp8_attention(dev, case, two_term):
+    """fp8 q and k with per-(head, block) scales.  Against the oracle fed the same quantised operands the
+    kernel has to be as exact as the 16-bit one.  Against the unquantised fp32 oracle the stated 3e-2
+    holds for the two-term q (q + q_lo: only k's rounding is left in the logits); a one-term q is a
+    faster form outside that contract (two e4m3 roundings per product: ~3.9e-2 on unit-variance data)."""
     import flashomni_amd as fo
     ql, kl, heads = case
     m = make_ragged_masks(ql, kl, heads, 0.75, 0.5, seed=21)
@@ -216,7 +221,9 @@ def test_fp8_attention(dev, case):
     k = torch.randn(nk, heads, 128, generator=g).to(torch.bfloat16)
     v = torch.randn(nk, heads, 128, generator=g).to(torch.bfloat16)
     t = lambda a: torch.from_numpy(a).to(dev)
-    q8, qs = fo.quant_fp8_block(q.to(dev), torch.from_numpy(m["qo_indptr"]))
+    q8, qs, q_lo = fo.quant_fp8_block(q.to(dev), torch.from_numpy(m["qo_indptr"]), residual=True)
+    if not two_term:
+        q_lo = None
     k8, ks = fo.quant_fp8_block(k.to(dev), torch.from_numpy(m["kv_indptr"]))
     w = fo.BatchFlashOmniFAWithRaggedKVWrapper(torch.empty(128 << 20, dtype=torch.uint8, device=dev))
     w.plan(t(m["qo_indptr"]), t(m["kv_indptr"]), heads, heads, 128, q_data_type=torch.float8_e4m3fn)
@@ -224,21 +231,70 @@ def test_fp8_attention(dev, case):
     out = out0.clone().to(dev)
     lse = torch.full((nq, heads), float("nan"), device=dev)
     w.run(q8, k8, v.to(dev), t(m["packed_info"]), t(m["packed_keep"]), t(m["info_indptr"]),
-          t(m["keep_indptr"]), out=out, lse=lse, return_lse=True, q_scale=qs, k_scale=ks)
+          t(m["keep_indptr"]), out=out, lse=lse, return_lse=True, q_scale=qs, k_scale=ks, q_lo=q_lo)
     exp_lse = torch.full((nq, heads), float("nan"))
     exp = oracle.sparse_attention(q8.cpu(), k8.cpu(), v, m["packed_info"], m["packed_keep"], m["info_indptr"],
                                   m["keep_indptr"], m["qo_indptr"], m["kv_indptr"], out=out0.clone(),
-                                  lse=exp_lse, q_scale=qs.cpu(), k_scale=ks.cpu())
+                                  lse=exp_lse, q_scale=qs.cpu(), k_scale=ks.cpu(),
+                                  q_lo=None if q_lo is None else q_lo.cpu())
     out = out.cpu()
     changed = _touched(m, heads, out.shape)
     assert torch.equal(out[~changed].view(torch.int16), out0[~changed].view(torch.int16))
-    assert rel_l2(out[changed], exp[changed]) <= FP8_REL_L2
+    assert rel_l2(out[changed], exp[changed]) <= REL_L2
     assert max_abs(out[changed], exp[changed]) <= MAX_ABS
     ok = ~torch.isnan(exp_lse)
     assert float((lse.cpu()[ok] - exp_lse[ok]).abs().max()) < 2e-2
     ref = oracle.sparse_attention(q, k, v, m["packed_info"], m["packed_keep"], m["info_indptr"],
                                   m["keep_indptr"], m["qo_indptr"], m["kv_indptr"], out=out0.clone())
-    assert rel_l2(out[changed], ref[changed]) < 6e-2
+    err = rel_l2(out[changed], ref[changed])
+    print("fp8 attention vs the unquantised oracle, %s-term q: rel-L2 %.4g" % ("two" if two_term else "one", err))
+    if two_term:
+        assert err <= FP8_REL_L2   # the stated fp8 tolerance
+    else:
+        assert err <= 4.5e-2       # not the contract: the level two e4m3 operands explain
+
+
+@pytest.mark.parametrize("config", [4])
+def test_fp8_attention_video_shape_sampled_rows(dev, config):
+    """fp8 attention (two-term q) at config 4's full size on unit-variance q, k, v: sampled rows within the
+    stated relative L2 3e-2 of the unquantised fp32 oracle."""
+    import flashomni_amd as fo
+    from flashomni_amd.workloads import make_workload
+    wl = make_workload(config, tensors=False)
+    s = wl.shape
+    g = torch.Generator(device=dev).manual_seed(300 + config)
+    draw = lambda: torch.randn(s.seq, s.heads, 128, generator=g, device=dev, dtype=torch.float32).to(torch.bfloat16)
+    q, k, v = draw(), draw(), draw()
+    q8, qs, q_lo = fo.quant_fp8_block(q, wl.qo_indptr, residual=True)
+    k8, ks = fo.quant_fp8_block(k, wl.kv_indptr)
+    out = torch.full((s.seq, s.heads, 128), -7.0, dtype=torch.bfloat16, device=dev)
+    w = fo.BatchFlashOmniFAWithRaggedKVWrapper(torch.empty(256 << 20, dtype=torch.uint8, device=dev))
+    w.plan(wl.qo_indptr, wl.kv_indptr, s.heads, s.heads, 128, q_data_type=torch.float8_e4m3fn)
+    w.run(q8, k8, v, wl.packed_info.to(dev), wl.packed_kv_info.to(dev), wl.info_indptr.to(dev),
+          wl.kv_info_indptr.to(dev), out=out, q_scale=qs, k_scale=ks, q_lo=q_lo)
+    torch.cuda.synchronize()
+    active = wl.sparse_info.to(dev).repeat_interleave(128, dim=0)[:s.seq]
+    assert bool((out[~active] == -7.0).all())
+    _, row_qb, row_head, ptr, _ = oracle.decode_kv_csr(
+        wl.packed_info.numpy(), wl.packed_kv_info.numpy(), wl.info_indptr.numpy(),
+        wl.kv_info_indptr.numpy(), wl.qo_indptr.numpy(), wl.kv_indptr.numpy(), s.heads, 128, 128)
+    edge = np.nonzero((row_qb == 0) | (row_qb == s.n_blocks - 1))[0]
+    rng = np.random.default_rng(config)
+    rows = np.unique(np.concatenate([edge, rng.choice(len(row_qb), 64, replace=False)]))
+    exp = torch.full((s.seq, s.heads, 128), -7.0, dtype=torch.bfloat16)
+    oracle.sparse_attention(q.cpu(), k.cpu(), v.cpu(), wl.packed_info, wl.packed_kv_info,
+                            wl.info_indptr, wl.kv_info_indptr, wl.qo_indptr, wl.kv_indptr,
+                            out=exp, rows=[int(i) for i in rows])
+    got = out.cpu()
+    num, den = 0.0, 0.0
+    for i in rows:
+        q0 = int(row_qb[i]) * 128
+        sl = (slice(q0, min(s.seq, q0 + 128)), int(row_head[i]))
+        a, b = got[sl].float(), exp[sl].float()
+        num += float(((a - b) ** 2).sum())
+        den += float((b ** 2).sum())
+    print("fp8 attention at config %d, two-term q: rel-L2 %.4g" % (config, math.sqrt(num / den)))
+    assert math.sqrt(num / den) <= FP8_REL_L2
 
 
 def test_fp8_attention_needs_scales(dev):

@@ -263,6 +263,25 @@ def test_gemm_q_with_fused_fp8_quantisation(dev, shape, write_out):
                 bound = 0.0625 * y.abs() + s * 2.0 ** -9 + 2e-3 * amax
                 assert bool(((deq - y).abs() <= bound).all())
                 assert float(deq_all[bi, rows, cols].abs().max()) == 448.0 or amax == 0.0
+    # the residual term: same first term and scales, second term = e4m3(result / scale - first term)
+    lo = torch.full((batch, m, n), 0x5A, dtype=torch.uint8, device=dev).view(torch.float8_e4m3fn)
+    q8b = q8_0.clone().to(dev).view(torch.float8_e4m3fn)
+    res3 = fo.flashomni_gemm(*args, out=False, quant_out=(q8b, sc_0.clone().to(dev), lo))
+    assert len(res3) == 4 and res3[3].data_ptr() == lo.data_ptr()
+    assert torch.equal(q8b.cpu().view(torch.uint8), q8c.view(torch.uint8))
+    two = deq_all + lo.cpu().float()
+    for bi in range(batch):
+        for iy in range(nqb):
+            rows = slice(iy * 128, min(m, (iy + 1) * 128))
+            for h in range(heads):
+                cols = slice(h * 128, (h + 1) * 128)
+                if not info[bi, iy, h]:
+                    assert torch.equal(lo.cpu().view(torch.uint8)[bi, rows, cols], q8_0[bi, rows, cols])
+                    continue
+                y = ref[bi, rows, cols].float()
+                s = float(scc[h, bi * nqb + iy])
+                bound = 2.0 ** -8 * y.abs() + s * 2.0 ** -9 + 2e-3 * float(y.abs().max()) * 2.0 ** -4
+                assert bool(((two[bi, rows, cols] * s - y).abs() <= bound).all())
     # the pair is what fp8 attention takes: against the separate quantiser on the 16-bit result
     if write_out and batch == 1 and p_active == 1.0:
         ws = torch.empty(64 << 20, dtype=torch.uint8, device=dev)

@@ -28,3 +28,26 @@ def test_quant_fp8_block_bit_exact(dev, dtype, lens):
     err = (deq - x.float()).abs()
     bound = x.float().abs() * 2 ** -4 + scale.cpu().max() * 2 ** -9
     assert bool((err <= bound).all())
+
+
+@pytest.mark.parametrize("lens", [[256], [300, 1, 128]])
+def test_quant_fp8_block_residual(dev, lens):
+    """The second term is the same rounding applied to what the first left: bit-exact against the
+    oracle, and the two terms together carry x to 2^-8 relative (two 3-bit-mantissa roundings)."""
+    import flashomni_amd as fo
+    heads = 2
+    g = torch.Generator().manual_seed(7 + sum(lens))
+    indptr = torch.tensor([0] + list(torch.tensor(lens).cumsum(0)), dtype=torch.int32)
+    x = (torch.randn(int(indptr[-1]), heads, 128, generator=g) * 2).to(torch.bfloat16)
+    x8, scale, lo = fo.quant_fp8_block(x.to(dev), indptr, residual=True)
+    e8, es, elo = oracle.quant_fp8_block(x, indptr, residual=True)
+    assert torch.equal(scale.cpu(), es)
+    assert torch.equal(x8.cpu().view(torch.uint8), e8.view(torch.uint8))
+    assert torch.equal(lo.cpu().view(torch.uint8), elo.view(torch.uint8))
+    one = oracle.dequant_fp8_block(x8.cpu(), scale.cpu(), indptr)
+    two = one + oracle.dequant_fp8_block(lo.cpu(), scale.cpu(), indptr)
+    floor = scale.cpu().max() * 2 ** -10
+    assert bool(((two - x.float()).abs() <= x.float().abs() * 2 ** -8 + floor).all())
+    assert float((two - x.float()).norm()) < 0.1 * float((one - x.float()).norm())
+    # without residual=True the result is the two-tuple it always was
+    assert len(fo.quant_fp8_block(x.to(dev), indptr)) == 2
