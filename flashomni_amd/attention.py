@@ -365,10 +365,19 @@ class BatchFlashOmniFAWithRaggedKVWrapper:
         rope_theta: Optional[float] = None,
         q_data_type: Union[str, torch.dtype] = "float16",
         kv_data_type: Optional[Union[str, torch.dtype]] = None,
+        *,
+        gqa_symbols: Optional[str] = None,
     ) -> None:
         r"""Plan sparse prefill attention for the given ragged batch.
 
-        Same parameters as the reference ``plan``.  The host planner tiles the batch into the
+        Same parameters as the reference ``plan``, plus ``gqa_symbols`` (keyword-only).  With
+        ``num_kv_heads < num_qo_heads`` the reference packs the q heads of a kv head into the row
+        dimension and reads one symbol per (128 packed rows = 128 / group tokens x group heads,
+        kv head) (include/flashomni/attention/prefill.cuh:1283-1290).  That tiling is not built
+        here; grouped-query attention is available with symbols per (128-token block, q head),
+        ``bit = q_block * num_qo_heads + q_head``, and has to be asked for by name,
+        ``gqa_symbols="per_q_head"``, so that symbols laid out for the reference are never
+        misread.  The host planner tiles the batch into the
         integer workspace; in addition the q-block table of the symbol decoder is built and the
         work-list buffers are sized for the worst case (every bit set).  Cannot be captured in a
         graph (it copies the indptrs to the host)."""
@@ -396,6 +405,13 @@ class BatchFlashOmniFAWithRaggedKVWrapper:
                 "prefill path")
         if num_kv_heads <= 0 or num_qo_heads % num_kv_heads != 0:
             raise ValueError("num_qo_heads must be a multiple of num_kv_heads")
+        if gqa_symbols not in (None, "per_q_head"):
+            raise ValueError("gqa_symbols must be None or 'per_q_head'")
+        if num_kv_heads != num_qo_heads and gqa_symbols != "per_q_head":
+            raise NotImplementedError(
+                "grouped-query attention with the reference's symbol layout (one symbol per 128 packed "
+                "rows and kv head) is not built; pass gqa_symbols='per_q_head' to use symbols per "
+                "(128-token block, q head)")
         if head_dim_qk != 128 or head_dim_vo != 128:
             raise NotImplementedError("only head_dim 128 is supported")
         if sparse_block_size_for_q != 128 or sparse_block_size_for_kv != 128:

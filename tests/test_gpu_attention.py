@@ -432,7 +432,13 @@ def test_grouped_query_attention(dev, heads, layout):
     v = torch.randn(nk, hkv, 128, generator=g).to(torch.bfloat16)
     t = lambda a: torch.from_numpy(a).to(dev)
     w = fo.BatchFlashOmniFAWithRaggedKVWrapper(torch.empty(256 << 20, dtype=torch.uint8, device=dev), layout)
-    w.plan(t(m["qo_indptr"]), t(m["kv_indptr"]), hq, hkv, 128, q_data_type=torch.bfloat16)
+    if hq != hkv:
+        # the reference's layout for group > 1 (one symbol per 128 packed rows and kv head,
+        # prefill.cuh:1283-1290) is not built: it has to be declined, not misread
+        with pytest.raises(NotImplementedError, match="per_q_head"):
+            w.plan(t(m["qo_indptr"]), t(m["kv_indptr"]), hq, hkv, 128, q_data_type=torch.bfloat16)
+    w.plan(t(m["qo_indptr"]), t(m["kv_indptr"]), hq, hkv, 128, q_data_type=torch.bfloat16,
+           gqa_symbols="per_q_head")
     kd, vd = k.to(dev), v.to(dev)
     if layout == "HND":
         kd, vd = kd.transpose(0, 1).contiguous(), vd.transpose(0, 1).contiguous()
