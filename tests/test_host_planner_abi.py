@@ -167,7 +167,7 @@ def test_argument_checks_without_gpu():
     assert L.fo_packbits(None, 8, 7, None, None) == -1 and b"bitorder" in L.fo_last_error()
     assert L.fo_gemm_q(1, 1, None, 1, 0, 1, 128, 100, 64, 128, 1, None, None, 0, 1, None, 0, None) == -1
     assert b"only support" in L.fo_last_error()
-    assert L.fo_sparse_fa_run(*([None] * 5), 0, None, None, *([0] * 8), *([None] * 4), 0, 0, *([None] * 7), 4, 2, 2, 64, 128, 128,
+    assert L.fo_sparse_fa_run(*([None] * 5), 0, None, None, None, *([0] * 8), *([None] * 4), 0, 0, *([None] * 7), 4, 2, 2, 64, 128, 128,
                               1.0, None, None, 0, None) == -1
     assert b"head_dim" in L.fo_last_error()
 
