@@ -20,11 +20,17 @@
 // from the shape.  GEMM-O walks the union of the two token blocks' selected heads; a token block
 // that does not select a head gets that k step's X operand zeroed.
 //
-// Data path.  BK = 32.  Operand tiles go global -> LDS directly (global_load_lds_dwordx4) into a
-// 4-stage ring, three k steps ahead of the math, one barrier per k step.  A wavefront's copy lands
-// on 1 KB of consecutive LDS (16 rows of 64 B), so rows are XOR-swizzled instead of padded: row r
-// keeps logical 16-byte chunk c at position c ^ ((r >> 2) & 3), applied on the global side; the
-// 128-bit operand reads of 16 consecutive rows then cover all 64 banks.
+// Data path.  Operands are staged in slabs of 64 k: a tile row is then 128 B, one whole memory line
+// (with 32-wide slabs every line crossed the L2 -> CU path twice, half of it unused each time, and
+// that path, not the matrix cores, bounded the loop).  Operand tiles go global -> LDS directly
+// (global_load_lds_dwordx4, 8 rows x 128 B per instruction) into two slab buffers: slab i is read
+// while slab i+1 lands; one barrier per slab, placed before the slab's last quarter so that the
+// copies of slab i+2 and the first operand reads of slab i+1 run in the shadow of the last MFMAs.  A
+// wavefront's copy lands on 1 KB of consecutive LDS, so rows are XOR-swizzled instead of padded: row
+// r keeps logical 16-byte chunk c at position c ^ ((r >> 1) & 7), applied on the global side; the
+// 128-bit operand reads of 16 consecutive rows then cover all 64 banks.  A k range that is not a
+// multiple of 64 (K or the head width of GEMM-O = 32 mod 64) ends in a slab that reaches 32 back into
+// its neighbour; that half of its X operand is zeroed.
 //
 // The product is formed transposed (A operand = W rows, B operand = X rows): in the 32 x 32
 // accumulator layout a lane owns one output row and runs of 4 consecutive columns.  Stored (or the
@@ -56,13 +62,14 @@ typedef __attribute__((address_space(1))) const void glb_void;
 
 constexpr int kThreads = 512;
 constexpr int kTile = 128;  // unit edge = granularity of the skip flags
-constexpr int kBK = 32;
-constexpr int kRowBytes = kBK * 2;                 // one LDS row: 32 elements, 4 chunks of 16 B
-constexpr int kUnitBytes = kTile * kRowBytes;      // one 128-row operand tile: 8 KB
+constexpr int kBK = 64;                            // k range of one LDS slab
+constexpr int kRowBytes = kBK * 2;                 // one LDS row: 64 elements = one 128-byte memory line, 8 chunks of 16 B
+constexpr int kUnitBytes = kTile * kRowBytes;      // one 128-row operand tile: 16 KB
 constexpr int kStageBytes = 4 * kUnitBytes;        // X0, X1, W0, W1
-constexpr int kStages = 4;
+constexpr int kStages = 2;
 constexpr int kSmemBytes = kStages * kStageBytes;  // 128 KB
-constexpr int kCopiesPerWave = kStageBytes / 1024 / 8;  // 4 copy instructions per wavefront per stage
+constexpr int kCopiesPerWave = kStageBytes / 1024 / 8;  // 8 copy instructions per wavefront per slab
+constexpr int kZeroFirst = 1 << 18, kZeroSecond = 1 << 19;  // slab entry: half of the slab does not count
 constexpr int kMaxHeads = 256;
 constexpr int kMaxSteps = 2048;  // GEMM-O: k steps of one work item (K <= 65536)
 constexpr int kXcds = 8;
@@ -317,10 +324,14 @@ __global__ void __launch_bounds__(kThreads) gemm_kernel(const GemmParams p) {
   // rows 16*wv.. of each of the four tiles (0,1 = X of token block 0,1; 2,3 = W of column block
   // 0,1).  Lane i lands on row 16*wv + i/4 at chunk position i%4 and must fetch logical chunk
   // (i%4) ^ ((row >> 2) & 3) = (i%4) ^ ((i >> 4) & 3).
-  const int cp_row = 16 * wv + (lane >> 2);
-  const int cp_chunk = ((lane & 3) ^ ((lane >> 4) & 3)) * 8;  // element offset inside the k step
-  // operand reads: row = tile row base + l32 (bases are multiples of 32), logical chunk 2*ks + g
-  const int rd_swz = (l32 >> 2) & 3;
+  // (slab layout: a copy instruction covers 8 rows x 128 B, i.e. whole memory lines; wavefront wv issues
+  // rows 16*wv + 8*n.. (n = 0, 1) of each of the four tiles.  Lane i lands on row 16*wv + 8*n + i/8 at
+  // chunk position i%8 and must fetch logical chunk (i%8) ^ ((row >> 1) & 7) = (i%8) ^ ((4*n + (i >> 4)) & 7).)
+  const int cp_row = 16 * wv + (lane >> 3);
+  const int cp_chunk0 = ((lane & 7) ^ ((lane >> 4) & 7)) * 8;        // element offset inside the slab, n = 0
+  const int cp_chunk1 = ((lane & 7) ^ ((4 + (lane >> 4)) & 7)) * 8;  // n = 1
+  // operand reads: row = tile row base + l32 (bases are multiples of 32), logical chunk 2*s + g of substep s
+  const int rd_swz = (l32 >> 1) & 7;
 
   const int xcd = blockIdx.x & (kXcds - 1), slot = blockIdx.x >> 3;
   const int per_xcd = gridDim.x >> 3;  // host launches a multiple of 8 workgroups
@@ -477,46 +488,59 @@ __global__ void __launch_bounds__(kThreads) gemm_kernel(const GemmParams p) {
         if (lane == 0) s_nsel = count;
       }
       __syncthreads();
-      const int iph = p.head_dim / kBK;
+      // slabs of a head slice: full 64-wide ones, then (head_dim % 64 == 32) one that reaches 32 back
+      // into the slab before it and counts for its second half only (the first slice of the matrix
+      // instead reaches forward and counts for its first half)
+      const int iph = (p.head_dim + kBK - 1) / kBK;
       n_iter = s_nsel * iph;
       if (n_iter > 0) {
         for (int i = tid; i < n_iter + 4; i += kThreads) {
           const int ii = i < n_iter ? i : n_iter - 1;
           const int hv = s_heads[ii / iph];
-          s_step[i] = ((hv & 0xFFFF) * p.head_dim + (ii % iph) * kBK) | (hv & 0x30000);
+          const int k0 = (hv & 0xFFFF) * p.head_dim + (ii % iph) * kBK;
+          int e = k0;
+          if ((ii % iph) * kBK + kBK > p.head_dim) e = k0 >= 32 ? (k0 - 32) | kZeroFirst : k0 | kZeroSecond;
+          s_step[i] = e | (hv & 0x30000);
         }
       }
       __syncthreads();
     } else {
-      n_iter = p.k / kBK;
+      n_iter = (p.k + kBK - 1) / kBK;
     }
 
     // ---- global row pointers of the four operand tiles: X(r0), X(r1), W(c0), W(c1) ----
     // this wavefront copies rows 16*wv.. of each; rows past M are clamped (their results are dropped)
-    const T* cp_src[4];
+    const T* cp_src[4][2];  // [tile][n]
     {
       const T* xb = xg + static_cast<int64_t>(bz) * p.m * p.k;
 #pragma unroll
-      for (int u = 0; u < 2; ++u) {
-        int xr = r[u] * kTile + cp_row;
-        xr = xr < p.m ? xr : p.m - 1;
-        cp_src[u] = xb + static_cast<int64_t>(xr) * p.k + cp_chunk;
-        cp_src[2 + u] = wg + static_cast<int64_t>(c[u] * kTile + cp_row) * p.k + cp_chunk;
-      }
+      for (int u = 0; u < 2; ++u)
+#pragma unroll
+        for (int n = 0; n < 2; ++n) {
+          int xr = r[u] * kTile + cp_row + 8 * n;
+          xr = xr < p.m ? xr : p.m - 1;
+          const int chunk = n ? cp_chunk1 : cp_chunk0;
+          cp_src[u][n] = xb + static_cast<int64_t>(xr) * p.k + chunk;
+          cp_src[2 + u][n] = wg + static_cast<int64_t>(c[u] * kTile + cp_row + 8 * n) * p.k + chunk;
+        }
     }
     // k offset of step it (steps past the end repeat the last one); GEMM-O: plus the select bits
     auto step_entry = [&](int it) -> int {
       if constexpr (kReduce) {
         return s_step[it];
       } else {
-        return (it < n_iter ? it : n_iter - 1) * kBK;
+        // (K % 64 == 32: the last slab reaches 32 back and counts for its second half only)
+        const int i = it < n_iter ? it : n_iter - 1;
+        return (i + 1) * kBK <= p.k ? i * kBK | 0x30000 : (p.k - kBK) | kZeroFirst | 0x30000;
       }
     };
     // copies past the last k step (kept so that every step issues the same instructions) land in a
     // scrap kilobyte, so the ring is free for the epilogue as soon as the last reads are done
-    auto copy_one = [&](int it, int entry, int j) {
-      uint8_t* dst = it < n_iter ? smem + (it % kStages) * kStageBytes + wv * 1024 + j * kUnitBytes : s_scrap;
-      copy16_to_lds(cp_src[j] + (entry & 0xFFFF), dst);
+    auto copy_one = [&](int it, int entry, int idx) {  // idx = 2 * tile + n
+      uint8_t* dst = it < n_iter ? smem + (it % kStages) * kStageBytes + (idx >> 1) * kUnitBytes + wv * 2048 +
+                                       (idx & 1) * 1024
+                                 : s_scrap;
+      copy16_to_lds(cp_src[idx >> 1][idx & 1] + (entry & 0xFFFF), dst);
     };
     auto copy_stage = [&](int it) {
       const int entry = step_entry(it);
@@ -530,14 +554,14 @@ __global__ void __launch_bounds__(kThreads) gemm_kernel(const GemmParams p) {
       // leaving its SIMD's matrix core to the other wavefront.
       __builtin_amdgcn_s_waitcnt(0x0f70);
       if (n_iter > 0) {
-#pragma unroll
-        for (int s = 0; s < kStages - 1; ++s) copy_stage(s);
-        __builtin_amdgcn_s_waitcnt(0x0f70 | (2 * kCopiesPerWave));
+        copy_stage(0);
+        copy_stage(1);
+        __builtin_amdgcn_s_waitcnt(0x0f70 | kCopiesPerWave);
         __builtin_amdgcn_s_barrier();
         for (int it = 0; it < n_iter; ++it) {
-          __builtin_amdgcn_s_waitcnt(0x0f70 | kCopiesPerWave);
+          __builtin_amdgcn_s_waitcnt(0x0f70);
           __builtin_amdgcn_s_barrier();
-          copy_stage(it + 3);
+          copy_stage(it + 2);
         }
         __builtin_amdgcn_s_barrier();  // the others' "ring is free" barrier before their epilogue
       }
@@ -556,9 +580,10 @@ __global__ void __launch_bounds__(kThreads) gemm_kernel(const GemmParams p) {
     // the previous work item's stores are complete: from here on vmcnt counts loads only
     __builtin_amdgcn_s_waitcnt(0x0f70);
     __builtin_amdgcn_sched_barrier(0);
-#pragma unroll
-    for (int s = 0; s < kStages - 1; ++s)
-      if (n_iter > 0) copy_stage(s);
+    if (n_iter > 0) {
+      copy_stage(0);
+      copy_stage(1);
+    }
     __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
     for (int nt = 0; nt < NT; ++nt)
@@ -572,29 +597,30 @@ __global__ void __launch_bounds__(kThreads) gemm_kernel(const GemmParams p) {
     const int b_base = wr * kUnitBytes + (wh * 64 + l32) * kRowBytes;  // X rows wh*64 + mt*32 + l32
 
     // ---- main loop ----
-    // Copies run up to three k steps ahead.  Operand reads run half a k step ahead of the MFMAs
-    // that use them (two register sets), so a wavefront's LDS reads overlap its own math:
-    //   MFMAs(it, first half) with reads(it, second half) in their shadow | tile it+1 landed, barrier,
-    //   copy(it+3) | MFMAs(it, second half) with reads(it+1, first half) in their shadow
+    // One slab = 64 k = four substeps of eight MFMAs.  Two slabs in LDS: slab it is read while slab
+    // it+1 lands.  Operand reads run one substep ahead of the MFMAs that use them (two register
+    // sets).  One barrier per slab, before its last substep: by then slab it+1 has landed for every
+    // wavefront and every wavefront has its last operands of slab it in registers, so the copies of
+    // slab it+2 may overwrite it; they and the first reads of slab it+1 go into the shadow of the last
+    // substep's MFMAs.
     x8 a[2][NT], b[2][MT];
-    // one operand read of half-step (it, ks): j = 0..3 W rows, j = 4..5 X rows
-    // one operand read of half-step (it, ks): j = 0..3 W rows, j = 4..5 X rows
-    auto read_one = [&](int it, int ks, int j) {
+    // one operand read of substep sub of slab it into register set sub & 1: j = 0..3 W rows, j = 4..5 X rows
+    auto read_one = [&](int it, int sub, int j) {
       const uint8_t* st = smem + (it % kStages) * kStageBytes;
-      const int sw = ((2 * ks + g) ^ rd_swz) << 4;
+      const int sw = ((2 * sub + g) ^ rd_swz) << 4;
       if (j < NT) {
-        a[ks][j] = *reinterpret_cast<const x8*>(st + a_base + j * 32 * kRowBytes + sw);
+        a[sub & 1][j] = *reinterpret_cast<const x8*>(st + a_base + j * 32 * kRowBytes + sw);
       } else {
-        b[ks][j - NT] = *reinterpret_cast<const x8*>(st + b_base + (j - NT) * 32 * kRowBytes + sw);
+        b[sub & 1][j - NT] = *reinterpret_cast<const x8*>(st + b_base + (j - NT) * 32 * kRowBytes + sw);
       }
     };
-    // the eight MFMAs of half-step ks; in their shadow the six operand reads of half-step (rit, rks)
-    // and, if cit >= 0, this wavefront's four copies of tile cit.  GEMM-O: a token block that does
-    // not select this step's head contributes nothing: its X operand is zeroed (keep = 0).  (Skipping
-    // the MFMAs instead puts them under a branch, and the register allocator then copies and spills
-    // accumulators in the loop.)
-    auto math_and_read = [&](int ks, unsigned keep, int rit, int rks, int cit, int centry) {
-      if constexpr (kReduce) {
+    // the eight MFMAs of register set ks; in their shadow the six operand reads of substep rsub of slab
+    // rit and, if cit >= 0, this wavefront's eight copies of slab cit.  An X operand that does not count
+    // (GEMM-O: the token block does not select this slab's head; the half of a slab that reaches into
+    // its neighbour) is zeroed (keep = 0).  (Skipping the MFMAs instead puts them under a branch, and
+    // the register allocator then copies and spills accumulators in the loop.)
+    auto math_and_read = [&](int ks, unsigned keep, bool masked, int rit, int rsub, int cit, int centry) {
+      if (masked) {
 #pragma unroll
         for (int mt = 0; mt < MT; ++mt) {
           u32x4 v = __builtin_bit_cast(u32x4, b[ks][mt]);
@@ -607,32 +633,42 @@ __global__ void __launch_bounds__(kThreads) gemm_kernel(const GemmParams p) {
         const int nt = i / MT, mt = i % MT;
         acc[nt][mt] = TT::mfma(a[ks][nt], b[ks][mt], acc[nt][mt]);
         if (cit >= 0 && i < kCopiesPerWave) copy_one(cit, centry, i);
-        if (i < NT + MT) read_one(rit, rks, i);
+        if (i < NT + MT) read_one(rit, rsub, i);
         __builtin_amdgcn_sched_barrier(0);
       }
     };
-    auto keep_of = [&](int entry) -> unsigned {
-      return kReduce ? (((entry >> (16 + wr)) & 1) ? 0xFFFFFFFFu : 0u) : 0xFFFFFFFFu;
+    // keep masks of a slab's first and second half for this wavefront's token block
+    auto keep_of = [&](int entry, int half) -> unsigned {
+      const bool sel = (entry >> (16 + wr)) & 1;
+      const bool zero = entry & (half ? kZeroSecond : kZeroFirst);
+      return sel && !zero ? 0xFFFFFFFFu : 0u;
     };
-    // Copies past the last k step repeat the last one (into a stage nobody reads any more), so the
-    // loop body and its vmcnt arithmetic are the same for every step.
+    // Copies past the last slab repeat the last one (into a scrap kilobyte), so the loop body is the
+    // same for every slab.
     if (n_iter > 0) {
-      __builtin_amdgcn_s_waitcnt(0x0f70 | (2 * kCopiesPerWave));  // tile 0 landed, 1 and 2 in flight
+      __builtin_amdgcn_s_waitcnt(0x0f70 | kCopiesPerWave);  // slab 0 landed, slab 1 in flight
       __builtin_amdgcn_s_barrier();
 #pragma unroll
       for (int j = 0; j < NT + MT; ++j) read_one(0, 0, j);
-      unsigned keep = keep_of(step_entry(0));
-      for (int it = 0; it < n_iter; ++it) {
-        // table entries of the tile to copy and of the next tile, read ahead of their use
-        const int centry = step_entry(it + 3);
-        const unsigned keep_next = keep_of(step_entry(it + 1));
-        math_and_read(0, keep, it, 1, -1, 0);
-        __builtin_amdgcn_s_waitcnt(0x0f70 | kCopiesPerWave);  // tile it+1 landed (it+2 may be in flight)
-        __builtin_amdgcn_s_barrier();  // ... for every wavefront; nobody reads stage (it-1)%4 any more
-        // copies of tile it+3 and reads of tile it+1 in the shadow of the second half's MFMAs
-        // (the reads of the last step fetch a stale stage; never used)
-        math_and_read(1, keep, it + 1, 0, it + 3, centry);
-        keep = keep_next;
+      int entry = step_entry(0);
+      auto slab = [&](int it, bool masked) {
+        const int centry = step_entry(it + 2);
+        const int entry_next = step_entry(it + 1);
+        const unsigned keep0 = keep_of(entry, 0), keep1 = keep_of(entry, 1);
+        math_and_read(0, keep0, masked, it, 1, -1, 0);
+        math_and_read(1, keep0, masked, it, 2, -1, 0);
+        math_and_read(0, keep1, masked, it, 3, -1, 0);
+        __builtin_amdgcn_s_waitcnt(0x0070);  // vmcnt(0), lgkmcnt(0): slab it+1 landed, last operands of slab it here
+        __builtin_amdgcn_s_barrier();        // ... for every wavefront
+        math_and_read(1, keep1, masked, it + 1, 0, it + 2, centry);
+        entry = entry_next;
+      };
+      if constexpr (kReduce) {
+        for (int it = 0; it < n_iter; ++it) slab(it, true);
+      } else {
+        // only the last slab can hold a half that does not count (K % 64 == 32)
+        for (int it = 0; it < n_iter - 1; ++it) slab(it, false);
+        slab(n_iter - 1, true);
       }
     }
 
@@ -881,6 +917,7 @@ int check_common(const void* x, const void* w, void* y, int dtype, int32_t batch
   FO_REQUIRE(batch > 0 && m > 0 && n > 0 && k > 0, "gemm: bad shape");
   FO_REQUIRE(n % 128 == 0 && k % 32 == 0, "only support N %% 128 == 0, K %% 32 == 0 (got N=%d K=%d)",
              n, k);
+  FO_REQUIRE(k >= kBK, "gemm: K = %d is below the 64 columns one operand slab holds", k);
   FO_REQUIRE(sparse_q_size > 0 && num_qo_heads > 0 && n % num_qo_heads == 0,
              "gemm: bad sparse_q_size / num_qo_heads");
   FO_REQUIRE(x && w && y, "gemm: null pointer");
@@ -979,7 +1016,7 @@ extern "C" int fo_gemm_o(const void* x, const void* w, const void* bias, void* y
   FO_REQUIRE(sparse_info && sparse_info_indptr, "gemm_reduction: sparse_info is required");
   FO_REQUIRE(num_text_tokens >= 0, "gemm: negative num_text_tokens");
   const int head_dim = n / num_qo_heads;
-  FO_REQUIRE(head_dim % kBK == 0 && k % head_dim == 0 && k / head_dim <= kMaxHeads && k / kBK <= kMaxSteps,
+  FO_REQUIRE(head_dim % 32 == 0 && k % head_dim == 0 && k / head_dim <= kMaxHeads && k / 32 <= kMaxSteps,
              "gemm_reduction: head slice width %d must be a multiple of 32 and divide K=%d <= 65536",
              head_dim, k);
   FO_REQUIRE(bias_kind == FO_BIAS_NONE || bias_kind == FO_BIAS_VECTOR || bias_kind == FO_BIAS_MATRIX,

@@ -75,6 +75,9 @@ def test_gemm_q_shape_errors(dev):
     x, w, b = _operands(1, 128, 192, 64, torch.bfloat16, seed=1)
     with pytest.raises(RuntimeError, match="only support"):
         fo.flashomni_gemm(x.to(dev), w.to(dev), 1, is_full=True)
+    x, w, b = _operands(1, 128, 128, 32, torch.bfloat16, seed=1)
+    with pytest.raises(RuntimeError, match="below the 64 columns"):
+        fo.flashomni_gemm(x.to(dev), w.to(dev), 1, is_full=True)
 
 
 def test_undersized_symbols_raise(dev):
@@ -99,7 +102,9 @@ def test_undersized_symbols_raise(dev):
 
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
 @pytest.mark.parametrize("use_bias", [False, True])
-@pytest.mark.parametrize("shape", [(1, 512, 384, 3, 0), (2, 256, 256, 2, 0), (1, 300, 512, 4, 0)])
+@pytest.mark.parametrize("shape", [(1, 512, 384, 3, 0), (2, 256, 256, 2, 0), (1, 300, 512, 4, 0),
+                                   # head widths that are not multiples of the 64-wide operand slabs: 96, 32, 160
+                                   (1, 384, 384, 4, 0), (1, 200, 128, 4, 0), (1, 256, 640, 4, 128)])
 def test_gemm_o_two_pass_protocol(dev, dtype, use_bias, shape):
     """cache pass, then final pass fed with the cached partial: each pass matches its oracle and the
     end result equals the dense linear layer (the identity the reference's own script checks,
