@@ -60,7 +60,7 @@ typedef __attribute__((ext_vector_type(4))) unsigned int u32x4;
 typedef __attribute__((address_space(3))) void lds_void;
 typedef __attribute__((address_space(1))) const void glb_void;
 
-constexpr int kThreads = 512;
+constexpr int kThreads = 256;
 constexpr int kTile = 128;  // unit edge = granularity of the skip flags
 constexpr int kBK = 64;                            // k range of one LDS slab
 constexpr int kRowBytes = kBK * 2;                 // one LDS row: 64 elements = one 128-byte memory line, 8 chunks of 16 B
@@ -68,13 +68,12 @@ constexpr int kUnitBytes = kTile * kRowBytes;      // one 128-row operand tile: 
 constexpr int kStageBytes = 4 * kUnitBytes;        // X0, X1, W0, W1
 constexpr int kStages = 2;
 constexpr int kSmemBytes = kStages * kStageBytes;  // 128 KB
-constexpr int kCopiesPerWave = kStageBytes / 1024 / 8;  // 8 copy instructions per wavefront per slab
 constexpr int kZeroFirst = 1 << 18, kZeroSecond = 1 << 19;  // slab entry: half of the slab does not count
 constexpr int kMaxHeads = 256;
 constexpr int kMaxSteps = 2048;  // GEMM-O: k steps of one work item (K <= 65536)
 constexpr int kXcds = 8;
 constexpr int kListThreads = 1024;
-constexpr int kInlineCells = 512;  // up to this many cells the GEMM-Q kernel lists its quads itself
+constexpr int kInlineCells = 256;  // up to this many cells the GEMM-Q kernel lists its quads itself
 constexpr int kWindow = 16;   // token blocks per scheduling window
 constexpr int kQuadInts = 8;  // b, r0, r1, c0, c1, valid mask, pad, pad
 
@@ -286,17 +285,15 @@ __global__ void __launch_bounds__(kListThreads) gemm_quads_kernel(ListArgs a, Li
 // ---------------------------------------------------------------------------------------------
 // Main kernel.  kReduce = false: GEMM-Q.  kReduce = true: GEMM-O.
 // ---------------------------------------------------------------------------------------------
-template <typename T, bool kReduce>
+template <typename T, bool kReduce, bool kHalf>
 __global__ void __launch_bounds__(kThreads) gemm_kernel(const GemmParams p) {
   using TT = Types<T>;
   using x8 = typename TT::x8;
   using x4 = typename TT::x4;
-  constexpr int NT = 4, MT = 2;  // wavefront tile: 128 columns (W rows) x 64 token rows (X rows)
+  constexpr int NT = 4, MT = 4;  // wavefront tile = one unit: 128 columns (W rows) x 128 token rows (X rows)
   extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
   __shared__ int32_t s_heads[kMaxHeads + 1];  // GEMM-O: head | (row0 selects) << 16 | (row1 selects) << 17
   __shared__ int32_t s_nsel;
-  __shared__ __attribute__((aligned(16))) uint8_t s_scrap[1024];
-  __shared__ float s_amax[kThreads / 64];
   // GEMM-O: per k step, k offset | (row0 selects) << 16 | (row1 selects) << 17; four entries past
   // the end repeat the last step
   __shared__ int32_t s_step[kReduce ? kMaxSteps + 4 : 1];
@@ -308,30 +305,26 @@ __global__ void __launch_bounds__(kThreads) gemm_kernel(const GemmParams p) {
   __shared__ int32_t s_entry[8];
 
   const int tid = threadIdx.x, lane = tid & 63;
-  const int wv = __builtin_amdgcn_readfirstlane(tid >> 6);  // wavefront index, kept scalar
+  const int wv = __builtin_amdgcn_readfirstlane(tid >> 6);  // wavefront index = unit of the quad, kept scalar
   const int l32 = lane & 31, g = lane >> 5;
-  // wavefront -> (unit, row half).  Wavefronts w and w+4 share SIMD w%4; SIMD s hosts half 0 of unit s
-  // and half 1 of unit 3-s (unit = 2*token block + column block), so a quad with only one row or
-  // only one column of units still puts one working wavefront on every SIMD.
-  const int wh = wv >> 2;
-  const int unit = wh ? 3 - (wv & 3) : (wv & 3);
-  const int wr = unit >> 1, wc = unit & 1;  // token block, column block
+  const int wr = wv >> 1, wc = wv & 1;  // token block, column block
 
   const T* __restrict__ xg = static_cast<const T*>(p.x);
   const T* __restrict__ wg = static_cast<const T*>(p.w);
 
-  // copy assignment: per stage 32 copy instructions, 16 LDS rows each; wavefront wv issues the
-  // rows 16*wv.. of each of the four tiles (0,1 = X of token block 0,1; 2,3 = W of column block
-  // 0,1).  Lane i lands on row 16*wv + i/4 at chunk position i%4 and must fetch logical chunk
-  // (i%4) ^ ((row >> 2) & 3) = (i%4) ^ ((i >> 4) & 3).
-  // (slab layout: a copy instruction covers 8 rows x 128 B, i.e. whole memory lines; wavefront wv issues
-  // rows 16*wv + 8*n.. (n = 0, 1) of each of the four tiles.  Lane i lands on row 16*wv + 8*n + i/8 at
-  // chunk position i%8 and must fetch logical chunk (i%8) ^ ((row >> 1) & 7) = (i%8) ^ ((4*n + (i >> 4)) & 7).)
-  const int cp_row = 16 * wv + (lane >> 3);
-  const int cp_chunk0 = ((lane & 7) ^ ((lane >> 4) & 7)) * 8;        // element offset inside the slab, n = 0
-  const int cp_chunk1 = ((lane & 7) ^ ((4 + (lane >> 4)) & 7)) * 8;  // n = 1
+  // Load assignment: a slab is 64 pieces of 8 rows x 128 B (whole memory lines), 16 per wavefront:
+  // pieces 0..7 = rows 64*(wv%2) + 8*j.. of X tile wv/2, pieces 8..15 = the same rows of W tile wv/2.
+  // Lane i fetches 16-byte chunk i%8 of row i/8 of its piece and writes it to LDS at chunk position
+  // (i%8) ^ ((row >> 1) & 7) = (i%8) ^ ((4*(j%2) + (i >> 4)) & 7).
+  const int ld_row = 64 * (wv & 1) + (lane >> 3), ld_chunk = lane & 7;
+  int wr_off[2];
+#pragma unroll
+  for (int par = 0; par < 2; ++par)
+    wr_off[par] = (lane >> 3) * kRowBytes + ((ld_chunk ^ ((4 * par + (lane >> 4)) & 7)) << 4);
+  // lanes that hold the first / the second half of a slab's k range
+  const unsigned mask_first = ld_chunk < 4 ? 0xFFFFFFFFu : 0u;
   // operand reads: row = tile row base + l32 (bases are multiples of 32), logical chunk 2*s + g of substep s
-  const int rd_swz = (l32 >> 1) & 7;
+  const int rd_x = (g ^ ((l32 >> 1) & 7)) << 4;
 
   const int xcd = blockIdx.x & (kXcds - 1), slot = blockIdx.x >> 3;
   const int per_xcd = gridDim.x >> 3;  // host launches a multiple of 8 workgroups
@@ -456,11 +449,18 @@ __global__ void __launch_bounds__(kThreads) gemm_kernel(const GemmParams p) {
       c[1] = has_c1 ? c[0] + 1 : c[0];
       valid = 0x1 | (has_c1 ? 0x2 : 0) | (has_r1 ? 0x4 : 0) | (has_r1 && has_c1 ? 0x8 : 0);
     }
+    bz = __builtin_amdgcn_readfirstlane(bz);
+    valid = __builtin_amdgcn_readfirstlane(valid);
+#pragma unroll
+    for (int u = 0; u < 2; ++u) {
+      r[u] = __builtin_amdgcn_readfirstlane(r[u]);
+      c[u] = __builtin_amdgcn_readfirstlane(c[u]);
+    }
     const bool my_valid = (valid >> (wr * 2 + wc)) & 1;
 
     // ---- k-step list ----
     int n_iter;
-    __builtin_amdgcn_s_waitcnt(0x0f70);  // this wavefront's copies and stores of the previous work item
+    __builtin_amdgcn_s_waitcnt(0x0f70);  // this wavefront's loads and stores of the previous work item
     __syncthreads();  // previous work item: LDS tiles and s_heads are free
     if constexpr (kReduce) {
       if (wv == 0) {
@@ -508,22 +508,22 @@ __global__ void __launch_bounds__(kThreads) gemm_kernel(const GemmParams p) {
       n_iter = (p.k + kBK - 1) / kBK;
     }
 
-    // ---- global row pointers of the four operand tiles: X(r0), X(r1), W(c0), W(c1) ----
-    // this wavefront copies rows 16*wv.. of each; rows past M are clamped (their results are dropped)
-    const T* cp_src[4][2];  // [tile][n]
-    {
-      const T* xb = xg + static_cast<int64_t>(bz) * p.m * p.k;
+    // ---- global sources of this wavefront's pieces: X tile r[wv/2], W tile c[wv/2] ----
+    // Buffer loads: a resource descriptor per tile (scalar registers), a 32-bit lane offset per piece,
+    // the slab's k offset as the scalar offset.  The X descriptor ends with the matrix, so rows past
+    // M read as zeros; a token block that does not select a slab's head (GEMM-O) loads through an
+    // empty descriptor, i.e. zeros without touching memory.
+    const int rows_left = min(p.m - r[wr] * kTile, kTile);  // >= 1
+    const __amdgpu_buffer_rsrc_t rsrc_x = __builtin_amdgcn_make_buffer_rsrc(
+        const_cast<T*>(xg + (static_cast<int64_t>(bz) * p.m + static_cast<int64_t>(r[wr]) * kTile) * p.k), 0,
+        rows_left * p.k * 2, 0x00020000);
+    const __amdgpu_buffer_rsrc_t rsrc_w = __builtin_amdgcn_make_buffer_rsrc(
+        const_cast<T*>(wg + static_cast<int64_t>(c[wr]) * kTile * p.k), 0, kTile * p.k * 2, 0x00020000);
+    const __amdgpu_buffer_rsrc_t rsrc_none =
+        __builtin_amdgcn_make_buffer_rsrc(const_cast<T*>(xg), 0, 0, 0x00020000);
+    int ld_off[8];
 #pragma unroll
-      for (int u = 0; u < 2; ++u)
-#pragma unroll
-        for (int n = 0; n < 2; ++n) {
-          int xr = r[u] * kTile + cp_row + 8 * n;
-          xr = xr < p.m ? xr : p.m - 1;
-          const int chunk = n ? cp_chunk1 : cp_chunk0;
-          cp_src[u][n] = xb + static_cast<int64_t>(xr) * p.k + chunk;
-          cp_src[2 + u][n] = wg + static_cast<int64_t>(c[u] * kTile + cp_row + 8 * n) * p.k + chunk;
-        }
-    }
+    for (int j = 0; j < 8; ++j) ld_off[j] = (ld_row + 8 * j) * p.k * 2 + ld_chunk * 16;
     // k offset of step it (steps past the end repeat the last one); GEMM-O: plus the select bits
     auto step_entry = [&](int it) -> int {
       if constexpr (kReduce) {
@@ -534,57 +534,95 @@ __global__ void __launch_bounds__(kThreads) gemm_kernel(const GemmParams p) {
         return (i + 1) * kBK <= p.k ? i * kBK | 0x30000 : (p.k - kBK) | kZeroFirst | 0x30000;
       }
     };
-    // copies past the last k step (kept so that every step issues the same instructions) land in a
-    // scrap kilobyte, so the ring is free for the epilogue as soon as the last reads are done
-    auto copy_one = [&](int it, int entry, int idx) {  // idx = 2 * tile + n
-      uint8_t* dst = it < n_iter ? smem + (it % kStages) * kStageBytes + (idx >> 1) * kUnitBytes + wv * 2048 +
-                                       (idx & 1) * 1024
-                                 : s_scrap;
-      copy16_to_lds(cp_src[idx >> 1][idx & 1] + (entry & 0xFFFF), dst);
+    // Staging registers: piece j of a slab waits here between its global load and its LDS write.
+    u32x4 stg[16];
+    auto gload = [&](int j, int entry) {  // j < 8: X, else W
+      const int koff = (entry & 0xFFFF) * 2;
+      if (j < 8) {
+        const bool sel = (entry >> (16 + wr)) & 1;
+        stg[j] = __builtin_amdgcn_raw_buffer_load_b128(sel ? rsrc_x : rsrc_none, ld_off[j], koff, 0);
+      } else {
+        stg[j] = __builtin_amdgcn_raw_buffer_load_b128(rsrc_w, ld_off[j - 8], koff, 0);
+      }
     };
-    auto copy_stage = [&](int it) {
-      const int entry = step_entry(it);
+    // kHalf: only one half of a slab that reaches into its neighbour counts; the other half of its X
+    // pieces is cleared on the way to LDS
+    auto keep_of = [&](int entry) -> unsigned {
+      return (entry & kZeroFirst) ? ~mask_first : ((entry & kZeroSecond) ? mask_first : 0xFFFFFFFFu);
+    };
+    auto lwrite = [&](int j, int stage, unsigned keep) {
+      uint8_t* dst = smem + stage * kStageBytes + ((j < 8 ? 0 : 2) + wr) * kUnitBytes +
+                     (64 * (wv & 1) + 8 * (j & 7)) * kRowBytes + wr_off[j & 1];
+      u32x4 v = stg[j];
+      if constexpr (kHalf) {
+        if (j < 8) v &= keep;
+      }
+      *reinterpret_cast<u32x4*>(dst) = v;
+    };
+
+    // ---- pipeline ----
+    // Two slab buffers in LDS (stage it % 2 holds slab it) and one slab in flight in the staging
+    // registers.  Iteration it: substeps 0..2 of slab it run while pieces 4..15 of slab it+1 go from
+    // the staging registers into the other stage and the same pieces of slab it+2 are requested; one
+    // barrier (every wavefront has read all of slab it and written all of slab it+1); substep 3 runs
+    // while the first operands of slab it+1 are read, pieces 0..3 of slab it+2 go into stage it % 2
+    // and those of slab it+3 are requested.  Every substep issues the same mix: sixteen MFMAs, eight
+    // operand reads, four LDS writes, four global loads, so the memory path sees an even stream and
+    // a load has a whole slab period to arrive.
+    if (n_iter > 0) {
+      const int e0 = step_entry(0), e1 = step_entry(1), e2 = step_entry(2);
 #pragma unroll
-      for (int j = 0; j < kCopiesPerWave; ++j) copy_one(it, entry, j);
-    };
+      for (int j = 0; j < 16; ++j) gload(j, e0);
+      {
+        const unsigned keep = keep_of(e0);
+#pragma unroll
+        for (int j = 0; j < 16; ++j) lwrite(j, 0, keep);
+      }
+#pragma unroll
+      for (int j = 0; j < 16; ++j) gload(j, e1);
+      {
+        const unsigned keep = keep_of(e1);
+#pragma unroll
+        for (int j = 0; j < 4; ++j) lwrite(j, 1, keep);
+      }
+#pragma unroll
+      for (int j = 0; j < 4; ++j) gload(j, e2);
+      __builtin_amdgcn_s_waitcnt(0xc07f);  // lgkmcnt(0)
+      __builtin_amdgcn_s_barrier();
+    }
 
     if (!my_valid) {
       // This wavefront's unit does not exist in this quad (unflagged, or past the matrix edge): it
-      // only does its share of the copies and keeps the barrier and vmcnt sequence of the others,
-      // leaving its SIMD's matrix core to the other wavefront.
-      __builtin_amdgcn_s_waitcnt(0x0f70);
-      if (n_iter > 0) {
-        copy_stage(0);
-        copy_stage(1);
-        __builtin_amdgcn_s_waitcnt(0x0f70 | kCopiesPerWave);
-        __builtin_amdgcn_s_barrier();
-        for (int it = 0; it < n_iter; ++it) {
-          __builtin_amdgcn_s_waitcnt(0x0f70);
-          __builtin_amdgcn_s_barrier();
-          copy_stage(it + 2);
+      // only moves its pieces and keeps the barrier sequence of the others.
+      for (int it = 0; it < n_iter; ++it) {
+        const int st = it & 1;
+        const int en1 = step_entry(it + 1), en2 = step_entry(it + 2), en3 = step_entry(it + 3);
+        const unsigned keep1 = keep_of(en1), keep2 = keep_of(en2);
+#pragma unroll
+        for (int j = 4; j < 16; ++j) {
+          lwrite(j, st ^ 1, keep1);
+          gload(j, en2);
         }
-        __builtin_amdgcn_s_barrier();  // the others' "ring is free" barrier before their epilogue
+        __builtin_amdgcn_s_waitcnt(0xc07f);
+        __builtin_amdgcn_s_barrier();
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+          lwrite(j, st, keep2);
+          gload(j, en3);
+        }
       }
-      if constexpr (!kReduce) {
-        if (p.y8) __builtin_amdgcn_s_barrier();  // ... and the one of their absmax exchange
+      if (n_iter > 0) {
+        __builtin_amdgcn_s_waitcnt(0xc07f);
+        __builtin_amdgcn_s_barrier();  // the others' "ring is free" barrier before their epilogue
       }
       continue;
     }
 
     // ---- accumulators (bias / cached partial are added in the epilogue) ----
     // acc[nt][mt][i]: n = n0 + nt*32 + (i/4)*8 + g*4 + i%4, m = m0 + mt*32 + l32
-    const int m0 = r[wr] * kTile + wh * 64;
+    const int m0 = r[wr] * kTile;
     const int n0 = c[wc] * kTile;
-    const int64_t y_batch = static_cast<int64_t>(bz) * p.m * p.n;
     f32x16 acc[NT][MT];
-    // the previous work item's stores are complete: from here on vmcnt counts loads only
-    __builtin_amdgcn_s_waitcnt(0x0f70);
-    __builtin_amdgcn_sched_barrier(0);
-    if (n_iter > 0) {
-      copy_stage(0);
-      copy_stage(1);
-    }
-    __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
     for (int nt = 0; nt < NT; ++nt)
 #pragma unroll
@@ -592,159 +630,113 @@ __global__ void __launch_bounds__(kThreads) gemm_kernel(const GemmParams p) {
 #pragma unroll
         for (int i = 0; i < 16; ++i) acc[nt][mt][i] = 0.f;
 
-    // LDS byte offsets of this wavefront's operand rows inside a stage
-    const int a_base = (2 + wc) * kUnitBytes + l32 * kRowBytes;        // W rows nt*32 + l32
-    const int b_base = wr * kUnitBytes + (wh * 64 + l32) * kRowBytes;  // X rows wh*64 + mt*32 + l32
-
-    // ---- main loop ----
-    // One slab = 64 k = four substeps of eight MFMAs.  Two slabs in LDS: slab it is read while slab
-    // it+1 lands.  Operand reads run one substep ahead of the MFMAs that use them (two register
-    // sets).  One barrier per slab, before its last substep: by then slab it+1 has landed for every
-    // wavefront and every wavefront has its last operands of slab it in registers, so the copies of
-    // slab it+2 may overwrite it; they and the first reads of slab it+1 go into the shadow of the last
-    // substep's MFMAs.
-    x8 a[2][NT], b[2][MT];
-    // one operand read of substep sub of slab it into register set sub & 1: j = 0..3 W rows, j = 4..5 X rows
-    auto read_one = [&](int it, int sub, int j) {
-      const uint8_t* st = smem + (it % kStages) * kStageBytes;
-      const int sw = ((2 * sub + g) ^ rd_swz) << 4;
-      if (j < NT) {
-        a[sub & 1][j] = *reinterpret_cast<const x8*>(st + a_base + j * 32 * kRowBytes + sw);
-      } else {
-        b[sub & 1][j - NT] = *reinterpret_cast<const x8*>(st + b_base + (j - NT) * 32 * kRowBytes + sw);
-      }
-    };
-    // the eight MFMAs of register set ks; in their shadow the six operand reads of substep rsub of slab
-    // rit and, if cit >= 0, this wavefront's eight copies of slab cit.  An X operand that does not count
-    // (GEMM-O: the token block does not select this slab's head; the half of a slab that reaches into
-    // its neighbour) is zeroed (keep = 0).  (Skipping the MFMAs instead puts them under a branch, and
-    // the register allocator then copies and spills accumulators in the loop.)
-    auto math_and_read = [&](int ks, unsigned keep, bool masked, int rit, int rsub, int cit, int centry) {
-      if (masked) {
-#pragma unroll
-        for (int mt = 0; mt < MT; ++mt) {
-          u32x4 v = __builtin_bit_cast(u32x4, b[ks][mt]);
-          v &= keep;
-          b[ks][mt] = __builtin_bit_cast(x8, v);
-        }
-      }
-#pragma unroll
-      for (int i = 0; i < NT * MT; ++i) {
-        const int nt = i / MT, mt = i % MT;
-        acc[nt][mt] = TT::mfma(a[ks][nt], b[ks][mt], acc[nt][mt]);
-        if (cit >= 0 && i < kCopiesPerWave) copy_one(cit, centry, i);
-        if (i < NT + MT) read_one(rit, rsub, i);
-        __builtin_amdgcn_sched_barrier(0);
-      }
-    };
-    // keep masks of a slab's first and second half for this wavefront's token block
-    auto keep_of = [&](int entry, int half) -> unsigned {
-      const bool sel = (entry >> (16 + wr)) & 1;
-      const bool zero = entry & (half ? kZeroSecond : kZeroFirst);
-      return sel && !zero ? 0xFFFFFFFFu : 0u;
-    };
-    // Copies past the last slab repeat the last one (into a scrap kilobyte), so the loop body is the
-    // same for every slab.
     if (n_iter > 0) {
-      __builtin_amdgcn_s_waitcnt(0x0f70 | kCopiesPerWave);  // slab 0 landed, slab 1 in flight
-      __builtin_amdgcn_s_barrier();
-#pragma unroll
-      for (int j = 0; j < NT + MT; ++j) read_one(0, 0, j);
-      int entry = step_entry(0);
-      auto slab = [&](int it, bool masked) {
-        const int centry = step_entry(it + 2);
-        const int entry_next = step_entry(it + 1);
-        const unsigned keep0 = keep_of(entry, 0), keep1 = keep_of(entry, 1);
-        math_and_read(0, keep0, masked, it, 1, -1, 0);
-        math_and_read(1, keep0, masked, it, 2, -1, 0);
-        math_and_read(0, keep1, masked, it, 3, -1, 0);
-        __builtin_amdgcn_s_waitcnt(0x0070);  // vmcnt(0), lgkmcnt(0): slab it+1 landed, last operands of slab it here
-        __builtin_amdgcn_s_barrier();        // ... for every wavefront
-        math_and_read(1, keep1, masked, it + 1, 0, it + 2, centry);
-        entry = entry_next;
+      // LDS byte offsets of this wavefront's operand rows inside a stage
+      const int a_base = (2 + wc) * kUnitBytes + l32 * kRowBytes;  // W rows nt*32 + l32
+      const int b_base = wr * kUnitBytes + l32 * kRowBytes;        // X rows mt*32 + l32
+      x8 a[2][NT], b[2][MT];
+      // operand read idx of substep sub of the slab in `stage` into register set sub & 1, in the order
+      // the MFMAs need them: W rows 0, X rows 0..3, W rows 1..3
+      auto lread = [&](int stage, int sub, int idx) {
+        const uint8_t* st = smem + stage * kStageBytes;
+        const int x = rd_x ^ (sub << 5);
+        if (idx == 0) {
+          a[sub & 1][0] = *reinterpret_cast<const x8*>(st + a_base + x);
+        } else if (idx <= MT) {
+          b[sub & 1][idx - 1] = *reinterpret_cast<const x8*>(st + b_base + (idx - 1) * 32 * kRowBytes + x);
+        } else {
+          a[sub & 1][idx - MT] = *reinterpret_cast<const x8*>(st + a_base + (idx - MT) * 32 * kRowBytes + x);
+        }
       };
-      if constexpr (kReduce) {
-        for (int it = 0; it < n_iter; ++it) slab(it, true);
-      } else {
-        // only the last slab can hold a half that does not count (K % 64 == 32)
-        for (int it = 0; it < n_iter - 1; ++it) slab(it, false);
-        slab(n_iter - 1, true);
+      // one substep: the sixteen MFMAs of register set `set`; in their shadow the eight operand reads
+      // of substep rsub of the slab in rstage, and pieces j0..j0+3: staged -> LDS stage wstage, then the
+      // same pieces of the slab with entry `lentry` -> staging
+      auto substep = [&](int set, int rstage, int rsub, int wstage, int j0, unsigned keep, int lentry) {
+#pragma unroll
+        for (int i = 0; i < NT * MT; ++i) {
+          const int nt = i / MT, mt = i % MT;
+          acc[nt][mt] = TT::mfma(a[set][nt], b[set][mt], acc[nt][mt]);
+          if ((i & 1) == 0) lread(rstage, rsub, i >> 1);
+          if ((i & 3) == 1) lwrite(j0 + (i >> 2), wstage, keep);
+          if ((i & 3) == 3) gload(j0 + (i >> 2), lentry);
+          __builtin_amdgcn_sched_barrier(0);
+        }
+      };
+#pragma unroll
+      for (int idx = 0; idx < NT + MT; ++idx) lread(0, 0, idx);
+      for (int it = 0; it < n_iter; ++it) {
+        const int st = it & 1;
+        const int en1 = step_entry(it + 1), en2 = step_entry(it + 2), en3 = step_entry(it + 3);
+        const unsigned keep1 = keep_of(en1), keep2 = keep_of(en2);
+        substep(0, st, 1, st ^ 1, 4, keep1, en2);
+        substep(1, st, 2, st ^ 1, 8, keep1, en2);
+        substep(0, st, 3, st ^ 1, 12, keep1, en2);
+        __builtin_amdgcn_s_waitcnt(0xc07f);  // lgkmcnt(0): my reads of slab it and my writes of slab it+1 are done
+        __builtin_amdgcn_s_barrier();        // ... for every wavefront
+        substep(1, st ^ 1, 0, st, 0, keep2, en3);
       }
+      __builtin_amdgcn_s_waitcnt(0xc07f);
+      __builtin_amdgcn_s_barrier();  // every wavefront is done with the ring
     }
 
     // ---- epilogue ----
     // In the accumulator layout a lane owns one output row and runs of four columns: written from
     // there, a store instruction is 64 scattered 8-byte pieces (measured: ~12 % of the FLUX-sized
     // launches; the bias matrix read the same way, as much again).  Each wavefront therefore turns
-    // its 64 x 128 block through its own 16 KB of the ring, 32 rows at a time in fp32, and adds the
+    // its 128 x 128 block through its own quarter of the ring, 32 rows at a time in fp32, and adds the
     // bias and stores from a layout in which 32 consecutive lanes cover one row.
-    if (n_iter > 0) __builtin_amdgcn_s_barrier();  // every wavefront is done reading the ring
     {
       // (the lane index is made opaque: otherwise the per-lane address terms are computed once per
       // kernel, spilled, and every reload waits for the store before it)
       int ln = lane;
       asm volatile("" : "+v"(ln));
       const int col4 = ln & 31, rsub = ln >> 5, wl32 = ln & 31, wg = ln >> 5;
-      uint8_t* region = smem + wv * (kSmemBytes / 8);
+      uint8_t* const region0 = smem + wv * (kSmemBytes / 4);
       const int64_t y_batch = static_cast<int64_t>(bz) * p.m * p.n;
       float bvec[4] = {0.f, 0.f, 0.f, 0.f};
-      // Fused quantisation (GEMM-Q): a unit is one (token block, head) slab, owned by two wavefronts.
-      // Its absmax needs the final values, so the bias is added in the accumulator layout here; the
-      // two wavefronts exchange their maxima through LDS; scale = absmax / 448 (1 for a zero slab).
+      // Fused quantisation (GEMM-Q): a unit is one (token block, head) slab.  Its absmax is taken
+      // over the final values (accumulator + bias, formed here in the accumulator layout without
+      // being kept: the bias is added for good after the turn below); scale = absmax / 448 (1 for a
+      // zero slab).
       float qscale = 1.f;
-      bool bias_added = false;
       if constexpr (!kReduce) {
         if (p.y8) {
-          if (p.bias_kind == FO_BIAS_VECTOR) {
-            // all sixteen pieces requested before the first is used (taken one by one, each load
-            // waits for the one before it and for the trailing tile copies)
-            x4 bvs[NT * 4];
-#pragma unroll
-            for (int nt = 0; nt < NT; ++nt)
-#pragma unroll
-              for (int i4 = 0; i4 < 4; ++i4)
-                bvs[nt * 4 + i4] = *reinterpret_cast<const x4*>(static_cast<const T*>(p.bias) + n0 + nt * 32 +
-                                                                i4 * 8 + wg * 4);
-            __builtin_amdgcn_sched_barrier(0);
-#pragma unroll
-            for (int nt = 0; nt < NT; ++nt)
-#pragma unroll
-              for (int i4 = 0; i4 < 4; ++i4)
-#pragma unroll
-                for (int mt = 0; mt < MT; ++mt)
-#pragma unroll
-                  for (int j = 0; j < 4; ++j) acc[nt][mt][i4 * 4 + j] += static_cast<float>(bvs[nt * 4 + i4][j]);
-            bias_added = true;
-          }
+          const bool has_vec = p.bias_kind == FO_BIAS_VECTOR;
           float amax = 0.f;
 #pragma unroll
-          for (int mt = 0; mt < MT; ++mt)
-            if (m0 + mt * 32 + wl32 < p.m) {
+          for (int nt = 0; nt < NT; ++nt)
 #pragma unroll
-              for (int nt = 0; nt < NT; ++nt)
+            for (int i4 = 0; i4 < 4; ++i4) {
+              float bq[4] = {0.f, 0.f, 0.f, 0.f};
+              if (has_vec) {
+                const x4 bv = *reinterpret_cast<const x4*>(static_cast<const T*>(p.bias) + n0 + nt * 32 + i4 * 8 + wg * 4);
 #pragma unroll
-                for (int i = 0; i < 16; ++i) amax = fmaxf(amax, fabsf(acc[nt][mt][i]));
+                for (int j = 0; j < 4; ++j) bq[j] = static_cast<float>(bv[j]);
+              }
+#pragma unroll
+              for (int mt = 0; mt < MT; ++mt)
+                if (m0 + mt * 32 + wl32 < p.m) {
+#pragma unroll
+                  for (int j = 0; j < 4; ++j) amax = fmaxf(amax, fabsf(acc[nt][mt][i4 * 4 + j] + bq[j]));
+                }
             }
 #pragma unroll
           for (int off = 32; off > 0; off >>= 1) amax = fmaxf(amax, __shfl_xor(amax, off, 64));
-          if (lane == 0) s_amax[wv] = amax;
-          __builtin_amdgcn_s_waitcnt(0xc07f);  // lgkmcnt(0)
-          __builtin_amdgcn_s_barrier();
-          amax = fmaxf(s_amax[wv], s_amax[7 - wv]);  // the other half of the unit is wavefront 7 - wv
           qscale = amax > 0.f ? amax / 448.0f : 1.0f;
-          if (wh == 0 && lane == 0)
+          if (lane == 0)
             p.y_scale[static_cast<int64_t>(c[wc]) * p.scale_row_len + bz * p.n_row_tiles + r[wr]] = qscale;
         }
       }
-      if (p.bias_kind == FO_BIAS_VECTOR && !bias_added) {
+      if (p.bias_kind == FO_BIAS_VECTOR) {
         const x4 bv = *reinterpret_cast<const x4*>(static_cast<const T*>(p.bias) + n0 + col4 * 4);
 #pragma unroll
         for (int j = 0; j < 4; ++j) bvec[j] = static_cast<float>(bv[j]);
       }
-      // one half (32 rows) of the block; BiasT: element type of the bias matrix, if there is one
+      // 32 rows of the block; BiasT: element type of the bias matrix, if there is one
       auto turn_half = [&](int mt, auto bias_tag) {
         using BiasT = decltype(bias_tag);
         const int row_base = m0 + mt * 32;
+        uint8_t* const region = region0 + (mt & 1) * (kSmemBytes / 8);
         // 16-byte chunk c of row r sits at chunk position c ^ r (rows are 512 bytes = 32 chunks)
 #pragma unroll
         for (int nt = 0; nt < NT; ++nt)
@@ -848,15 +840,15 @@ int64_t workspace_ints(const ListGeom& gm, int64_t* max_quads_out) {
   return 16 + kQuadInts * max_quads;
 }
 
-template <typename T, bool kReduce>
-int launch(GemmParams& p, const ListGeom& gm, bool use_flags, void* workspace, hipStream_t stream) {
+template <typename T, bool kReduce, bool kHalf>
+int launch_half(GemmParams& p, const ListGeom& gm, bool use_flags, void* workspace, hipStream_t stream) {
   // (the attribute belongs to the kernel's code object on one device: set once per device; the flags
   // are atomic because host threads may launch concurrently, and setting it twice is harmless)
   static std::atomic<bool> attr_set[64] = {};
   int dev = 0;
   FO_HIP_CALL(hipGetDevice(&dev));
   if (dev < 0 || dev >= 64 || !attr_set[dev].load(std::memory_order_acquire)) {
-    FO_HIP_CALL(hipFuncSetAttribute(reinterpret_cast<const void*>(&gemm_kernel<T, kReduce>),
+    FO_HIP_CALL(hipFuncSetAttribute(reinterpret_cast<const void*>(&gemm_kernel<T, kReduce, kHalf>),
                                     hipFuncAttributeMaxDynamicSharedMemorySize, kSmemBytes));
     if (dev >= 0 && dev < 64) attr_set[dev].store(true, std::memory_order_release);
   }
@@ -877,7 +869,7 @@ int launch(GemmParams& p, const ListGeom& gm, bool use_flags, void* workspace, h
     // every unit is computed: no list, the kernel enumerates the quads itself
     p.quads = nullptr;
     p.qoff = nullptr;
-    gemm_kernel<T, kReduce><<<static_cast<unsigned>(grid), kThreads, kSmemBytes, stream>>>(p);
+    gemm_kernel<T, kReduce, kHalf><<<static_cast<unsigned>(grid), kThreads, kSmemBytes, stream>>>(p);
     FO_CHECK_LAUNCH();
     return FO_OK;
   }
@@ -887,7 +879,7 @@ int launch(GemmParams& p, const ListGeom& gm, bool use_flags, void* workspace, h
     p.quads = nullptr;
     p.qoff = nullptr;
     p.inline_cells = static_cast<int32_t>(n_cells);
-    gemm_kernel<T, kReduce><<<static_cast<unsigned>(grid), kThreads, kSmemBytes, stream>>>(p);
+    gemm_kernel<T, kReduce, kHalf><<<static_cast<unsigned>(grid), kThreads, kSmemBytes, stream>>>(p);
     FO_CHECK_LAUNCH();
     return FO_OK;
   }
@@ -905,9 +897,18 @@ int launch(GemmParams& p, const ListGeom& gm, bool use_flags, void* workspace, h
   FO_CHECK_LAUNCH();
   p.quads = quads;
   p.qoff = qoff;
-  gemm_kernel<T, kReduce><<<static_cast<unsigned>(grid), kThreads, kSmemBytes, stream>>>(p);
+  gemm_kernel<T, kReduce, kHalf><<<static_cast<unsigned>(grid), kThreads, kSmemBytes, stream>>>(p);
   FO_CHECK_LAUNCH();
   return FO_OK;
+}
+
+// kHalf: the k range is cut into slabs of 64 and some slab counts for one half only (GEMM-Q: K % 64 == 32;
+// GEMM-O: head slices of width 32 mod 64)
+template <typename T, bool kReduce>
+int launch(GemmParams& p, const ListGeom& gm, bool use_flags, void* workspace, hipStream_t stream) {
+  const bool half = (kReduce ? p.head_dim : p.k) % kBK != 0;
+  return half ? launch_half<T, kReduce, true>(p, gm, use_flags, workspace, stream)
+              : launch_half<T, kReduce, false>(p, gm, use_flags, workspace, stream);
 }
 
 int check_common(const void* x, const void* w, void* y, int dtype, int32_t batch, int32_t m,
