@@ -285,7 +285,7 @@ __global__ void __launch_bounds__(kListThreads) gemm_quads_kernel(ListArgs a, Li
 // ---------------------------------------------------------------------------------------------
 // Main kernel.  kReduce = false: GEMM-Q.  kReduce = true: GEMM-O.
 // ---------------------------------------------------------------------------------------------
-template <typename T, bool kReduce, bool kHalf>
+template <typename T, bool kReduce, bool kHalf, bool kQuant>
 __global__ void __launch_bounds__(kThreads) gemm_kernel(const GemmParams p) {
   using TT = Types<T>;
   using x8 = typename TT::x8;
@@ -303,6 +303,7 @@ __global__ void __launch_bounds__(kThreads) gemm_kernel(const GemmParams p) {
   __shared__ uint32_t s_cell_mask[kReduce ? 1 : 2 * kInlineCells];
   __shared__ int32_t s_cell_wave[kThreads / 64];
   __shared__ int32_t s_entry[8];
+  __shared__ float s_amax[kThreads / 64];
 
   const int tid = threadIdx.x, lane = tid & 63;
   const int wv = __builtin_amdgcn_readfirstlane(tid >> 6);  // wavefront index = unit of the quad, kept scalar
@@ -332,8 +333,9 @@ __global__ void __launch_bounds__(kThreads) gemm_kernel(const GemmParams p) {
   // (8 row pairs; the last window may be shorter), column pairs inside a window, row pairs inside
   // a column pair
   const int full_w = p.n_row_tiles / kWindow, last_rows = p.n_row_tiles % kWindow;
+  constexpr int per_win = kWindow / 2;  // work items per window and column pair
   const int last_q = (last_rows + 1) / 2;
-  const int quads_per_batch = (full_w * (kWindow / 2) + last_q) * p.n_cp;
+  const int quads_per_batch = (full_w * per_win + last_q) * p.n_cp;
   int q_lo, q_len;
   bool inline_list = false;
   if constexpr (!kReduce) inline_list = p.inline_cells > 0;
@@ -386,7 +388,20 @@ __global__ void __launch_bounds__(kThreads) gemm_kernel(const GemmParams p) {
     q_len = static_cast<int>(total * (xcd + 1) / kXcds) - q_lo;
   }
 
-  for (int work = slot; work < q_len; work += per_xcd) {
+  // ---- work items ----
+  // A work item = a quad: four operand tiles per slab (X r0, X r1, W c0, W c1), wavefront = unit,
+  // 128 x 128 each.  (A second shape was measured and dropped: quads with two units that share a
+  // tile, computed by two wavefronts per unit at 64 x 128 each from three tiles.  Its slab takes as
+  // long as a full one (nine LDS transfers per eight MFMAs saturate a wavefront's LDS path), and work
+  // items of unequal length let the workgroups of an XCD drift apart in k, which costs the L2 hits on
+  // the tiles they share.)
+  constexpr int P = 16;      // pieces per wavefront and slab: rows 32*wv + 8*jj.. (jj = 0..3) of every tile
+  constexpr int PS = P / 4;  // pieces per substep
+  struct Item {
+    int bz, valid, r[2], c[2];
+  };
+  // (called by all threads together: the listing form hands the entry over through LDS)
+  auto decode_item = [&](int work) -> Item {
     int bz, valid, r[2], c[2];
     if (inline_list) {
       if constexpr (!kReduce) {
@@ -429,14 +444,14 @@ __global__ void __launch_bounds__(kThreads) gemm_kernel(const GemmParams p) {
       bz = q / quads_per_batch;
       int rem = q - bz * quads_per_batch;
       int w, cp, i, rows;
-      if (rem < full_w * p.n_cp * (kWindow / 2)) {
-        const int cell = rem / (kWindow / 2);
-        i = rem - cell * (kWindow / 2);
+      if (rem < full_w * p.n_cp * per_win) {
+        const int cell = rem / per_win;
+        i = rem - cell * per_win;
         w = cell / p.n_cp;
         cp = cell - w * p.n_cp;
         rows = kWindow;
       } else {
-        rem -= full_w * p.n_cp * (kWindow / 2);
+        rem -= full_w * p.n_cp * per_win;
         cp = rem / last_q;
         i = rem - cp * last_q;
         w = full_w;
@@ -449,19 +464,22 @@ __global__ void __launch_bounds__(kThreads) gemm_kernel(const GemmParams p) {
       c[1] = has_c1 ? c[0] + 1 : c[0];
       valid = 0x1 | (has_c1 ? 0x2 : 0) | (has_r1 ? 0x4 : 0) | (has_r1 && has_c1 ? 0x8 : 0);
     }
-    bz = __builtin_amdgcn_readfirstlane(bz);
-    valid = __builtin_amdgcn_readfirstlane(valid);
+    Item it;
+    it.bz = __builtin_amdgcn_readfirstlane(bz);
+    it.valid = __builtin_amdgcn_readfirstlane(valid);
 #pragma unroll
     for (int u = 0; u < 2; ++u) {
-      r[u] = __builtin_amdgcn_readfirstlane(r[u]);
-      c[u] = __builtin_amdgcn_readfirstlane(c[u]);
+      it.r[u] = __builtin_amdgcn_readfirstlane(r[u]);
+      it.c[u] = __builtin_amdgcn_readfirstlane(c[u]);
     }
-    const bool my_valid = (valid >> (wr * 2 + wc)) & 1;
-
-    // ---- k-step list ----
+    return it;
+  };
+  // k-step list of an item (GEMM-O: the union of the two token blocks' selected heads); returns the
+  // number of slabs.  Called by all threads together, when nobody reads the previous list any more.
+  auto build_steps = [&](const Item& item) -> int {
+    const int bz = item.bz, valid = item.valid;
+    const int r[2] = {item.r[0], item.r[1]};
     int n_iter;
-    __builtin_amdgcn_s_waitcnt(0x0f70);  // this wavefront's loads and stores of the previous work item
-    __syncthreads();  // previous work item: LDS tiles and s_heads are free
     if constexpr (kReduce) {
       if (wv == 0) {
         const uint8_t* info = p.sparse_info + p.sparse_info_indptr[bz];
@@ -492,7 +510,7 @@ __global__ void __launch_bounds__(kThreads) gemm_kernel(const GemmParams p) {
       // into the slab before it and counts for its second half only (the first slice of the matrix
       // instead reaches forward and counts for its first half)
       const int iph = (p.head_dim + kBK - 1) / kBK;
-      n_iter = s_nsel * iph;
+      n_iter = __builtin_amdgcn_readfirstlane(s_nsel) * iph;
       if (n_iter > 0) {
         for (int i = tid; i < n_iter + 4; i += kThreads) {
           const int ii = i < n_iter ? i : n_iter - 1;
@@ -508,89 +526,154 @@ __global__ void __launch_bounds__(kThreads) gemm_kernel(const GemmParams p) {
       n_iter = (p.k + kBK - 1) / kBK;
     }
 
-    // ---- global sources of this wavefront's pieces: X tile r[wv/2], W tile c[wv/2] ----
-    // Buffer loads: a resource descriptor per tile (scalar registers), a 32-bit lane offset per piece,
-    // the slab's k offset as the scalar offset.  The X descriptor ends with the matrix, so rows past
-    // M read as zeros; a token block that does not select a slab's head (GEMM-O) loads through an
-    // empty descriptor, i.e. zeros without touching memory.
-    const int rows_left = min(p.m - r[wr] * kTile, kTile);  // >= 1
-    const __amdgpu_buffer_rsrc_t rsrc_x = __builtin_amdgcn_make_buffer_rsrc(
-        const_cast<T*>(xg + (static_cast<int64_t>(bz) * p.m + static_cast<int64_t>(r[wr]) * kTile) * p.k), 0,
-        rows_left * p.k * 2, 0x00020000);
-    const __amdgpu_buffer_rsrc_t rsrc_w = __builtin_amdgcn_make_buffer_rsrc(
-        const_cast<T*>(wg + static_cast<int64_t>(c[wr]) * kTile * p.k), 0, kTile * p.k * 2, 0x00020000);
-    const __amdgpu_buffer_rsrc_t rsrc_none =
-        __builtin_amdgcn_make_buffer_rsrc(const_cast<T*>(xg), 0, 0, 0x00020000);
-    int ld_off[8];
+    return n_iter;
+  };
+  int n_iter = 0;
+  // k offset of step it (steps past the end repeat the last one); GEMM-O: plus the select bits
+  auto step_entry = [&](int it) -> int {
+    if constexpr (kReduce) {
+      return __builtin_amdgcn_readfirstlane(s_step[it]);  // uniform: the descriptor choice below stays scalar
+    } else {
+      // (K % 64 == 32: the last slab reaches 32 back and counts for its second half only)
+      const int i = it < n_iter ? it : n_iter - 1;
+      return (i + 1) * kBK <= p.k ? i * kBK | 0x30000 : (p.k - kBK) | kZeroFirst | 0x30000;
+    }
+  };
+  // the same without making the list's value scalar (that needs the LDS read to have returned)
+  auto step_entry_raw = [&](int it) -> int {
+    if constexpr (kReduce) {
+      return s_step[it];
+    } else {
+      return step_entry(it);
+    }
+  };
+  // ---- operand tiles: buffer resource descriptors in scalar registers ----
+  // The X descriptors end with the matrix, so rows past M read as zeros; a token block that does
+  // not select a slab's head (GEMM-O) loads through an empty descriptor: zeros, no memory access.
+  const __amdgpu_buffer_rsrc_t rsrc_none = __builtin_amdgcn_make_buffer_rsrc(const_cast<T*>(xg), 0, 0, 0x00020000);
+  __amdgpu_buffer_rsrc_t rsrc[4] = {rsrc_none, rsrc_none, rsrc_none, rsrc_none};
+  auto make_rsrc = [&](const Item& item) {
 #pragma unroll
-    for (int j = 0; j < 8; ++j) ld_off[j] = (ld_row + 8 * j) * p.k * 2 + ld_chunk * 16;
-    // k offset of step it (steps past the end repeat the last one); GEMM-O: plus the select bits
-    auto step_entry = [&](int it) -> int {
-      if constexpr (kReduce) {
-        return s_step[it];
-      } else {
-        // (K % 64 == 32: the last slab reaches 32 back and counts for its second half only)
-        const int i = it < n_iter ? it : n_iter - 1;
-        return (i + 1) * kBK <= p.k ? i * kBK | 0x30000 : (p.k - kBK) | kZeroFirst | 0x30000;
-      }
-    };
-    // Staging registers: piece j of a slab waits here between its global load and its LDS write.
-    u32x4 stg[16];
-    auto gload = [&](int j, int entry) {  // j < 8: X, else W
-      const int koff = (entry & 0xFFFF) * 2;
-      if (j < 8) {
-        const bool sel = (entry >> (16 + wr)) & 1;
-        stg[j] = __builtin_amdgcn_raw_buffer_load_b128(sel ? rsrc_x : rsrc_none, ld_off[j], koff, 0);
-      } else {
-        stg[j] = __builtin_amdgcn_raw_buffer_load_b128(rsrc_w, ld_off[j - 8], koff, 0);
-      }
-    };
-    // kHalf: only one half of a slab that reaches into its neighbour counts; the other half of its X
-    // pieces is cleared on the way to LDS
-    auto keep_of = [&](int entry) -> unsigned {
-      return (entry & kZeroFirst) ? ~mask_first : ((entry & kZeroSecond) ? mask_first : 0xFFFFFFFFu);
-    };
-    auto lwrite = [&](int j, int stage, unsigned keep) {
-      uint8_t* dst = smem + stage * kStageBytes + ((j < 8 ? 0 : 2) + wr) * kUnitBytes +
-                     (64 * (wv & 1) + 8 * (j & 7)) * kRowBytes + wr_off[j & 1];
-      u32x4 v = stg[j];
-      if constexpr (kHalf) {
-        if (j < 8) v &= keep;
-      }
-      *reinterpret_cast<u32x4*>(dst) = v;
-    };
+    for (int u = 0; u < 2; ++u) {
+      const int rows_left = min(p.m - item.r[u] * kTile, kTile);  // >= 1
+      rsrc[u] = __builtin_amdgcn_make_buffer_rsrc(
+          const_cast<T*>(xg + (static_cast<int64_t>(item.bz) * p.m + static_cast<int64_t>(item.r[u]) * kTile) * p.k), 0,
+          rows_left * p.k * 2, 0x00020000);
+      rsrc[2 + u] = __builtin_amdgcn_make_buffer_rsrc(
+          const_cast<T*>(wg + static_cast<int64_t>(item.c[u]) * kTile * p.k), 0, kTile * p.k * 2, 0x00020000);
+    }
+  };
+  int ld_off[4];
+#pragma unroll
+  for (int jj = 0; jj < 4; ++jj) ld_off[jj] = (32 * wv + 8 * jj + (lane >> 3)) * p.k * 2 + ld_chunk * 16;
+  // Staging registers: piece j of a slab waits here between its global load and its LDS write.
+  u32x4 stg[P];
+  auto gload = [&](int j, int entry) {
+    const int t = j >> 2;  // tiles 0, 1: X of token block 0, 1 (select bits 16, 17 of the entry); 2, 3: W
+    const bool sel = t >= 2 || ((entry >> (16 + t)) & 1) != 0;
+    stg[j] = __builtin_amdgcn_raw_buffer_load_b128(sel ? rsrc[t] : rsrc_none, ld_off[j & 3], (entry & 0xFFFF) * 2, 0);
+  };
+  // kHalf: only one half of a slab that reaches into its neighbour counts; the other half of the X
+  // pieces is cleared on the way to LDS
+  auto keep_of = [&](int entry) -> unsigned {
+    return (entry & kZeroFirst) ? ~mask_first : ((entry & kZeroSecond) ? mask_first : 0xFFFFFFFFu);
+  };
+  auto lwrite = [&](int j, int stage, unsigned keep) {
+    const int t = j >> 2;
+    uint8_t* dst = smem + stage * kStageBytes + t * kUnitBytes + (32 * wv + 8 * (j & 3)) * kRowBytes + wr_off[j & 1];
+    u32x4 v = stg[j];
+    if constexpr (kHalf) {
+      if (t < 2) v &= keep;
+    }
+    *reinterpret_cast<u32x4*>(dst) = v;
+  };
+
+  // The first slab of an item is requested before the epilogue of the item before it, so that its
+  // latency (and the list work above) hides behind the stores.
+  int work = slot;
+  bool have = work < q_len;
+  Item cur{};
+  if (have) {
+    cur = decode_item(work);
+    n_iter = build_steps(cur);
+    make_rsrc(cur);
+    if (n_iter > 0) {
+      const int e0 = step_entry(0);
+#pragma unroll
+      for (int j = 0; j < P; ++j) gload(j, e0);
+    }
+  }
+  while (have) {
+    const int bz = cur.bz, valid = cur.valid;
+    // (no indexing by a run-time value: the item has to stay in scalar registers)
+    const int out_r = wr ? cur.r[1] : cur.r[0], out_c = wc ? cur.c[1] : cur.c[0];
+    const bool my_valid = (valid >> (wr * 2 + wc)) & 1;
+    // (the next item is looked up here, while no accumulator is live)
+    const int next_work = work + per_xcd;
+    const bool have_next = next_work < q_len;
+    Item nxt{};
+    if (have_next) nxt = decode_item(next_work);
+    // every wavefront is done with the ring (the previous item's epilogue turned through it)
+    __builtin_amdgcn_s_waitcnt(0xc07f);  // lgkmcnt(0)
+    __builtin_amdgcn_s_barrier();
 
     // ---- pipeline ----
     // Two slab buffers in LDS (stage it % 2 holds slab it) and one slab in flight in the staging
-    // registers.  Iteration it: substeps 0..2 of slab it run while pieces 4..15 of slab it+1 go from
-    // the staging registers into the other stage and the same pieces of slab it+2 are requested; one
-    // barrier (every wavefront has read all of slab it and written all of slab it+1); substep 3 runs
-    // while the first operands of slab it+1 are read, pieces 0..3 of slab it+2 go into stage it % 2
-    // and those of slab it+3 are requested.  Every substep issues the same mix: sixteen MFMAs, eight
-    // operand reads, four LDS writes, four global loads, so the memory path sees an even stream and
-    // a load has a whole slab period to arrive.
+    // registers.  Iteration it: substeps 0..2 of slab it run while the last three quarters of the
+    // pieces of slab it+1 go from the staging registers into the other stage and the same pieces of
+    // slab it+2 are requested; one barrier (every wavefront has read all of slab it and written all of
+    // slab it+1); substep 3 runs while the first operands of slab it+1 are read, the first quarter of
+    // slab it+2 goes into stage it % 2 and that of slab it+3 is requested.  Every substep issues the
+    // same mix (sixteen MFMAs, eight operand reads, four LDS writes, four global loads), so the memory
+    // path sees an even stream and a load has a whole slab period to arrive.
     if (n_iter > 0) {
       const int e0 = step_entry(0), e1 = step_entry(1), e2 = step_entry(2);
-#pragma unroll
-      for (int j = 0; j < 16; ++j) gload(j, e0);
       {
         const unsigned keep = keep_of(e0);
 #pragma unroll
-        for (int j = 0; j < 16; ++j) lwrite(j, 0, keep);
+        for (int j = 0; j < P; ++j) lwrite(j, 0, keep);
       }
 #pragma unroll
-      for (int j = 0; j < 16; ++j) gload(j, e1);
+      for (int j = 0; j < P; ++j) gload(j, e1);
       {
         const unsigned keep = keep_of(e1);
 #pragma unroll
-        for (int j = 0; j < 4; ++j) lwrite(j, 1, keep);
+        for (int j = 0; j < PS; ++j) lwrite(j, 1, keep);
       }
 #pragma unroll
-      for (int j = 0; j < 4; ++j) gload(j, e2);
+      for (int j = 0; j < PS; ++j) gload(j, e2);
       __builtin_amdgcn_s_waitcnt(0xc07f);  // lgkmcnt(0)
       __builtin_amdgcn_s_barrier();
     }
 
+    // ---- next item: list work and the request for its first slab (every wavefront, once per item,
+    // after its last use of the ring and of the step list).  GEMM-Q does it before the epilogue, so
+    // that the slab's latency hides behind the stores; GEMM-O after it (its list work, a scan of the
+    // flags with two barriers, would hold the stores back for longer than the request gains). ----
+    int next_iter = 0;
+    auto ring_free = [&]() {
+      __builtin_amdgcn_s_waitcnt(0xc07f);
+      __builtin_amdgcn_s_barrier();  // every wavefront is done with the ring and with the step list
+    };
+    auto prefetch_next = [&]() {
+      if (have_next) {
+        next_iter = build_steps(nxt);
+        make_rsrc(nxt);
+        if (next_iter > 0) {
+          const int saved = n_iter;
+          n_iter = next_iter;  // (step_entry of the listless form clamps against it)
+          const int e0 = step_entry(0);
+          n_iter = saved;
+#pragma unroll
+          for (int j = 0; j < P; ++j) gload(j, e0);
+        }
+      }
+    };
+    // ---- accumulators (bias / cached partial are added in the epilogue) ----
+    // acc[nt][mt][i]: n = n0 + nt*32 + (i/4)*8 + g*4 + i%4, m = m0 + mt*32 + l32
+    const int m0 = out_r * kTile;
+    const int n0 = out_c * kTile;
+    f32x16 acc[NT][MT];
     if (!my_valid) {
       // This wavefront's unit does not exist in this quad (unflagged, or past the matrix edge): it
       // only moves its pieces and keeps the barrier sequence of the others.
@@ -599,92 +682,90 @@ __global__ void __launch_bounds__(kThreads) gemm_kernel(const GemmParams p) {
         const int en1 = step_entry(it + 1), en2 = step_entry(it + 2), en3 = step_entry(it + 3);
         const unsigned keep1 = keep_of(en1), keep2 = keep_of(en2);
 #pragma unroll
-        for (int j = 4; j < 16; ++j) {
+        for (int j = PS; j < P; ++j) {
           lwrite(j, st ^ 1, keep1);
           gload(j, en2);
         }
         __builtin_amdgcn_s_waitcnt(0xc07f);
         __builtin_amdgcn_s_barrier();
 #pragma unroll
-        for (int j = 0; j < 4; ++j) {
+        for (int j = 0; j < PS; ++j) {
           lwrite(j, st, keep2);
           gload(j, en3);
         }
       }
+      ring_free();
+      prefetch_next();
+    } else {
+#pragma unroll
+      for (int nt = 0; nt < NT; ++nt)
+#pragma unroll
+        for (int mt = 0; mt < MT; ++mt)
+#pragma unroll
+          for (int i = 0; i < 16; ++i) acc[nt][mt][i] = 0.f;
       if (n_iter > 0) {
-        __builtin_amdgcn_s_waitcnt(0xc07f);
-        __builtin_amdgcn_s_barrier();  // the others' "ring is free" barrier before their epilogue
-      }
-      continue;
-    }
-
-    // ---- accumulators (bias / cached partial are added in the epilogue) ----
-    // acc[nt][mt][i]: n = n0 + nt*32 + (i/4)*8 + g*4 + i%4, m = m0 + mt*32 + l32
-    const int m0 = r[wr] * kTile;
-    const int n0 = c[wc] * kTile;
-    f32x16 acc[NT][MT];
+        // LDS byte offsets of this wavefront's operand rows inside a stage
+        const int a_base = (2 + wc) * kUnitBytes + l32 * kRowBytes;  // W rows nt*32 + l32
+        const int b_base = wr * kUnitBytes + l32 * kRowBytes;        // X rows mt*32 + l32
+        x8 a[2][NT], b[2][MT];
+        // operand read idx of substep sub of the slab in `stage` into register set sub & 1, in the order
+        // the MFMAs need them: W rows 0, all X rows, W rows 1..3
+        auto lread = [&](int stage, int sub, int idx) {
+          const uint8_t* st = smem + stage * kStageBytes;
+          const int x = rd_x ^ (sub << 5);
+          if (idx == 0) {
+            a[sub & 1][0] = *reinterpret_cast<const x8*>(st + a_base + x);
+          } else if (idx <= MT) {
+            b[sub & 1][idx - 1] = *reinterpret_cast<const x8*>(st + b_base + (idx - 1) * 32 * kRowBytes + x);
+          } else {
+            a[sub & 1][idx - MT] = *reinterpret_cast<const x8*>(st + a_base + (idx - MT) * 32 * kRowBytes + x);
+          }
+        };
+        // one substep: the MFMAs of register set `set`; in their shadow the operand reads of substep
+        // rsub of the slab in rstage, and pieces j0..j0+3: staged -> LDS stage wstage, then the same
+        // pieces of the slab with entry `lentry` -> staging
+        auto substep = [&](int set, int rstage, int rsub, int wstage, int j0, unsigned keep, int lentry) {
 #pragma unroll
-    for (int nt = 0; nt < NT; ++nt)
+          for (int i = 0; i < NT * MT; ++i) {
+            const int nt = i / MT, mt = i % MT;
+            acc[nt][mt] = TT::mfma(a[set][nt], b[set][mt], acc[nt][mt]);
+            if ((i & 1) == 0) lread(rstage, rsub, i >> 1);
+            if ((i & 3) == 1) lwrite(j0 + (i >> 2), wstage, keep);
+            if ((i & 3) == 3) gload(j0 + (i >> 2), lentry);
+            __builtin_amdgcn_sched_barrier(0);
+          }
+        };
 #pragma unroll
-      for (int mt = 0; mt < MT; ++mt)
-#pragma unroll
-        for (int i = 0; i < 16; ++i) acc[nt][mt][i] = 0.f;
-
-    if (n_iter > 0) {
-      // LDS byte offsets of this wavefront's operand rows inside a stage
-      const int a_base = (2 + wc) * kUnitBytes + l32 * kRowBytes;  // W rows nt*32 + l32
-      const int b_base = wr * kUnitBytes + l32 * kRowBytes;        // X rows mt*32 + l32
-      x8 a[2][NT], b[2][MT];
-      // operand read idx of substep sub of the slab in `stage` into register set sub & 1, in the order
-      // the MFMAs need them: W rows 0, X rows 0..3, W rows 1..3
-      auto lread = [&](int stage, int sub, int idx) {
-        const uint8_t* st = smem + stage * kStageBytes;
-        const int x = rd_x ^ (sub << 5);
-        if (idx == 0) {
-          a[sub & 1][0] = *reinterpret_cast<const x8*>(st + a_base + x);
-        } else if (idx <= MT) {
-          b[sub & 1][idx - 1] = *reinterpret_cast<const x8*>(st + b_base + (idx - 1) * 32 * kRowBytes + x);
-        } else {
-          a[sub & 1][idx - MT] = *reinterpret_cast<const x8*>(st + a_base + (idx - MT) * 32 * kRowBytes + x);
+        for (int idx = 0; idx < NT + MT; ++idx) lread(0, 0, idx);
+        // (the step entries of the next three slabs ride along in scalar registers; the fourth is
+        // read from the list a slab ahead and becomes scalar after the wait the barrier needs anyway,
+        // so the list costs no wait of its own)
+        int en1 = step_entry(1), en2 = step_entry(2), en3 = step_entry(3);
+        for (int it = 0; it < n_iter; ++it) {
+          const int st = it & 1;
+          const int en4_raw = step_entry_raw(it + 4);
+          const unsigned keep1 = keep_of(en1), keep2 = keep_of(en2);
+          substep(0, st, 1, st ^ 1, PS, keep1, en2);
+          substep(1, st, 2, st ^ 1, 2 * PS, keep1, en2);
+          substep(0, st, 3, st ^ 1, 3 * PS, keep1, en2);
+          __builtin_amdgcn_s_waitcnt(0xc07f);  // lgkmcnt(0): my reads of slab it and my writes of slab it+1 are done
+          __builtin_amdgcn_s_barrier();        // ... for every wavefront
+          const int en4 = __builtin_amdgcn_readfirstlane(en4_raw);
+          substep(1, st ^ 1, 0, st, 0, keep2, en3);
+          en1 = en2;
+          en2 = en3;
+          en3 = en4;
         }
-      };
-      // one substep: the sixteen MFMAs of register set `set`; in their shadow the eight operand reads
-      // of substep rsub of the slab in rstage, and pieces j0..j0+3: staged -> LDS stage wstage, then the
-      // same pieces of the slab with entry `lentry` -> staging
-      auto substep = [&](int set, int rstage, int rsub, int wstage, int j0, unsigned keep, int lentry) {
-#pragma unroll
-        for (int i = 0; i < NT * MT; ++i) {
-          const int nt = i / MT, mt = i % MT;
-          acc[nt][mt] = TT::mfma(a[set][nt], b[set][mt], acc[nt][mt]);
-          if ((i & 1) == 0) lread(rstage, rsub, i >> 1);
-          if ((i & 3) == 1) lwrite(j0 + (i >> 2), wstage, keep);
-          if ((i & 3) == 3) gload(j0 + (i >> 2), lentry);
-          __builtin_amdgcn_sched_barrier(0);
-        }
-      };
-#pragma unroll
-      for (int idx = 0; idx < NT + MT; ++idx) lread(0, 0, idx);
-      for (int it = 0; it < n_iter; ++it) {
-        const int st = it & 1;
-        const int en1 = step_entry(it + 1), en2 = step_entry(it + 2), en3 = step_entry(it + 3);
-        const unsigned keep1 = keep_of(en1), keep2 = keep_of(en2);
-        substep(0, st, 1, st ^ 1, 4, keep1, en2);
-        substep(1, st, 2, st ^ 1, 8, keep1, en2);
-        substep(0, st, 3, st ^ 1, 12, keep1, en2);
-        __builtin_amdgcn_s_waitcnt(0xc07f);  // lgkmcnt(0): my reads of slab it and my writes of slab it+1 are done
-        __builtin_amdgcn_s_barrier();        // ... for every wavefront
-        substep(1, st ^ 1, 0, st, 0, keep2, en3);
       }
-      __builtin_amdgcn_s_waitcnt(0xc07f);
-      __builtin_amdgcn_s_barrier();  // every wavefront is done with the ring
-    }
+      ring_free();
+      if constexpr (!kReduce) prefetch_next();
 
     // ---- epilogue ----
     // In the accumulator layout a lane owns one output row and runs of four columns: written from
     // there, a store instruction is 64 scattered 8-byte pieces (measured: ~12 % of the FLUX-sized
     // launches; the bias matrix read the same way, as much again).  Each wavefront therefore turns
-    // its 128 x 128 block through its own quarter of the ring, 32 rows at a time in fp32, and adds the
-    // bias and stores from a layout in which 32 consecutive lanes cover one row.
+    // its block through its own quarter of the ring, 32 rows at a time in fp32, and adds the bias and
+    // stores from a layout in which 32 consecutive lanes cover one row.
     {
       // (the lane index is made opaque: otherwise the per-lane address terms are computed once per
       // kernel, spilled, and every reload waits for the store before it)
@@ -699,8 +780,8 @@ __global__ void __launch_bounds__(kThreads) gemm_kernel(const GemmParams p) {
       // being kept: the bias is added for good after the turn below); scale = absmax / 448 (1 for a
       // zero slab).
       float qscale = 1.f;
-      if constexpr (!kReduce) {
-        if (p.y8) {
+      if constexpr (kQuant) {
+        {
           const bool has_vec = p.bias_kind == FO_BIAS_VECTOR;
           float amax = 0.f;
 #pragma unroll
@@ -724,7 +805,7 @@ __global__ void __launch_bounds__(kThreads) gemm_kernel(const GemmParams p) {
           for (int off = 32; off > 0; off >>= 1) amax = fmaxf(amax, __shfl_xor(amax, off, 64));
           qscale = amax > 0.f ? amax / 448.0f : 1.0f;
           if (lane == 0)
-            p.y_scale[static_cast<int64_t>(c[wc]) * p.scale_row_len + bz * p.n_row_tiles + r[wr]] = qscale;
+            p.y_scale[static_cast<int64_t>(out_c) * p.scale_row_len + bz * p.n_row_tiles + out_r] = qscale;
         }
       }
       if (p.bias_kind == FO_BIAS_VECTOR) {
@@ -789,8 +870,8 @@ __global__ void __launch_bounds__(kThreads) gemm_kernel(const GemmParams p) {
               for (int j = 0; j < 4; ++j) out[j] = static_cast<T>(v[j]);
               *reinterpret_cast<x4*>(static_cast<T*>(p.y) + off) = out;
             }
-            if constexpr (!kReduce) {
-              if (p.y8) {
+            if constexpr (kQuant) {
+              {
                 float f[4];
 #pragma unroll
                 for (int j = 0; j < 4; ++j) f[j] = fminf(fmaxf(v[j] / qscale, -448.0f), 448.0f);
@@ -820,6 +901,12 @@ __global__ void __launch_bounds__(kThreads) gemm_kernel(const GemmParams p) {
         for (int mt = 0; mt < MT; ++mt) turn_half(mt, T{});
       }
     }
+      if constexpr (kReduce) prefetch_next();
+    }
+    cur = nxt;
+    n_iter = next_iter;
+    work = next_work;
+    have = have_next;
   }
 }
 
@@ -840,7 +927,7 @@ int64_t workspace_ints(const ListGeom& gm, int64_t* max_quads_out) {
   return 16 + kQuadInts * max_quads;
 }
 
-template <typename T, bool kReduce, bool kHalf>
+template <typename T, bool kReduce, bool kHalf, bool kQuant>
 int launch_half(GemmParams& p, const ListGeom& gm, bool use_flags, void* workspace, hipStream_t stream) {
   // (the attribute belongs to the kernel's code object on one device: set once per device; the flags
   // are atomic because host threads may launch concurrently, and setting it twice is harmless)
@@ -848,7 +935,7 @@ int launch_half(GemmParams& p, const ListGeom& gm, bool use_flags, void* workspa
   int dev = 0;
   FO_HIP_CALL(hipGetDevice(&dev));
   if (dev < 0 || dev >= 64 || !attr_set[dev].load(std::memory_order_acquire)) {
-    FO_HIP_CALL(hipFuncSetAttribute(reinterpret_cast<const void*>(&gemm_kernel<T, kReduce, kHalf>),
+    FO_HIP_CALL(hipFuncSetAttribute(reinterpret_cast<const void*>(&gemm_kernel<T, kReduce, kHalf, kQuant>),
                                     hipFuncAttributeMaxDynamicSharedMemorySize, kSmemBytes));
     if (dev >= 0 && dev < 64) attr_set[dev].store(true, std::memory_order_release);
   }
@@ -869,7 +956,7 @@ int launch_half(GemmParams& p, const ListGeom& gm, bool use_flags, void* workspa
     // every unit is computed: no list, the kernel enumerates the quads itself
     p.quads = nullptr;
     p.qoff = nullptr;
-    gemm_kernel<T, kReduce, kHalf><<<static_cast<unsigned>(grid), kThreads, kSmemBytes, stream>>>(p);
+    gemm_kernel<T, kReduce, kHalf, kQuant><<<static_cast<unsigned>(grid), kThreads, kSmemBytes, stream>>>(p);
     FO_CHECK_LAUNCH();
     return FO_OK;
   }
@@ -879,7 +966,7 @@ int launch_half(GemmParams& p, const ListGeom& gm, bool use_flags, void* workspa
     p.quads = nullptr;
     p.qoff = nullptr;
     p.inline_cells = static_cast<int32_t>(n_cells);
-    gemm_kernel<T, kReduce, kHalf><<<static_cast<unsigned>(grid), kThreads, kSmemBytes, stream>>>(p);
+    gemm_kernel<T, kReduce, kHalf, kQuant><<<static_cast<unsigned>(grid), kThreads, kSmemBytes, stream>>>(p);
     FO_CHECK_LAUNCH();
     return FO_OK;
   }
@@ -897,7 +984,7 @@ int launch_half(GemmParams& p, const ListGeom& gm, bool use_flags, void* workspa
   FO_CHECK_LAUNCH();
   p.quads = quads;
   p.qoff = qoff;
-  gemm_kernel<T, kReduce, kHalf><<<static_cast<unsigned>(grid), kThreads, kSmemBytes, stream>>>(p);
+  gemm_kernel<T, kReduce, kHalf, kQuant><<<static_cast<unsigned>(grid), kThreads, kSmemBytes, stream>>>(p);
   FO_CHECK_LAUNCH();
   return FO_OK;
 }
@@ -907,8 +994,13 @@ int launch_half(GemmParams& p, const ListGeom& gm, bool use_flags, void* workspa
 template <typename T, bool kReduce>
 int launch(GemmParams& p, const ListGeom& gm, bool use_flags, void* workspace, hipStream_t stream) {
   const bool half = (kReduce ? p.head_dim : p.k) % kBK != 0;
-  return half ? launch_half<T, kReduce, true>(p, gm, use_flags, workspace, stream)
-              : launch_half<T, kReduce, false>(p, gm, use_flags, workspace, stream);
+  if constexpr (!kReduce) {
+    if (p.y8)  // fused quantisation: its own instantiation, so that the plain kernel does not carry its registers
+      return half ? launch_half<T, kReduce, true, true>(p, gm, use_flags, workspace, stream)
+                  : launch_half<T, kReduce, false, true>(p, gm, use_flags, workspace, stream);
+  }
+  return half ? launch_half<T, kReduce, true, false>(p, gm, use_flags, workspace, stream)
+              : launch_half<T, kReduce, false, false>(p, gm, use_flags, workspace, stream);
 }
 
 int check_common(const void* x, const void* w, void* y, int dtype, int32_t batch, int32_t m,
