@@ -783,24 +783,41 @@ __global__ void __launch_bounds__(kThreads) gemm_kernel(const GemmParams p) {
       if constexpr (kQuant) {
         {
           const bool has_vec = p.bias_kind == FO_BIAS_VECTOR;
+          // all sixteen bias pieces requested before the first is used
+          x4 bvs[NT * 4];
+#pragma unroll
+          for (int i = 0; i < NT * 4; ++i)
+#pragma unroll
+            for (int j = 0; j < 4; ++j) bvs[i][j] = static_cast<T>(0.f);
+          if (has_vec) {
+#pragma unroll
+            for (int nt = 0; nt < NT; ++nt)
+#pragma unroll
+              for (int i4 = 0; i4 < 4; ++i4)
+                bvs[nt * 4 + i4] = *reinterpret_cast<const x4*>(static_cast<const T*>(p.bias) + n0 + nt * 32 +
+                                                                i4 * 8 + wg * 4);
+          }
+          __builtin_amdgcn_sched_barrier(0);
           float amax = 0.f;
 #pragma unroll
-          for (int nt = 0; nt < NT; ++nt)
+          for (int nt = 0; nt < NT; ++nt) {
 #pragma unroll
             for (int i4 = 0; i4 < 4; ++i4) {
-              float bq[4] = {0.f, 0.f, 0.f, 0.f};
-              if (has_vec) {
-                const x4 bv = *reinterpret_cast<const x4*>(static_cast<const T*>(p.bias) + n0 + nt * 32 + i4 * 8 + wg * 4);
-#pragma unroll
-                for (int j = 0; j < 4; ++j) bq[j] = static_cast<float>(bv[j]);
-              }
 #pragma unroll
               for (int mt = 0; mt < MT; ++mt)
                 if (m0 + mt * 32 + wl32 < p.m) {
 #pragma unroll
-                  for (int j = 0; j < 4; ++j) amax = fmaxf(amax, fabsf(acc[nt][mt][i4 * 4 + j] + bq[j]));
+                  for (int j = 0; j < 4; ++j) {
+                    // (an opaque copy: otherwise the copies read out of the accumulator registers here
+                    // are kept for the turn below, and spilled)
+                    float v = acc[nt][mt][i4 * 4 + j];
+                    asm volatile("" : "+v"(v));
+                    amax = fmaxf(amax, fabsf(v + static_cast<float>(bvs[nt * 4 + i4][j])));
+                  }
                 }
             }
+            __builtin_amdgcn_sched_barrier(0);  // (quarter by quarter: taken together they do not fit the registers)
+          }
 #pragma unroll
           for (int off = 32; off > 0; off >>= 1) amax = fmaxf(amax, __shfl_xor(amax, off, 64));
           qscale = amax > 0.f ? amax / 448.0f : 1.0f;
