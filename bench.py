@@ -409,9 +409,10 @@ def main():
     c2["gemm_o_cache"] = entry(time_gpu(layer.gemm_o_cache, K, W), flops=layer.w2.gemm_o_flops(True))
     c2["gemm_o_final"] = entry(time_gpu(layer.gemm_o_final, K, W), flops=layer.w2.gemm_o_flops(False))
     kernels[layer.w2.shape.name] = c2
-    # packbits at the config-0 mask size and at 16 Mi flags
+    # packbits at the config-0 mask size, at 16 Mi flags (both bounded by the host's call rate: the
+    # kernel is shorter than a call) and at 256 Mi flags (bounded by HBM)
     pk = {}
-    for n in (31104, 1 << 24):
+    for n in (31104, 1 << 24, 1 << 28):
         xb = (torch.rand(n, device=dev) < 0.5)
         pk["n=%d" % n] = entry(time_gpu(lambda: layer.fo.packbits(xb, "little"), K, W), nbytes=n + n // 8)
     kernels["packbits"] = pk
