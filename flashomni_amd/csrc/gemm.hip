@@ -773,7 +773,6 @@ __global__ void __launch_bounds__(kThreads) gemm_kernel(const GemmParams p) {
       asm volatile("" : "+v"(ln));
       const int col4 = ln & 31, rsub = ln >> 5, wl32 = ln & 31, wg = ln >> 5;
       uint8_t* const region0 = smem + wv * (kSmemBytes / 4);
-      const int64_t y_batch = static_cast<int64_t>(bz) * p.m * p.n;
       float bvec[4] = {0.f, 0.f, 0.f, 0.f};
       // Fused quantisation (GEMM-Q): a unit is one (token block, head) slab.  Its absmax is taken
       // over the final values (accumulator + bias, formed here in the accumulator layout without
@@ -830,10 +829,21 @@ __global__ void __launch_bounds__(kThreads) gemm_kernel(const GemmParams p) {
 #pragma unroll
         for (int j = 0; j < 4; ++j) bvec[j] = static_cast<float>(bv[j]);
       }
-      // 32 rows of the block; BiasT: element type of the bias matrix, if there is one
-      auto turn_half = [&](int mt, auto bias_tag) {
+      // Output (and the cached partial, if there is one) go through buffer descriptors that end with the
+      // matrix: rows past M are dropped (read as zeros) by the address unit, no lane is masked and no
+      // row is tested.  A null output gets an empty descriptor.
+      const int rows_out = min(p.m - m0, kTile);
+      const int64_t row0 = static_cast<int64_t>(bz) * p.m + m0;
+      auto out_rsrc = [&](const void* base, int elem_bytes) {
+        return __builtin_amdgcn_make_buffer_rsrc(
+            const_cast<uint8_t*>(static_cast<const uint8_t*>(base) + row0 * p.n * elem_bytes), 0,
+            base ? rows_out * p.n * elem_bytes : 0, 0x00020000);
+      };
+      // 32 rows of the block.  kMatrix: a cached partial [B, M, N] of element type BiasT is added;
+      // kOutF32: the output is fp32
+      auto turn_half = [&](int mt, auto matrix_tag, auto bias_tag, auto f32_tag) {
+        constexpr bool kMatrix = decltype(matrix_tag)::value, kOutF32 = decltype(f32_tag)::value;
         using BiasT = decltype(bias_tag);
-        const int row_base = m0 + mt * 32;
         uint8_t* const region = region0 + (mt & 1) * (kSmemBytes / 8);
         // 16-byte chunk c of row r sits at chunk position c ^ r (rows are 512 bytes = 32 chunks)
 #pragma unroll
@@ -846,76 +856,89 @@ __global__ void __launch_bounds__(kThreads) gemm_kernel(const GemmParams p) {
             const int chunk = nt * 8 + i4 * 2 + wg;
             *reinterpret_cast<f32x4*>(region + wl32 * 512 + ((chunk ^ wl32) << 4)) = v;
           }
+        // this lane's rows are mt*32 + rsub + 2*i, its columns n0 + col4*4 .. +3: a lane offset and a
+        // scalar offset per row
+        const int el_off = n0 + col4 * 4 + rsub * p.n;  // in elements, row mt*32 + rsub
+        auto row_off = [&](int i, int elem_bytes) { return (mt * 32 + 2 * i) * p.n * elem_bytes; };
         // cached partial of these rows: all sixteen loads in flight together
         using BiasVec = typename std::conditional<sizeof(BiasT) == 4, f32x4, x4>::type;
         BiasVec bm[16];
-        const bool has_matrix = p.bias_kind == FO_BIAS_MATRIX;
-        if (has_matrix) {
+        if constexpr (kMatrix) {
+          const __amdgpu_buffer_rsrc_t rb = out_rsrc(p.bias, sizeof(BiasT));
 #pragma unroll
           for (int i = 0; i < 16; ++i) {
-            int grow = row_base + i * 2 + rsub;
-            grow = grow < p.m ? grow : p.m - 1;
-            const int64_t off = y_batch + static_cast<int64_t>(grow) * p.n + n0 + col4 * 4;
-            bm[i] = *reinterpret_cast<const BiasVec*>(static_cast<const BiasT*>(p.bias) + off);
+            if constexpr (sizeof(BiasT) == 4) {
+              bm[i] = __builtin_bit_cast(BiasVec, __builtin_amdgcn_raw_buffer_load_b128(rb, el_off * 4, row_off(i, 4), 0));
+            } else {
+              bm[i] = __builtin_bit_cast(BiasVec, __builtin_amdgcn_raw_buffer_load_b64(rb, el_off * 2, row_off(i, 2), 0));
+            }
           }
         }
-        // four rows are read back and biased before the first of them is stored (row by row, every
-        // read waited for the stores before it: one memory counter for loads and stores)
+        const __amdgpu_buffer_rsrc_t ry = out_rsrc(p.y, kOutF32 ? 4 : 2);
+        // four rows are read back and biased before the first of them is stored
         f32x4 vals[4];
 #pragma unroll
         for (int i = 0; i < 16; ++i) {
-          const int row = i * 2 + rsub;
           if ((i & 3) == 0) {  // four rows at a time
 #pragma unroll
             for (int k = 0; k < 4; ++k) {
               const int rk = (i + k) * 2 + rsub;
               vals[k] = *reinterpret_cast<const f32x4*>(region + rk * 512 + ((col4 ^ rk) << 4));
 #pragma unroll
-              for (int j = 0; j < 4; ++j) vals[k][j] += has_matrix ? static_cast<float>(bm[i + k][j]) : bvec[j];
+              for (int j = 0; j < 4; ++j) {
+                if constexpr (kMatrix) {
+                  vals[k][j] += static_cast<float>(bm[i + k][j]);
+                } else {
+                  vals[k][j] += bvec[j];
+                }
+              }
             }
             __builtin_amdgcn_sched_barrier(0);
           }
           const f32x4 v = vals[i & 3];
-          const int grow = row_base + row;
-          if (grow < p.m) {
-            const int64_t off = y_batch + static_cast<int64_t>(grow) * p.n + n0 + col4 * 4;
-            if (p.y_f32) {
-              *reinterpret_cast<f32x4*>(static_cast<float*>(p.y) + off) = v;
-            } else if (p.y) {
-              x4 out;
+          if constexpr (kOutF32) {
+            __builtin_amdgcn_raw_buffer_store_b128(__builtin_bit_cast(u32x4, v), ry, el_off * 4, row_off(i, 4), 0);
+          } else {
+            x4 out;
 #pragma unroll
-              for (int j = 0; j < 4; ++j) out[j] = static_cast<T>(v[j]);
-              *reinterpret_cast<x4*>(static_cast<T*>(p.y) + off) = out;
-            }
-            if constexpr (kQuant) {
-              {
-                float f[4];
+            for (int j = 0; j < 4; ++j) out[j] = static_cast<T>(v[j]);
+            typedef __attribute__((ext_vector_type(2))) unsigned int u32x2;
+            __builtin_amdgcn_raw_buffer_store_b64(__builtin_bit_cast(u32x2, out), ry, el_off * 2, row_off(i, 2), 0);
+          }
+          if constexpr (kQuant) {
+            float f[4];
 #pragma unroll
-                for (int j = 0; j < 4; ++j) f[j] = fminf(fmaxf(v[j] / qscale, -448.0f), 448.0f);
-                unsigned w8 = 0;
-                w8 = __builtin_amdgcn_cvt_pk_fp8_f32(f[0], f[1], w8, false);
-                w8 = __builtin_amdgcn_cvt_pk_fp8_f32(f[2], f[3], w8, true);
-                *reinterpret_cast<unsigned*>(p.y8 + off) = w8;
-                if (p.y8_lo) {
-                  typedef __attribute__((ext_vector_type(2))) float f32x2;
-                  const f32x2 h0 = __builtin_amdgcn_cvt_pk_f32_fp8(w8, false);
-                  const f32x2 h1 = __builtin_amdgcn_cvt_pk_f32_fp8(w8, true);
-                  unsigned l8 = 0;
-                  l8 = __builtin_amdgcn_cvt_pk_fp8_f32(f[0] - h0[0], f[1] - h0[1], l8, false);
-                  l8 = __builtin_amdgcn_cvt_pk_fp8_f32(f[2] - h1[0], f[3] - h1[1], l8, true);
-                  *reinterpret_cast<unsigned*>(p.y8_lo + off) = l8;
-                }
-              }
-            }
+            for (int j = 0; j < 4; ++j) f[j] = fminf(fmaxf(v[j] / qscale, -448.0f), 448.0f);
+            unsigned w8 = 0;
+            w8 = __builtin_amdgcn_cvt_pk_fp8_f32(f[0], f[1], w8, false);
+            w8 = __builtin_amdgcn_cvt_pk_fp8_f32(f[2], f[3], w8, true);
+            __builtin_amdgcn_raw_buffer_store_b32(w8, out_rsrc(p.y8, 1), el_off, row_off(i, 1), 0);
+            typedef __attribute__((ext_vector_type(2))) float f32x2;
+            const f32x2 h0 = __builtin_amdgcn_cvt_pk_f32_fp8(w8, false);
+            const f32x2 h1 = __builtin_amdgcn_cvt_pk_f32_fp8(w8, true);
+            unsigned l8 = 0;
+            l8 = __builtin_amdgcn_cvt_pk_fp8_f32(f[0] - h0[0], f[1] - h0[1], l8, false);
+            l8 = __builtin_amdgcn_cvt_pk_fp8_f32(f[2] - h1[0], f[3] - h1[1], l8, true);
+            __builtin_amdgcn_raw_buffer_store_b32(l8, out_rsrc(p.y8_lo, 1), el_off, row_off(i, 1), 0);  // (dropped if null)
           }
         }
       };
-      if (p.bias_kind == FO_BIAS_MATRIX && p.bias_f32) {
+      auto turn_all = [&](auto matrix_tag, auto bias_tag, auto f32_tag) {
 #pragma unroll
-        for (int mt = 0; mt < MT; ++mt) turn_half(mt, 0.f);
+        for (int mt = 0; mt < MT; ++mt) turn_half(mt, matrix_tag, bias_tag, f32_tag);
+      };
+      using std::false_type;
+      using std::true_type;
+      if constexpr (!kReduce) {
+        turn_all(false_type{}, T{}, false_type{});  // GEMM-Q: bias vector or none, output in the activation type
+      } else if (p.bias_kind == FO_BIAS_MATRIX) {
+        if (p.bias_f32) {
+          if (p.y_f32) turn_all(true_type{}, 0.f, true_type{}); else turn_all(true_type{}, 0.f, false_type{});
+        } else {
+          if (p.y_f32) turn_all(true_type{}, T{}, true_type{}); else turn_all(true_type{}, T{}, false_type{});
+        }
       } else {
-#pragma unroll
-        for (int mt = 0; mt < MT; ++mt) turn_half(mt, T{});
+        if (p.y_f32) turn_all(false_type{}, T{}, true_type{}); else turn_all(false_type{}, T{}, false_type{});
       }
     }
       if constexpr (kReduce) prefetch_next();
