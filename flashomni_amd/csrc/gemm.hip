@@ -875,27 +875,27 @@ __global__ void __launch_bounds__(kThreads) gemm_kernel(const GemmParams p) {
           }
         }
         const __amdgpu_buffer_rsrc_t ry = out_rsrc(p.y, kOutF32 ? 4 : 2);
-        // four rows are read back and biased before the first of them is stored
-        f32x4 vals[4];
+        // eight rows at a time are read back (two LDS latencies per turn) and biased, then stored
+        f32x4 vals[8];
 #pragma unroll
         for (int i = 0; i < 16; ++i) {
-          if ((i & 3) == 0) {  // four rows at a time
+          if ((i & 7) == 0) {
 #pragma unroll
-            for (int k = 0; k < 4; ++k) {
+            for (int k = 0; k < 8; ++k) {
               const int rk = (i + k) * 2 + rsub;
               vals[k] = *reinterpret_cast<const f32x4*>(region + rk * 512 + ((col4 ^ rk) << 4));
-#pragma unroll
-              for (int j = 0; j < 4; ++j) {
-                if constexpr (kMatrix) {
-                  vals[k][j] += static_cast<float>(bm[i + k][j]);
-                } else {
-                  vals[k][j] += bvec[j];
-                }
-              }
             }
             __builtin_amdgcn_sched_barrier(0);
           }
-          const f32x4 v = vals[i & 3];
+#pragma unroll
+          for (int j = 0; j < 4; ++j) {
+            if constexpr (kMatrix) {
+              vals[i & 7][j] += static_cast<float>(bm[i][j]);
+            } else {
+              vals[i & 7][j] += bvec[j];
+            }
+          }
+          const f32x4 v = vals[i & 7];
           if constexpr (kOutF32) {
             __builtin_amdgcn_raw_buffer_store_b128(__builtin_bit_cast(u32x4, v), ry, el_off * 4, row_off(i, 4), 0);
           } else {
