@@ -8,42 +8,51 @@
 //           (reference: gemm/w16a16/gemm_reduction.cuh:77-95, 126-160).
 //
 // Tiling.  The skip flags have a 128 x 128 granularity ("unit"), but a CU can pull only ~50-60 B/clk
-// from L2 while its matrix cores eat a 128 x 128 x 64 step in ~1000 clocks, so small workgroup
-// tiles starve.  A workgroup (8 wavefronts, two per SIMD) therefore computes a *quad*: two token
-// blocks x two column blocks that share their operand tiles (four 128 x BK tiles feed four units).
-// Every unit is owned by two wavefronts (64 rows x 128 columns each, 128 accumulators); six LDS
-// operand reads feed eight MFMAs.  A list kernel packs the flagged units of every
-// (16-token-block window, column pair) cell into quads: rows flagged in both columns pair up into
-// full quads, rows flagged in one column pair up among themselves, leftovers are merged; a 4-bit
-// mask says which units of a quad exist (the others are computed on duplicated tiles and dropped).
-// GEMM-O (and GEMM-Q with is_full) computes every unit: no list then, the kernel derives its quads
-// from the shape.  GEMM-O walks the union of the two token blocks' selected heads; a token block
-// that does not select a head gets that k step's X operand zeroed.
+// from L2 while its matrix cores eat a 128 x 128 x 64 step in ~500 clocks, so small workgroup tiles
+// starve.  A workgroup (4 wavefronts, one per SIMD, 512 registers each) therefore computes a *quad*:
+// two token blocks x two column blocks that share their operand tiles (four 128 x 64 tiles feed four
+// units).  A wavefront owns one unit: 128 x 128 accumulators (256 registers, kept in the accumulator
+// half of the register file), sixteen MFMAs per eight 128-bit operand reads.  (With eight wavefronts
+// of 64 x 128 the same loop spent a third more LDS reads per MFMA and ran 25 % slower.)  A list
+// kernel packs the flagged units of every (16-token-block window, column pair) cell into quads: rows
+// flagged in both columns pair up into full quads, rows flagged in one column pair up among
+// themselves, leftovers are merged; a 4-bit mask says which units of a quad exist (the wavefront of
+// a missing unit only moves data).  GEMM-O (and GEMM-Q with is_full) computes every unit: no list
+// then, the kernel derives its quads from the shape.  GEMM-O walks the union of the two token
+// blocks' selected heads; a token block that does not select a head reads that k step's X operand
+// as zeros.
 //
-// Data path.  Operands are staged in slabs of 64 k: a tile row is then 128 B, one whole memory line
-// (with 32-wide slabs every line crossed the L2 -> CU path twice, half of it unused each time, and
-// that path, not the matrix cores, bounded the loop).  Operand tiles go global -> LDS directly
-// (global_load_lds_dwordx4, 8 rows x 128 B per instruction) into two slab buffers: slab i is read
-// while slab i+1 lands; one barrier per slab, placed before the slab's last quarter so that the
-// copies of slab i+2 and the first operand reads of slab i+1 run in the shadow of the last MFMAs.  A
-// wavefront's copy lands on 1 KB of consecutive LDS, so rows are XOR-swizzled instead of padded: row
-// r keeps logical 16-byte chunk c at position c ^ ((r >> 1) & 7), applied on the global side; the
-// 128-bit operand reads of 16 consecutive rows then cover all 64 banks.  A k range that is not a
-// multiple of 64 (K or the head width of GEMM-O = 32 mod 64) ends in a slab that reaches 32 back into
-// its neighbour; that half of its X operand is zeroed.
+// Data path.  Operands are staged in slabs of 64 k: a tile row is then 128 B, one whole memory line.
+// A wavefront fetches its sixteen 8-row pieces of a slab with buffer loads (a resource descriptor
+// per tile in scalar registers, 32-bit lane offsets, the k offset as the scalar offset: no vector
+// address arithmetic; rows past M and unselected heads read as zeros through the descriptor's range
+// check) into staging registers one slab ahead, and writes them to LDS (two slab buffers) a slab
+// later; loads, LDS writes and operand reads are spread evenly between the MFMAs (per sixteen MFMAs:
+// eight reads, four writes, four loads), so the memory path sees an even stream and nothing queues
+// behind a burst.  (Direct global -> LDS copies need no registers but can only be issued once a
+// buffer is free, i.e. in a burst after the barrier: the issue stalls of that burst, 100-150 clocks
+// per copy and wavefront, cost a quarter of the loop.)  One barrier per slab.  Rows are XOR-swizzled
+// instead of padded: row r keeps logical 16-byte chunk c at position c ^ ((r >> 1) & 7), applied to
+// the LDS write address; the 128-bit operand reads of 16 consecutive rows then cover all 64 banks.
+// A k range that is not a multiple of 64 (K or the head width of GEMM-O = 32 mod 64) ends in a slab
+// that reaches 32 back into its neighbour; that half of its X operand is cleared on the way to LDS
+// (a separate instantiation, so that the common case carries no masking).
 //
 // The product is formed transposed (A operand = W rows, B operand = X rows): in the 32 x 32
 // accumulator layout a lane owns one output row and runs of 4 consecutive columns.  Stored (or the
 // init matrix read) from that layout, a wavefront instruction is 64 scattered 8-byte pieces, so the
-// epilogue turns each wavefront's block through its own part of the (by then free) operand ring,
+// epilogue turns each wavefront's block through its own quarter of the (by then free) slab buffers,
 // 32 rows at a time in fp32, into a layout where 32 consecutive lanes cover one row; there the bias
-// vector or the cached partial is added in fp32 and the result is rounded once and stored.
+// vector or the cached partial is added in fp32 and the result is rounded once and stored through a
+// buffer descriptor that ends with the matrix (no per-row tests).  GEMM-Q requests the first slab of
+// its next work item before the epilogue, so that its latency hides behind the stores.
 //
 // Work order.  Workgroups are persistent (one per CU).  The quad list is ordered by token window,
 // then column pair, then row pair, and XCD x (= blockIdx % 8) owns the x-th contiguous eighth of it.
 // The ~32 workgroups of an XCD therefore work at the same time on one token window and four
 // neighbouring column pairs (16 + 8 operand tiles for 32 quads), whose tiles they share through
-// that XCD's L2.
+// that XCD's L2; work items of equal length keep them in step in k, which is what makes the tiles
+// hit (measured at the Wan size: 6.8 GB fetched per launch against 28 GB of operand loads).
 #include "fo_common.h"
 
 #include <type_traits>
@@ -57,8 +66,6 @@ typedef __attribute__((ext_vector_type(4))) _Float16 f16x4;
 typedef __attribute__((ext_vector_type(16))) float f32x16;
 typedef __attribute__((ext_vector_type(4))) float f32x4;
 typedef __attribute__((ext_vector_type(4))) unsigned int u32x4;
-typedef __attribute__((address_space(3))) void lds_void;
-typedef __attribute__((address_space(1))) const void glb_void;
 
 constexpr int kThreads = 256;
 constexpr int kTile = 128;  // unit edge = granularity of the skip flags
@@ -122,11 +129,6 @@ struct GemmParams {
   float* y_scale;
   int32_t scale_row_len;
 };
-
-// 64 lanes x 16 bytes, global -> LDS at lds_base + lane*16 (lds_base is wavefront-uniform)
-__device__ __forceinline__ void copy16_to_lds(const void* gsrc, uint8_t* lds_base) {
-  __builtin_amdgcn_global_load_lds((glb_void*)gsrc, (lds_void*)lds_base, 16, 0, 0);
-}
 
 __device__ __forceinline__ bool flag_bit(const uint8_t* info, uint32_t bit) {
   return (info[bit >> 3] >> (bit & 7)) & 1;
@@ -303,7 +305,6 @@ __global__ void __launch_bounds__(kThreads) gemm_kernel(const GemmParams p) {
   __shared__ uint32_t s_cell_mask[kReduce ? 1 : 2 * kInlineCells];
   __shared__ int32_t s_cell_wave[kThreads / 64];
   __shared__ int32_t s_entry[8];
-  __shared__ float s_amax[kThreads / 64];
 
   const int tid = threadIdx.x, lane = tid & 63;
   const int wv = __builtin_amdgcn_readfirstlane(tid >> 6);  // wavefront index = unit of the quad, kept scalar
