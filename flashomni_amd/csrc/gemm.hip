@@ -44,8 +44,11 @@
 // epilogue turns each wavefront's block through its own quarter of the (by then free) slab buffers,
 // 32 rows at a time in fp32, into a layout where 32 consecutive lanes cover one row; there the bias
 // vector or the cached partial is added in fp32 and the result is rounded once and stored through a
-// buffer descriptor that ends with the matrix (no per-row tests).  GEMM-Q requests the first slab of
-// its next work item before the epilogue, so that its latency hides behind the stores.
+// buffer descriptor that ends with the matrix (no per-row tests).  The first slab of the next work
+// item is requested before the epilogue, so that its latency hides behind the stores (GEMM-O: the
+// item's flags are fetched a whole item ahead and its k-step list is built just before that request;
+// where a cached partial is added, the request follows the stores, because the partial's pieces need
+// the staging registers).
 //
 // Work order.  Workgroups are persistent (one per CU).  The quad list is ordered by token window,
 // then column pair, then row pair, and XCD x (= blockIdx % 8) owns the x-th contiguous eighth of it.
@@ -285,10 +288,12 @@ __global__ void __launch_bounds__(kListThreads) gemm_quads_kernel(ListArgs a, Li
 }
 
 // ---------------------------------------------------------------------------------------------
-// Main kernel.  kReduce = false: GEMM-Q.  kReduce = true: GEMM-O.
+// Main kernel.  kReduce = false: GEMM-Q.  kReduce = true: GEMM-O.  kAux: GEMM-Q with fused
+// quantisation / GEMM-O that adds a cached partial (epilogues with register needs of their own).
 // ---------------------------------------------------------------------------------------------
-template <typename T, bool kReduce, bool kHalf, bool kQuant>
+template <typename T, bool kReduce, bool kHalf, bool kAux>
 __global__ void __launch_bounds__(kThreads) gemm_kernel(const GemmParams p) {
+  constexpr bool kQuant = !kReduce && kAux, kPartial = kReduce && kAux;
   using TT = Types<T>;
   using x8 = typename TT::x8;
   using x4 = typename TT::x4;
@@ -477,7 +482,43 @@ __global__ void __launch_bounds__(kThreads) gemm_kernel(const GemmParams p) {
   };
   // k-step list of an item (GEMM-O: the union of the two token blocks' selected heads); returns the
   // number of slabs.  Called by all threads together, when nobody reads the previous list any more.
-  auto build_steps = [&](const Item& item) -> int {
+  // GEMM-O: the flags of an item's two token blocks, fetched by the first wavefront (lane = head, two
+  // bits per group of 64 heads; up to 128 heads travel this way, more are read when the list is built).
+  // Asked for at the top of the item before, so that the two dependent memory latencies (segment
+  // offset, flag byte) pass behind that item's main loop.
+  constexpr int kFetchedHeads = 128;
+  int seg_bz = -1, seg_off = 0;
+  auto fetch_flags = [&](const Item& item) -> uint32_t {
+    uint32_t f = 0;
+    if constexpr (kReduce) {
+      const int n_slices = p.k / p.head_dim;
+      if (wv == 0 && n_slices <= kFetchedHeads) {
+        // (the segment offset of the batch entry is kept: one memory latency less on the way to the flags)
+        if (item.bz != seg_bz) {
+          seg_bz = item.bz;
+          seg_off = p.sparse_info_indptr[item.bz];
+        }
+        const uint8_t* info = p.sparse_info + seg_off;
+        const uint32_t base0 =
+            static_cast<uint32_t>(p.num_text_tokens + item.r[0] * kTile) / p.sparse_q_size * p.num_heads;
+        const uint32_t base1 =
+            static_cast<uint32_t>(p.num_text_tokens + item.r[1] * kTile) / p.sparse_q_size * p.num_heads;
+        const bool want1 = (item.valid & 0xC) != 0;
+        const bool pick = p.flag == 0;  // final pass picks bit 1, cache pass bit 0
+#pragma unroll
+        for (int g = 0; g < kFetchedHeads / 64; ++g) {
+          const int h = g * 64 + lane;
+          if (h < n_slices) {
+            const uint32_t s0 = flag_bit(info, base0 + h) == pick ? 1u : 0u;
+            const uint32_t s1 = want1 && (flag_bit(info, base1 + h) == pick) ? 2u : 0u;
+            f |= (s0 | s1) << (2 * g);
+          }
+        }
+      }
+    }
+    return f;
+  };
+  auto build_steps = [&](const Item& item, uint32_t fetched) -> int {
     const int bz = item.bz, valid = item.valid;
     const int r[2] = {item.r[0], item.r[1]};
     int n_iter;
@@ -492,10 +533,15 @@ __global__ void __launch_bounds__(kThreads) gemm_kernel(const GemmParams p) {
         const bool pick = p.flag == 0;  // final pass picks bit 1, cache pass bit 0
         int count = 0;
         const int n_slices = p.k / p.head_dim;
+        const bool have_fetched = n_slices <= kFetchedHeads;
         for (int h0 = 0; h0 < n_slices; h0 += 64) {
           const int h = h0 + lane;
           bool s0 = false, s1 = false;
-          if (h < n_slices) {
+          if (have_fetched) {
+            const uint32_t two = fetched >> (2 * (h0 >> 6));
+            s0 = (two & 1) != 0;
+            s1 = (two & 2) != 0;
+          } else if (h < n_slices) {
             s0 = flag_bit(info, base0 + h) == pick;
             s1 = want1 && (flag_bit(info, base1 + h) == pick);
           }
@@ -596,7 +642,7 @@ __global__ void __launch_bounds__(kThreads) gemm_kernel(const GemmParams p) {
   Item cur{};
   if (have) {
     cur = decode_item(work);
-    n_iter = build_steps(cur);
+    n_iter = build_steps(cur, fetch_flags(cur));
     make_rsrc(cur);
     if (n_iter > 0) {
       const int e0 = step_entry(0);
@@ -613,7 +659,11 @@ __global__ void __launch_bounds__(kThreads) gemm_kernel(const GemmParams p) {
     const int next_work = work + per_xcd;
     const bool have_next = next_work < q_len;
     Item nxt{};
-    if (have_next) nxt = decode_item(next_work);
+    uint32_t nxt_flags = 0;
+    if (have_next) {
+      nxt = decode_item(next_work);
+      nxt_flags = fetch_flags(nxt);
+    }
     // every wavefront is done with the ring (the previous item's epilogue turned through it)
     __builtin_amdgcn_s_waitcnt(0xc07f);  // lgkmcnt(0)
     __builtin_amdgcn_s_barrier();
@@ -648,9 +698,8 @@ __global__ void __launch_bounds__(kThreads) gemm_kernel(const GemmParams p) {
     }
 
     // ---- next item: list work and the request for its first slab (every wavefront, once per item,
-    // after its last use of the ring and of the step list).  GEMM-Q does it before the epilogue, so
-    // that the slab's latency hides behind the stores; GEMM-O after it (its list work, a scan of the
-    // flags with two barriers, would hold the stores back for longer than the request gains). ----
+    // after its last use of the ring and of the step list, before the epilogue: the slab's latency
+    // hides behind the stores). ----
     int next_iter = 0;
     auto ring_free = [&]() {
       __builtin_amdgcn_s_waitcnt(0xc07f);
@@ -658,7 +707,7 @@ __global__ void __launch_bounds__(kThreads) gemm_kernel(const GemmParams p) {
     };
     auto prefetch_next = [&]() {
       if (have_next) {
-        next_iter = build_steps(nxt);
+        next_iter = build_steps(nxt, nxt_flags);
         make_rsrc(nxt);
         if (next_iter > 0) {
           const int saved = n_iter;
@@ -759,7 +808,10 @@ __global__ void __launch_bounds__(kThreads) gemm_kernel(const GemmParams p) {
         }
       }
       ring_free();
-      if constexpr (!kReduce) prefetch_next();
+      // The request for the next item's first slab goes out before the epilogue and its data waits in
+      // the staging registers, except where the epilogue adds a cached partial: its pieces need those
+      // registers, so there the request follows the stores.
+      if constexpr (!kPartial) prefetch_next();
 
     // ---- epilogue ----
     // In the accumulator layout a lane owns one output row and runs of four columns: written from
@@ -842,9 +894,27 @@ __global__ void __launch_bounds__(kThreads) gemm_kernel(const GemmParams p) {
       };
       // 32 rows of the block.  kMatrix: a cached partial [B, M, N] of element type BiasT is added;
       // kOutF32: the output is fp32
-      auto turn_half = [&](int mt, auto matrix_tag, auto bias_tag, auto f32_tag) {
+      // (the cached partial of 32 rows: sixteen pieces, the four values this lane adds to each of its
+      // rows, all in flight together while the rows turn through LDS.  Requesting the next 32 rows'
+      // pieces earlier, in a second register set or piece by piece as the first set is consumed, was
+      // measured: the compiler then spills 100-300 registers, some of them inside the main loop.)
+      auto load_partial = [&](int mt, auto* bm) {
+        using BiasVec = typename std::remove_reference<decltype(bm[0])>::type;
+        constexpr int kBytes = sizeof(BiasVec) / 4;  // of one element
+        const __amdgpu_buffer_rsrc_t rb = out_rsrc(p.bias, kBytes);
+        const int el_off = n0 + col4 * 4 + rsub * p.n;
+#pragma unroll
+        for (int i = 0; i < 16; ++i) {
+          const int row_off = (mt * 32 + 2 * i) * p.n * kBytes;
+          if constexpr (kBytes == 4) {
+            bm[i] = __builtin_bit_cast(BiasVec, __builtin_amdgcn_raw_buffer_load_b128(rb, el_off * 4, row_off, 0));
+          } else {
+            bm[i] = __builtin_bit_cast(BiasVec, __builtin_amdgcn_raw_buffer_load_b64(rb, el_off * 2, row_off, 0));
+          }
+        }
+      };
+      auto turn_half = [&](int mt, auto matrix_tag, auto* bm, auto f32_tag) {
         constexpr bool kMatrix = decltype(matrix_tag)::value, kOutF32 = decltype(f32_tag)::value;
-        using BiasT = decltype(bias_tag);
         uint8_t* const region = region0 + (mt & 1) * (kSmemBytes / 8);
         // 16-byte chunk c of row r sits at chunk position c ^ r (rows are 512 bytes = 32 chunks)
 #pragma unroll
@@ -861,20 +931,7 @@ __global__ void __launch_bounds__(kThreads) gemm_kernel(const GemmParams p) {
         // scalar offset per row
         const int el_off = n0 + col4 * 4 + rsub * p.n;  // in elements, row mt*32 + rsub
         auto row_off = [&](int i, int elem_bytes) { return (mt * 32 + 2 * i) * p.n * elem_bytes; };
-        // cached partial of these rows: all sixteen loads in flight together
-        using BiasVec = typename std::conditional<sizeof(BiasT) == 4, f32x4, x4>::type;
-        BiasVec bm[16];
-        if constexpr (kMatrix) {
-          const __amdgpu_buffer_rsrc_t rb = out_rsrc(p.bias, sizeof(BiasT));
-#pragma unroll
-          for (int i = 0; i < 16; ++i) {
-            if constexpr (sizeof(BiasT) == 4) {
-              bm[i] = __builtin_bit_cast(BiasVec, __builtin_amdgcn_raw_buffer_load_b128(rb, el_off * 4, row_off(i, 4), 0));
-            } else {
-              bm[i] = __builtin_bit_cast(BiasVec, __builtin_amdgcn_raw_buffer_load_b64(rb, el_off * 2, row_off(i, 2), 0));
-            }
-          }
-        }
+        if constexpr (kMatrix) load_partial(mt, bm);
         const __amdgpu_buffer_rsrc_t ry = out_rsrc(p.y, kOutF32 ? 4 : 2);
         // eight rows at a time are read back (two LDS latencies per turn) and biased, then stored
         f32x4 vals[8];
@@ -925,14 +982,17 @@ __global__ void __launch_bounds__(kThreads) gemm_kernel(const GemmParams p) {
         }
       };
       auto turn_all = [&](auto matrix_tag, auto bias_tag, auto f32_tag) {
+        using BiasT = decltype(bias_tag);
+        using BiasVec = typename std::conditional<sizeof(BiasT) == 4, f32x4, x4>::type;
+        BiasVec bm[16];
 #pragma unroll
-        for (int mt = 0; mt < MT; ++mt) turn_half(mt, matrix_tag, bias_tag, f32_tag);
+        for (int mt = 0; mt < MT; ++mt) turn_half(mt, matrix_tag, bm, f32_tag);
       };
       using std::false_type;
       using std::true_type;
       if constexpr (!kReduce) {
         turn_all(false_type{}, T{}, false_type{});  // GEMM-Q: bias vector or none, output in the activation type
-      } else if (p.bias_kind == FO_BIAS_MATRIX) {
+      } else if constexpr (kPartial) {
         if (p.bias_f32) {
           if (p.y_f32) turn_all(true_type{}, 0.f, true_type{}); else turn_all(true_type{}, 0.f, false_type{});
         } else {
@@ -942,7 +1002,7 @@ __global__ void __launch_bounds__(kThreads) gemm_kernel(const GemmParams p) {
         if (p.y_f32) turn_all(false_type{}, T{}, true_type{}); else turn_all(false_type{}, T{}, false_type{});
       }
     }
-      if constexpr (kReduce) prefetch_next();
+      if constexpr (kPartial) prefetch_next();
     }
     cur = nxt;
     n_iter = next_iter;
@@ -968,7 +1028,7 @@ int64_t workspace_ints(const ListGeom& gm, int64_t* max_quads_out) {
   return 16 + kQuadInts * max_quads;
 }
 
-template <typename T, bool kReduce, bool kHalf, bool kQuant>
+template <typename T, bool kReduce, bool kHalf, bool kAux>
 int launch_half(GemmParams& p, const ListGeom& gm, bool use_flags, void* workspace, hipStream_t stream) {
   // (the attribute belongs to the kernel's code object on one device: set once per device; the flags
   // are atomic because host threads may launch concurrently, and setting it twice is harmless)
@@ -976,7 +1036,7 @@ int launch_half(GemmParams& p, const ListGeom& gm, bool use_flags, void* workspa
   int dev = 0;
   FO_HIP_CALL(hipGetDevice(&dev));
   if (dev < 0 || dev >= 64 || !attr_set[dev].load(std::memory_order_acquire)) {
-    FO_HIP_CALL(hipFuncSetAttribute(reinterpret_cast<const void*>(&gemm_kernel<T, kReduce, kHalf, kQuant>),
+    FO_HIP_CALL(hipFuncSetAttribute(reinterpret_cast<const void*>(&gemm_kernel<T, kReduce, kHalf, kAux>),
                                     hipFuncAttributeMaxDynamicSharedMemorySize, kSmemBytes));
     if (dev >= 0 && dev < 64) attr_set[dev].store(true, std::memory_order_release);
   }
@@ -997,7 +1057,7 @@ int launch_half(GemmParams& p, const ListGeom& gm, bool use_flags, void* workspa
     // every unit is computed: no list, the kernel enumerates the quads itself
     p.quads = nullptr;
     p.qoff = nullptr;
-    gemm_kernel<T, kReduce, kHalf, kQuant><<<static_cast<unsigned>(grid), kThreads, kSmemBytes, stream>>>(p);
+    gemm_kernel<T, kReduce, kHalf, kAux><<<static_cast<unsigned>(grid), kThreads, kSmemBytes, stream>>>(p);
     FO_CHECK_LAUNCH();
     return FO_OK;
   }
@@ -1007,7 +1067,7 @@ int launch_half(GemmParams& p, const ListGeom& gm, bool use_flags, void* workspa
     p.quads = nullptr;
     p.qoff = nullptr;
     p.inline_cells = static_cast<int32_t>(n_cells);
-    gemm_kernel<T, kReduce, kHalf, kQuant><<<static_cast<unsigned>(grid), kThreads, kSmemBytes, stream>>>(p);
+    gemm_kernel<T, kReduce, kHalf, kAux><<<static_cast<unsigned>(grid), kThreads, kSmemBytes, stream>>>(p);
     FO_CHECK_LAUNCH();
     return FO_OK;
   }
@@ -1025,7 +1085,7 @@ int launch_half(GemmParams& p, const ListGeom& gm, bool use_flags, void* workspa
   FO_CHECK_LAUNCH();
   p.quads = quads;
   p.qoff = qoff;
-  gemm_kernel<T, kReduce, kHalf, kQuant><<<static_cast<unsigned>(grid), kThreads, kSmemBytes, stream>>>(p);
+  gemm_kernel<T, kReduce, kHalf, kAux><<<static_cast<unsigned>(grid), kThreads, kSmemBytes, stream>>>(p);
   FO_CHECK_LAUNCH();
   return FO_OK;
 }
@@ -1035,11 +1095,11 @@ int launch_half(GemmParams& p, const ListGeom& gm, bool use_flags, void* workspa
 template <typename T, bool kReduce>
 int launch(GemmParams& p, const ListGeom& gm, bool use_flags, void* workspace, hipStream_t stream) {
   const bool half = (kReduce ? p.head_dim : p.k) % kBK != 0;
-  if constexpr (!kReduce) {
-    if (p.y8)  // fused quantisation: its own instantiation, so that the plain kernel does not carry its registers
-      return half ? launch_half<T, kReduce, true, true>(p, gm, use_flags, workspace, stream)
-                  : launch_half<T, kReduce, false, true>(p, gm, use_flags, workspace, stream);
-  }
+  // fused quantisation (GEMM-Q) and the cached partial (GEMM-O) get instantiations of their own, so
+  // that the plain kernels do not carry their registers
+  if (kReduce ? p.bias_kind == FO_BIAS_MATRIX : p.y8 != nullptr)
+    return half ? launch_half<T, kReduce, true, true>(p, gm, use_flags, workspace, stream)
+                : launch_half<T, kReduce, false, true>(p, gm, use_flags, workspace, stream);
   return half ? launch_half<T, kReduce, true, false>(p, gm, use_flags, workspace, stream)
               : launch_half<T, kReduce, false, false>(p, gm, use_flags, workspace, stream);
 }

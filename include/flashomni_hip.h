@@ -205,7 +205,7 @@ int fo_sparse_fa_run(const void* q, const void* k, const void* v, void* o, float
  * reference demands M % 128 == 0).
  * `workspace`: device scratch of at least fo_gemm_workspace_bytes(batch, m, n) bytes, 16-byte
  * aligned; it receives the list of tile quads that the GEMM kernel walks (short launches, up to
- * 512 windows x column pairs, build the list inside the GEMM kernel and leave it untouched).
+ * 256 windows x column pairs, build the list inside the GEMM kernel and leave it untouched).
  * ------------------------------------------------------------------------------------------- */
 int64_t fo_gemm_workspace_bytes(int32_t batch, int32_t m, int32_t n);
 int fo_gemm_q(const void* x, const void* w, const void* bias, void* y, int dtype, int32_t batch,
