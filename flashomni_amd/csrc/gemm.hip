@@ -116,6 +116,7 @@ struct GemmParams {
   const int32_t* quads;  // kQuadInts per quad, queue by queue; null: every unit is computed and the
                          // quads are enumerated arithmetically (GEMM-O, GEMM-Q with is_full)
   const int32_t* qoff;   // qoff[0..8] queue boundaries inside `quads`
+  int32_t* cursor;       // GEMM-O, long launches: one work-item cursor per XCD (zero at launch), or null
   int32_t n_row_tiles, n_col_tiles, n_cp;  // geometry for the arithmetic enumeration
   int32_t n_win;         // windows of 16 token blocks per batch
   int32_t inline_cells;  // > 0: GEMM-Q builds its quad list itself from the flags of this many cells
@@ -287,6 +288,10 @@ __global__ void __launch_bounds__(kListThreads) gemm_quads_kernel(ListArgs a, Li
   }
 }
 
+// (the cursors of a launch that hands out its work items dynamically; a kernel, not a memset, so that
+// a captured graph replays it faithfully)
+__global__ void gemm_cursor_clear_kernel(int32_t* cursor) { cursor[threadIdx.x] = 0; }
+
 // ---------------------------------------------------------------------------------------------
 // Main kernel.  kReduce = false: GEMM-Q.  kReduce = true: GEMM-O.  kAux: GEMM-Q with fused
 // quantisation / GEMM-O that adds a cached partial (epilogues with register needs of their own).
@@ -299,6 +304,7 @@ __global__ void __launch_bounds__(kThreads) gemm_kernel(const GemmParams p) {
   using x4 = typename TT::x4;
   constexpr int NT = 4, MT = 4;  // wavefront tile = one unit: 128 columns (W rows) x 128 token rows (X rows)
   extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
+  __shared__ int32_t s_popped;
   __shared__ int32_t s_heads[kMaxHeads + 1];  // GEMM-O: head | (row0 selects) << 16 | (row1 selects) << 17
   __shared__ int32_t s_nsel;
   // GEMM-O: per k step, k offset | (row0 selects) << 16 | (row1 selects) << 17; four entries past
@@ -637,6 +643,18 @@ __global__ void __launch_bounds__(kThreads) gemm_kernel(const GemmParams p) {
 
   // The first slab of an item is requested before the epilogue of the item before it, so that its
   // latency (and the list work above) hides behind the stores.
+  // Work items of unequal length (GEMM-O: every item walks its own head list) let the workgroups of an
+  // XCD drift apart when each strides through the queue in fixed steps, and items that run together
+  // then no longer share tiles in L2.  Long GEMM-O launches therefore take their items from a cursor
+  // per XCD: the items in flight are always neighbours in the queue.  One thread pops, an item ahead
+  // (the value is needed at the top of the next item and waits in a register until then).
+  bool popping = false;
+  if constexpr (kReduce) popping = p.cursor != nullptr;
+  int popped = 0;
+  auto pop = [&]() {
+    if (tid == 0) popped = per_xcd + atomicAdd(p.cursor + xcd, 1);  // (the first per_xcd items are dealt by slot)
+  };
+  if (popping) pop();
   int work = slot;
   bool have = work < q_len;
   Item cur{};
@@ -656,7 +674,14 @@ __global__ void __launch_bounds__(kThreads) gemm_kernel(const GemmParams p) {
     const int out_r = wr ? cur.r[1] : cur.r[0], out_c = wc ? cur.c[1] : cur.c[0];
     const bool my_valid = (valid >> (wr * 2 + wc)) & 1;
     // (the next item is looked up here, while no accumulator is live)
-    const int next_work = work + per_xcd;
+    int next_work = work + per_xcd;
+    if (popping) {
+      if (tid == 0) s_popped = popped;
+      __builtin_amdgcn_s_waitcnt(0xc07f);
+      __builtin_amdgcn_s_barrier();
+      next_work = __builtin_amdgcn_readfirstlane(s_popped);
+      if (next_work < q_len) pop();  // for the item after the next
+    }
     const bool have_next = next_work < q_len;
     Item nxt{};
     uint32_t nxt_flags = 0;
@@ -1057,6 +1082,16 @@ int launch_half(GemmParams& p, const ListGeom& gm, bool use_flags, void* workspa
     // every unit is computed: no list, the kernel enumerates the quads itself
     p.quads = nullptr;
     p.qoff = nullptr;
+    // (cursors pay off when a workgroup sees several items; short launches keep the fixed stride and
+    // save the extra launch)
+    const int64_t items = static_cast<int64_t>(gm.batch) * gm.n_cp *
+                          (gm.n_row_tiles / kWindow * (kWindow / 2) + (gm.n_row_tiles % kWindow + 1) / 2);
+    if (kReduce && p.cursor != nullptr && items >= 4 * grid) {
+      gemm_cursor_clear_kernel<<<1, 16, 0, stream>>>(p.cursor);
+      FO_CHECK_LAUNCH();
+    } else {
+      p.cursor = nullptr;
+    }
     gemm_kernel<T, kReduce, kHalf, kAux><<<static_cast<unsigned>(grid), kThreads, kSmemBytes, stream>>>(p);
     FO_CHECK_LAUNCH();
     return FO_OK;
@@ -1233,6 +1268,10 @@ extern "C" int fo_gemm_o(const void* x, const void* w, const void* bias, void* y
   p.bias_kind = bias_kind;
   p.bias_f32 = bias_dtype == FO_F32;
   p.y_f32 = y_dtype == FO_F32;
+  // (optional workspace: room for the work-item cursors of a long launch)
+  p.cursor = workspace != nullptr && workspace_bytes >= 64 && (reinterpret_cast<uintptr_t>(workspace) & 3) == 0
+                 ? static_cast<int32_t*>(workspace)
+                 : nullptr;
   const ListGeom gm = make_geom(batch, m, n);
   hipStream_t s = static_cast<hipStream_t>(stream);
   return dtype == FO_BF16 ? launch<__bf16, true>(p, gm, false, workspace, s)

@@ -49,7 +49,7 @@ def _symbols(sparse_info, sparse_info_indptr, device, name, batch, m, num_qo_hea
     return info, indptr
 
 
-# tile-list scratch of GEMM-Q, one buffer per (device, stream): calls on one stream run in order, so
+# scratch of the GEMMs (GEMM-Q's tile list, GEMM-O's work-item cursors), one buffer per (device, stream): calls on one stream run in order, so
 # they can share it; calls on different streams may overlap and get their own
 _workspaces = {}
 
@@ -210,11 +210,15 @@ def flashomni_gemm_reduction(
     info, indptr = _symbols(sparse_info, sparse_info_indptr, A.device, "flashomni_gemm_reduction",
                             Bsz, M, num_qo_heads, num_text_tokens, sparse_q_size)
     L = _lib.lib()
-    workspace, ws_bytes = None, 0  # the reduction visits every token block: no tile list
+    # (the reduction visits every token block and needs no tile list; long launches keep their
+    # work-item cursors in the first bytes of the stream's scratch buffer)
+    stream = _lib.current_stream(A.device)
+    ws_bytes = 256
+    workspace = _gemm_workspace(A.device, stream, ws_bytes)
     with _lib.device_guard(A.device):
         _lib.check(L.fo_gemm_o(
             _lib.ptr(A), _lib.ptr(B), _lib.ptr(bias), _lib.ptr(out), _lib.dtype_code(A.dtype), kind,
             bias_code, _lib.dtype_code(out_dtype), Bsz, M, N, A.shape[2], sparse_q_size, num_qo_heads,
             _lib.ptr(info), _lib.ptr(indptr), num_text_tokens, int(bool(is_for_cache)),
-            _lib.ptr(workspace), ws_bytes, _lib.current_stream(A.device)))
+            _lib.ptr(workspace), ws_bytes, stream))
     return out

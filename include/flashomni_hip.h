@@ -224,8 +224,11 @@ int fo_gemm_q(const void* x, const void* w, const void* bias, void* y, int dtype
  *           slice selection).
  * bias_dtype: the activation dtype (as in the reference) or FO_F32 for the matrix form;
  * y_dtype: the activation dtype or FO_F32 (so a cached partial can stay in fp32).
- * hd must be a multiple of 32.  `workspace` is not used (every token block is visited, the tile
- * order is computed arithmetically) and may be NULL; fo_gemm_q with is_full != 0 likewise.
+ * hd must be a multiple of 32.  No tile list is needed (every token block is visited, the tile
+ * order is computed arithmetically), so `workspace` may be NULL; fo_gemm_q with is_full != 0
+ * likewise.  Given 64 bytes or more of 4-byte-aligned device scratch, a launch with several work
+ * items per CU hands them out through cursors kept there (work items of unequal length then stay
+ * neighbours in L2); launches that share the scratch must not overlap in time.
  * ------------------------------------------------------------------------------------------- */
 int fo_gemm_o(const void* x, const void* w, const void* bias, void* y, int dtype, int bias_kind,
               int bias_dtype, int y_dtype, int32_t batch, int32_t m, int32_t n, int32_t k,
