@@ -194,12 +194,13 @@ def flashomni_gemm_reduction(x, w, y, bias, sparse_q_size, num_qo_heads, sparse_
     if M > 0:
         need = (((num_text_tokens + M - 1) // sparse_q_size + 1) * num_qo_heads + 7) // 8
         _check(info.numel() >= need, "flashomni_gemm_reduction: sparse_info is shorter than the bits the tiles read")
+    stream = _lib.current_stream(x.device)
+    ws = _gemm_workspace(x.device, stream, 256)  # work-item cursors of a long launch
     with _lib.device_guard(x.device):
         _lib.check(_lib.lib().fo_gemm_o(
             _lib.ptr(x), _lib.ptr(w), _lib.ptr(bias), _lib.ptr(y), _lib.dtype_code(x.dtype), kind, bias_code,
             _lib.dtype_code(y.dtype), B, M, N, K, sparse_q_size, num_qo_heads, _lib.ptr(info),
-            _lib.ptr(indptr), num_text_tokens, int(bool(is_for_cached)), None, 0,
-            _lib.current_stream(x.device)))
+            _lib.ptr(indptr), num_text_tokens, int(bool(is_for_cached)), _lib.ptr(ws), 256, stream))
 
 
 # ---- bit packing -----------------------------------------------------------------------------------

@@ -362,3 +362,35 @@ def test_video_gemms_sampled_token_blocks(dev):
         got_final = final[:, r0:r1].cpu()
         assert max_abs(got_final, exp_final) <= MAX_ABS, iy
         assert rel_l2(got_final, exp_final) <= REL_L2, iy
+
+
+def test_gemm_o_cursors_and_fixed_stride_agree(dev):
+    """A long GEMM-O launch hands out its work items through cursors when it is given scratch memory and
+    in fixed strides when it is not: the order of the work items changes, no result may.  (M = 22016:
+    86 row pairs x 12 column pairs, four work items per CU; the wrapper passes scratch, the bare entry
+    point here gets none.)"""
+    import flashomni_amd as fo
+    from flashomni_amd import _lib
+    batch, m, n, heads = 1, 22016, 3072, 24
+    info, packed, indptr = _flags(batch, m // 128, heads, 0.3, seed=77)
+    g = torch.Generator(device=dev).manual_seed(78)
+    x = torch.randn(batch, m, n, generator=g, device=dev).to(torch.bfloat16)
+    w = (torch.randn(n, n, generator=g, device=dev) * 0.02).to(torch.bfloat16)
+    b = (torch.randn(n, generator=g, device=dev) * 0.02).to(torch.bfloat16)
+    pk, ip = torch.from_numpy(packed).to(dev), torch.from_numpy(indptr).to(dev)
+    code = _lib.dtype_code(torch.bfloat16)
+    for is_for_cache, bias, kind in ((True, b, _lib.FO_BIAS_VECTOR), (False, None, _lib.FO_BIAS_MATRIX)):
+        if bias is None:
+            bias = got_cache
+        got = fo.flashomni_gemm_reduction(x, w, heads, pk, ip, 0, bias=bias, is_for_cache=is_for_cache)
+        bare = torch.full_like(got, -3.0)
+        with _lib.device_guard(dev):
+            _lib.check(_lib.lib().fo_gemm_o(
+                _lib.ptr(x), _lib.ptr(w), _lib.ptr(bias), _lib.ptr(bare), code, kind, code, code, batch, m, n, n,
+                128, heads, _lib.ptr(pk), _lib.ptr(ip), 0, int(is_for_cache), None, 0, _lib.current_stream(dev)))
+        torch.cuda.synchronize()
+        assert torch.equal(got.view(torch.int16), bare.view(torch.int16))
+        got_cache = got
+    # and the end result is the dense layer
+    dense = F.linear(x[0, :256].float(), w.float(), b.float()).cpu()
+    assert rel_l2(got[0, :256].cpu(), dense) <= REL_L2
