@@ -364,15 +364,17 @@ def test_video_gemms_sampled_token_blocks(dev):
         assert rel_l2(got_final, exp_final) <= REL_L2, iy
 
 
-def test_gemm_o_cursors_and_fixed_stride_agree(dev):
+@pytest.mark.parametrize("shape", [(1, 22016, 3072, 24), (2, 43800, 768, 8)])
+def test_gemm_o_cursors_and_fixed_stride_agree(dev, shape):
     """A long GEMM-O launch hands out its work items through cursors when it is given scratch memory and
     in fixed strides when it is not: the order of the work items changes, no result may.  (M = 22016:
-    86 row pairs x 12 column pairs, four work items per CU; the wrapper passes scratch, the bare entry
-    point here gets none.)"""
+    86 row pairs x 12 column pairs, four work items per CU; the second shape has two batch entries, a
+    ragged last token block and heads of width 96, i.e. slabs that count for one half only.  The
+    wrapper passes scratch, the bare entry point here gets none.)"""
     import flashomni_amd as fo
     from flashomni_amd import _lib
-    batch, m, n, heads = 1, 22016, 3072, 24
-    info, packed, indptr = _flags(batch, m // 128, heads, 0.3, seed=77)
+    batch, m, n, heads = shape
+    info, packed, indptr = _flags(batch, (m + 127) // 128, heads, 0.3, seed=77)
     g = torch.Generator(device=dev).manual_seed(78)
     x = torch.randn(batch, m, n, generator=g, device=dev).to(torch.bfloat16)
     w = (torch.randn(n, n, generator=g, device=dev) * 0.02).to(torch.bfloat16)
