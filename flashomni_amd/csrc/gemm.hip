@@ -169,17 +169,32 @@ __device__ __forceinline__ void cell_masks(const ListGeom& gm, int cell, bool us
     return;
   }
   const uint8_t* info = sparse_info + sparse_info_indptr[b];
-  uint32_t a0 = 0, a1 = 0;
-  for (int r = 0; r < rows; ++r) {
-    const uint32_t base =
-        static_cast<uint32_t>(num_text_tokens + (w * kWindow + r) * kTile) / sparse_q_size * num_heads;
-    a0 |= static_cast<uint32_t>(flag_bit(info, base + static_cast<uint32_t>(2 * cp * kTile) / head_dim)) << r;
-    if (has1)
-      a1 |= static_cast<uint32_t>(
-                flag_bit(info, base + static_cast<uint32_t>((2 * cp + 1) * kTile) / head_dim)) << r;
+  // All flag bytes of the cell are requested before the first is looked at (rows past the end repeat
+  // the last one): one memory latency for the cell instead of one per row.
+  const uint32_t head0 = static_cast<uint32_t>(2 * cp * kTile) / head_dim;
+  const uint32_t head1 = has1 ? static_cast<uint32_t>((2 * cp + 1) * kTile) / head_dim : head0;
+  const bool unit_blocks = sparse_q_size == kTile;  // flag blocks = token blocks: no division per row
+  const uint32_t text_blocks = static_cast<uint32_t>(num_text_tokens) / kTile;
+  uint32_t bit0[kWindow], bit1[kWindow];
+  uint8_t byte0[kWindow], byte1[kWindow];
+#pragma unroll
+  for (int r = 0; r < kWindow; ++r) {
+    const int row = w * kWindow + min(r, rows - 1);
+    const uint32_t blk = unit_blocks ? text_blocks + static_cast<uint32_t>(row)
+                                     : static_cast<uint32_t>(num_text_tokens + row * kTile) / sparse_q_size;
+    bit0[r] = blk * num_heads + head0;
+    bit1[r] = blk * num_heads + head1;
+    byte0[r] = info[bit0[r] >> 3];
+    byte1[r] = info[bit1[r] >> 3];
   }
-  *m0 = a0;
-  *m1 = a1;
+  uint32_t a0 = 0, a1 = 0;
+#pragma unroll
+  for (int r = 0; r < kWindow; ++r) {
+    a0 |= ((byte0[r] >> (bit0[r] & 7)) & 1u) << r;
+    a1 |= ((byte1[r] >> (bit1[r] & 7)) & 1u) << r;
+  }
+  *m0 = a0 & all;
+  *m1 = has1 ? a1 & all : 0u;
 }
 
 __device__ __forceinline__ int pop_lowest(uint32_t* m) {
