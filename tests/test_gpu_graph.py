@@ -78,3 +78,44 @@ def test_captured_layer_pass_replays(dev):
         torch.cuda.synchronize()
         for name, a, b in zip(("gemm_q", "attention", "gemm_o"), got, (q_ref, o_ref, y_ref)):
             assert torch.equal(a, b), "replay %d: %s differs from the eager pass" % (replay, name)
+
+
+def test_captured_long_gemm_o_replays(dev):
+    """A GEMM-O launch long enough to hand out its work items through cursors (four items or more per CU):
+    the kernel that clears the cursors is captured with it, so every replay starts from zero.  Flags and
+    activations are rewritten in place between replays; each replay equals the eager call of that moment."""
+    import flashomni_amd as fo
+    m, n, heads = 22016, 3072, 24
+    g = torch.Generator(device=dev).manual_seed(9)
+    x = torch.randn(1, m, n, generator=g, device=dev).to(torch.bfloat16)
+    w = (torch.randn(n, n, generator=g, device=dev) * 0.02).to(torch.bfloat16)
+    b = (torch.randn(n, generator=g, device=dev) * 0.02).to(torch.bfloat16)
+    rng = np.random.default_rng(3)
+    bits = lambda: torch.from_numpy(rng.random((m // 128) * heads) < 0.3)
+    info = fo.packbits(bits().to(dev), "little")
+    ip = torch.tensor([0, info.numel()], dtype=torch.int32, device=dev)
+
+    def two_passes():
+        cache = fo.flashomni_gemm_reduction(x, w, heads, info, ip, 0, bias=b, is_for_cache=True)
+        return cache, fo.flashomni_gemm_reduction(x, w, heads, info, ip, 0, bias=cache, is_for_cache=False)
+
+    s = torch.cuda.Stream(device=dev)
+    s.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(s):
+        two_passes()
+    torch.cuda.current_stream().wait_stream(s)
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        cache_g, final_g = two_passes()
+    for replay in range(3):
+        x.copy_(torch.randn(1, m, n, generator=g, device=dev).to(torch.bfloat16))
+        if replay >= 1:
+            info.copy_(fo.packbits(bits().to(dev), "little"))
+        graph.replay()
+        torch.cuda.synchronize()
+        got = (cache_g.clone(), final_g.clone())
+        ref = two_passes()
+        torch.cuda.synchronize()
+        for name, a, r in zip(("cache pass", "final pass"), got, ref):
+            assert torch.equal(a, r), "replay %d: %s differs from the eager call" % (replay, name)
