@@ -104,7 +104,9 @@ def test_undersized_symbols_raise(dev):
 @pytest.mark.parametrize("use_bias", [False, True])
 @pytest.mark.parametrize("shape", [(1, 512, 384, 3, 0), (2, 256, 256, 2, 0), (1, 300, 512, 4, 0),
                                    # head widths that are not multiples of the 64-wide operand slabs: 96, 32, 160
-                                   (1, 384, 384, 4, 0), (1, 200, 128, 4, 0), (1, 256, 640, 4, 128)])
+                                   (1, 384, 384, 4, 0), (1, 200, 128, 4, 0), (1, 256, 640, 4, 128),
+                                   # more heads than the kernel fetches a work item ahead (160 slices of width 32)
+                                   (1, 300, 5120, 160, 0)])
 def test_gemm_o_two_pass_protocol(dev, dtype, use_bias, shape):
     """cache pass, then final pass fed with the cached partial: each pass matches its oracle and the
     end result equals the dense linear layer (the identity the reference's own script checks,
