@@ -1162,6 +1162,7 @@ int check_common(const void* x, const void* w, void* y, int dtype, int32_t batch
   FO_REQUIRE(n % 128 == 0 && k % 32 == 0, "only support N %% 128 == 0, K %% 32 == 0 (got N=%d K=%d)",
              n, k);
   FO_REQUIRE(k >= kBK, "gemm: K = %d is below the 64 columns one operand slab holds", k);
+  FO_REQUIRE(k <= 65536, "gemm: K = %d is above 65536 (a k-step entry keeps its k offset in 16 bits)", k);
   FO_REQUIRE(sparse_q_size > 0 && num_qo_heads > 0 && n % num_qo_heads == 0,
              "gemm: bad sparse_q_size / num_qo_heads");
   FO_REQUIRE(x && w && y, "gemm: null pointer");

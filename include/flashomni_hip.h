@@ -201,7 +201,7 @@ int fo_sparse_fa_run(const void* q, const void* k, const void* v, void* o, float
  * x [B,M,K], w [N,K], y [B,M,N] row-major contiguous; bias [N] or NULL; dtype FO_BF16/FO_F16.
  * Tile (b, iy, ix) tests bit ((num_text_tokens + iy*128)/sparse_q_size)*num_qo_heads
  * + (ix*128)/(N/num_qo_heads) of sparse_info + sparse_info_indptr[b] (gemm.cuh:50-58).
- * Requires N % 128 == 0, K % 32 == 0 (csrc/gemm.cu:36) and K >= 64; M may have a tail (the
+ * Requires N % 128 == 0, K % 32 == 0 (csrc/gemm.cu:36) and 64 <= K <= 65536; M may have a tail (the
  * reference demands M % 128 == 0).
  * `workspace`: device scratch of at least fo_gemm_workspace_bytes(batch, m, n) bytes, 16-byte
  * aligned; it receives the list of tile quads that the GEMM kernel walks (short launches, up to

@@ -78,6 +78,10 @@ def test_gemm_q_shape_errors(dev):
     x, w, b = _operands(1, 128, 128, 32, torch.bfloat16, seed=1)
     with pytest.raises(RuntimeError, match="below the 64 columns"):
         fo.flashomni_gemm(x.to(dev), w.to(dev), 1, is_full=True)
+    x = torch.zeros(1, 128, 65600, dtype=torch.bfloat16, device=dev)
+    w = torch.zeros(128, 65600, dtype=torch.bfloat16, device=dev)
+    with pytest.raises(RuntimeError, match="above 65536"):
+        fo.flashomni_gemm(x, w, 1, is_full=True)
 
 
 def test_undersized_symbols_raise(dev):
