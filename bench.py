@@ -262,17 +262,33 @@ def bench_wan_chain(dev, iters, warmup):
     cache = fo.flashomni_gemm_reduction(o.view(1, s.seq, s.hidden), wo, s.heads, info, ip, 0, bias=None,
                                         is_for_cache=True)
 
+    # As in the FLUX step, what does not depend on the Q projection (the decode of the symbols; for fp8
+    # also the quantisation of K) runs on a second stream (default priority) beside GEMM-Q.
+    side = torch.cuda.Stream(device=dev)
+
     def chain_fp8():
+        cur = torch.cuda.current_stream()
+        side.wait_stream(cur)
+        with torch.cuda.stream(side):
+            w8.decode(info, kv_info, ip, kv_ip)
+            k8, ks = fo.quant_fp8_block(k, wl.kv_indptr, blocks=blocks)
         fo.flashomni_gemm(x, wq, s.heads, info, ip, 0, bq, out=False, quant_out=(q8, q8s, q8lo))
-        k8, ks = fo.quant_fp8_block(k, wl.kv_indptr, blocks=blocks)
+        cur.wait_stream(side)
+        k8.record_stream(cur)
+        ks.record_stream(cur)
         w8.run(q8.view(s.seq, s.heads, 128), k8, v, info, kv_info, ip, kv_ip, out=o, q_scale=q8s, k_scale=ks,
-               q_lo=q8lo.view(s.seq, s.heads, 128))
+               q_lo=q8lo.view(s.seq, s.heads, 128), reuse_decoded=True)
         return fo.flashomni_gemm_reduction(o.view(1, s.seq, s.hidden), wo, s.heads, info, ip, 0, bias=cache,
                                            is_for_cache=False)
 
     def chain_bf16():
+        cur = torch.cuda.current_stream()
+        side.wait_stream(cur)
+        with torch.cuda.stream(side):
+            w16.decode(info, kv_info, ip, kv_ip)
         fo.flashomni_gemm(x, wq, s.heads, info, ip, 0, bq, out=q16)
-        w16.run(q16.view(s.seq, s.heads, 128), k, v, info, kv_info, ip, kv_ip, out=o)
+        cur.wait_stream(side)
+        w16.run(q16.view(s.seq, s.heads, 128), k, v, info, kv_info, ip, kv_ip, out=o, reuse_decoded=True)
         return fo.flashomni_gemm_reduction(o.view(1, s.seq, s.hidden), wo, s.heads, info, ip, 0, bias=cache,
                                            is_for_cache=False)
 
