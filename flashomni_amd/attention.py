@@ -122,6 +122,7 @@ class PlannedBatch:
         self.q_blk_base = q_base.to(torch.int32).to(self.device)
         self.kv_blk_base = kv_base.to(torch.int32).to(self.device)
         self.n_kv_blk = int(kv_base[-1])
+        self.max_kv_len = int(klen.max()) if klen.numel() else 0
         # sizes the tensors given to run() must have (checked there without reading the device):
         # token counts, and the packed bytes of the byte-aligned per-request segments
         self.total_q_rows = int(qo_indptr_host[-1]) if qo_indptr_host.numel() else 0
@@ -204,7 +205,8 @@ class PlannedBatch:
             cur.wait_event(ev)
         return self.worklist
 
-    def launch(self, q, k, v, out, lse, kv_layout, sm_scale, q_scale=None, k_scale=None, q_lo=None) -> None:
+    def launch(self, q, k, v, out, lse, kv_layout, sm_scale, q_scale=None, k_scale=None, q_lo=None,
+               k_lo=None) -> None:
         """Shape checks against the planned batch, then fo_sparse_fa_run over the decoded list."""
         if q.dim() != 3 or k.dim() != 3 or v.dim() != 3 or k.size(2) != 128 or v.size(2) != 128:
             raise ValueError("q, k and v must be 3-dimensional with head_dim 128")
@@ -218,8 +220,15 @@ class PlannedBatch:
             if q_lo is not None and (q_lo.dtype != q.dtype or q_lo.shape != q.shape
                                      or q_lo.stride() != q.stride() or q_lo.device != q.device):
                 raise ValueError("q_lo must be a float8_e4m3fn tensor laid out like q")
-        elif q_lo is not None:
-            raise ValueError("q_lo is the second term of an fp8 q")
+            if k_lo is not None and (k_lo.dtype != k.dtype or k_lo.shape != k.shape
+                                     or k_lo.stride() != k.stride() or k_lo.device != k.device):
+                raise ValueError("k_lo must be a float8_e4m3fn tensor laid out like k")
+            if k_lo is not None and q_lo is None:
+                raise ValueError("k_lo (the second term of an fp8 k) needs q_lo as well")
+            if k_lo is not None and self.max_kv_len > 2048 * 128:
+                raise NotImplementedError("with k_lo a request may hold at most 262144 kv tokens")
+        elif q_lo is not None or k_lo is not None:
+            raise ValueError("q_lo / k_lo are the second terms of an fp8 q / k")
         if q.device != self.device:
             raise ValueError(f"Invalid device of q: expected {self.device}, got {q.device}")
         if q.size(1) != self.num_qo_heads or q.size(2) != 128:
@@ -251,7 +260,7 @@ class PlannedBatch:
         with _lib.device_guard(self.device):
             _lib.check(_lib.lib().fo_sparse_fa_run(
                 _lib.ptr(q), _lib.ptr(k), _lib.ptr(v), _lib.ptr(out), _lib.ptr(lse),
-                _lib.dtype_code(q.dtype), _lib.ptr(q_lo), _lib.ptr(q_scale if fp8 else None),
+                _lib.dtype_code(q.dtype), _lib.ptr(q_lo), _lib.ptr(k_lo), _lib.ptr(q_scale if fp8 else None),
                 _lib.ptr(k_scale if fp8 else None),
                 q.stride(0), q.stride(1), k_sn, k_sh, v_sn, v_sh, out.stride(0), out.stride(1),
                 _lib.ptr(self.qo_indptr), _lib.ptr(self.kv_indptr), _lib.ptr(self.q_blk_base),
@@ -528,6 +537,7 @@ class BatchFlashOmniFAWithRaggedKVWrapper:
         q_scale: Optional[torch.Tensor] = None,
         k_scale: Optional[torch.Tensor] = None,
         q_lo: Optional[torch.Tensor] = None,
+        k_lo: Optional[torch.Tensor] = None,
         reuse_decoded: bool = False,
     ) -> Union[torch.Tensor, Tuple[torch.Tensor, torch.Tensor]]:
         r"""Compute block-sparse prefill attention.
@@ -543,7 +553,10 @@ class BatchFlashOmniFAWithRaggedKVWrapper:
         ``quant_fp8_block(..., residual=True)`` / ``flashomni_gemm(..., quant_out="residual")``
         return): the logits are computed from ``q + q_lo``, which leaves only the rounding of ``k``
         in them and brings the output within relative L2 3e-2 of the unquantised result for
-        unit-variance q (two e4m3 operands alone give ~3.9e-2).
+        unit-variance q (two e4m3 operands alone give ~3.9e-2).  ``k_lo`` (needs ``q_lo``): the
+        same for ``k`` (``quant_fp8_block(k, ..., residual=True)``); the logits then are
+        ``k.q + k.q_lo + k_lo.q`` under the same scales, as accurate as 16-bit logits, for data
+        on which one e4m3 byte per element of ``k`` is too coarse (q with rms well above 1).
 
         ``reuse_decoded`` (keyword-only extension): the symbols are decoded on every call, because
         a buffer rewritten in place (by a kernel of the caller's, through the C ABI, ...) looks the
@@ -573,7 +586,8 @@ class BatchFlashOmniFAWithRaggedKVWrapper:
             pb.reuse_decoded(is_full)
         else:
             pb.decode(sparse_info, sparse_kv_info, sparse_info_indptr, sparse_kv_info_indptr, is_full)
-        pb.launch(q, k, v, out, lse if return_lse else None, self._kv_layout, sm_scale, q_scale, k_scale, q_lo)
+        pb.launch(q, k, v, out, lse if return_lse else None, self._kv_layout, sm_scale, q_scale, k_scale, q_lo,
+                  k_lo)
         return (out, lse) if return_lse else out
 
     run_return_lse = functools.partialmethod(run, return_lse=True)

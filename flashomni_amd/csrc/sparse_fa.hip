@@ -79,9 +79,10 @@ constexpr int kOutTileOff = kMergeOBytes + 4 * 64 * 8;  // behind the merge area
 constexpr int kOutRowBytes = 256 + 16;                  // one output row of 128 16-bit elements, padded
 constexpr int kOutTileBytes = 128 * kOutRowBytes;
 // LDS geometry of one kv group: two stages of (K tile, V tile); K is 16-bit or fp8
-template <bool kFp8>
+template <bool kFp8, bool kKLo = false>
 struct Geom {
-  static constexpr int kKBytes = kTileKV * (kFp8 ? kRowBytes8 : kRowBytes);
+  // (fp8 K with a second term: the tile of k, then the tile of k_lo)
+  static constexpr int kKBytes = kTileKV * (kFp8 ? (kKLo ? 2 : 1) * kRowBytes8 : kRowBytes);
   static constexpr int kStageBytes = kKBytes + kVBytes;
   static constexpr int kGroupBytes = 2 * kStageBytes;
   static constexpr int kTilesBytes = 2 * kGroupBytes;
@@ -92,6 +93,7 @@ struct Geom {
 };
 constexpr int kXcds = 8;
 constexpr int kMaxRowBlocks = 4096;  // kv blocks of one row held in LDS (512 Ki tokens per request)
+constexpr int kMaxRowBlocksKLo = 2048;  // the same for the two-term k, whose tiles leave less LDS
 constexpr float kLazyLog2 = 8.0f;  // the running max is raised only past a 2^8 overshoot
 // merge area (reuses the tile buffers): O^T of kv group 1, then its (m, d)
 static_assert(kOutTileOff + kOutTileBytes <= Geom<true>::kSmemBytes, "merge area must fit");
@@ -103,6 +105,7 @@ struct FaParams {
   void* o;
   float* lse;
   const void* q_lo;  // fp8: optional second e4m3 term of q (same layout and scale as q)
+  const void* k_lo;  // fp8: optional second e4m3 term of k (same layout and scale as k)
   const float* q_scale;
   const float* k_scale;
   int64_t q_sn, q_sh, k_sn, k_sh, v_sn, v_sh, o_sn, o_sh;
@@ -254,13 +257,17 @@ __device__ __forceinline__ int pop_row(const FaParams& p, int xcd, const int* q,
 // per slab: e4m3 keeps 3 mantissa bits, and with both operands rounded to it the logits are too
 // noisy for the accuracy this path promises; with the two-term q only k's rounding is left.  The
 // fp8 matrix cores run at twice the 16-bit rate, so the two terms cost what a 16-bit S^T costs.
-template <typename T, bool kFp8, bool kQLo>
+// kKLo: k comes as two e4m3 terms as well, k + k_lo; S^T = k.q^T + k.q_lo^T + k_lo.q^T (the product
+// of the two residuals, 2^-8 of the logit, is left out): both operands then carry ~7 significant
+// bits and the logits are as accurate as 16-bit ones.  This is the accuracy form, not a fast one.
+template <typename T, bool kFp8, bool kQLo, bool kKLo>
 __global__ void __launch_bounds__(kThreads) sparse_fa_kernel(const FaParams p) {
   static_assert(kFp8 || !kQLo, "the two-term q is an fp8 form");
+  static_assert(kQLo || !kKLo, "the two-term k is built on the two-term q");
   using TT = Types<T>;
   using x8 = typename TT::x8;
   using x4 = typename TT::x4;
-  using G = Geom<kFp8>;
+  using G = Geom<kFp8, kKLo>;
   using TQK = typename std::conditional<kFp8, uint8_t, T>::type;
   constexpr int kStageBytes = G::kStageBytes, kKBytes = G::kKBytes, kGroupBytes = G::kGroupBytes;
   extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
@@ -286,10 +293,11 @@ __global__ void __launch_bounds__(kThreads) sparse_fa_kernel(const FaParams p) {
   __shared__ int s_queue[16];  // queue bounds and even-share words of `sched`, read once
   __shared__ int s_share[1];   // even shares: items of this workgroup's share handed out so far
   __shared__ RowInfo s_items[kItemBatch];  // even shares: records of the share's next items
-  __shared__ uint16_t s_blk2[2][kMaxRowBlocks];  // kv block list of this row / the next one
+  constexpr int kRowBlocks = kKLo ? kMaxRowBlocksKLo : kMaxRowBlocks;
+  __shared__ uint16_t s_blk2[2][kRowBlocks];  // kv block list of this row / the next one
   // fp8: the k dequantisation scales of the listed blocks (read per tile: from global memory the
   // compiler would wait for every tile copy in flight along with them)
-  __shared__ float s_ksc2[2][kFp8 ? kMaxRowBlocks : 1];
+  __shared__ float s_ksc2[2][kFp8 ? kRowBlocks : 1];
 
   const int tid = threadIdx.x, lane = tid & 63;
   const int wv = __builtin_amdgcn_readfirstlane(tid >> 6);  // wavefront index, kept scalar
@@ -379,7 +387,7 @@ __global__ void __launch_bounds__(kThreads) sparse_fa_kernel(const FaParams p) {
           it.kv_begin = p.kv_indptr[it.req];
           it.kv_len = p.kv_indptr[it.req + 1] - it.kv_begin;
           // this share's range of the row's kv blocks
-          const int blk_lo = max(a, u) - u, blk_hi = min(min(b, e) - u, kMaxRowBlocks);
+          const int blk_lo = max(a, u) - u, blk_hi = min(min(b, e) - u, kRowBlocks);
           it.ptr0 = p.kv_row_ptr[w] + blk_lo;
           it.nb = max(blk_hi - blk_lo, 0);
           fill_scales(it);
@@ -421,7 +429,7 @@ __global__ void __launch_bounds__(kThreads) sparse_fa_kernel(const FaParams p) {
           ri.qb = r0[2];
           ri.head = r0[3];
           ri.ptr0 = r1[0];
-          ri.nb = min(r1[1], kMaxRowBlocks);
+          ri.nb = min(r1[1], kRowBlocks);
         } else {
           const int w = p.order[at];
           ri.row = w;
@@ -430,7 +438,7 @@ __global__ void __launch_bounds__(kThreads) sparse_fa_kernel(const FaParams p) {
           ri.head = p.row_head[w];
           ri.ptr0 = p.kv_row_ptr[w];
           // (a row longer than the LDS list is cut; the host side refuses such requests at plan time)
-          ri.nb = min(p.kv_row_ptr[w + 1] - ri.ptr0, kMaxRowBlocks);
+          ri.nb = min(p.kv_row_ptr[w + 1] - ri.ptr0, kRowBlocks);
         }
         ri.q_begin = p.qo_indptr[ri.req] + ri.qb * kBlockQ;
         ri.q_rows = min(kBlockQ, p.qo_indptr[ri.req + 1] - ri.q_begin);
@@ -582,7 +590,11 @@ __global__ void __launch_bounds__(kThreads) sparse_fa_kernel(const FaParams p) {
                                  : static_cast<uint32_t>((4 * qs + cp_row) * p.k_sn + cp_chunk) * sizeof(T);
     const int64_t k_jstep = (kFp8 ? 32 : 16) * p.k_sn * static_cast<int64_t>(sizeof(TQK));
     const int64_t v_jstep = 16 * p.v_sn * static_cast<int64_t>(sizeof(T));
-    constexpr int kKCopies = kFp8 ? 2 : 4, kVCopies = 4;  // copy instructions per wavefront and tile
+    constexpr int kKCopies = (kFp8 && !kKLo) ? 2 : 4, kVCopies = 4;  // copy instructions per wavefront and tile
+    const uint8_t* klo_head = nullptr;
+    if constexpr (kKLo)
+      klo_head = static_cast<const uint8_t*>(p.k_lo) + static_cast<int64_t>(kv_begin) * p.k_sn +
+                 static_cast<int64_t>(kv_head) * p.k_sh;
     auto tile_start = [&](int j) { return s_blk[j] * kBlockKV + kg * kTileKV; };
     auto tile_valid = [&](int j) { return min(kTileKV, kv_len - tile_start(j)); };
     // all K copies of tile j at once
@@ -591,18 +603,22 @@ __global__ void __launch_bounds__(kThreads) sparse_fa_kernel(const FaParams p) {
       const int valid = min(kTileKV, kv_len - start);
       const uint8_t* kt = reinterpret_cast<const uint8_t*>(k_head + static_cast<int64_t>(start) * p.k_sn);
       const uint32_t kdst = lds_group + (j & 1) * kStageBytes + qs * 1024;
+      // (two-term k: copy instructions 0, 1 fetch the tile of k, 2, 3 that of k_lo behind it)
+      constexpr int kPerTerm = kKLo ? 2 : kKCopies;
+      const uint8_t* kt_lo = kKLo ? klo_head + static_cast<int64_t>(start) * p.k_sn : nullptr;
       if (__builtin_expect(valid == kTileKV, 1)) {
 #pragma unroll
-        for (int n = 0; n < kKCopies; ++n) copy16_to_lds(kt + n * k_jstep, k_voff, kdst + n * 4096);
+        for (int n = 0; n < kKCopies; ++n)
+          copy16_to_lds((n < kPerTerm ? kt : kt_lo) + (n % kPerTerm) * k_jstep, k_voff, kdst + n * 4096);
       } else {
         // ragged tail: re-read the last valid row, never overrun
 #pragma unroll
         for (int n = 0; n < kKCopies; ++n) {
-          int r = (kFp8 ? 8 : 4) * (4 * n + qs) + (kFp8 ? cp8_row : cp_row);
+          int r = (kFp8 ? 8 : 4) * (4 * (n % kPerTerm) + qs) + (kFp8 ? cp8_row : cp_row);
           r = r < valid ? r : valid - 1;
           const uint32_t off = kFp8 ? static_cast<uint32_t>(r * p.k_sn + cp8_chunk)
                                     : static_cast<uint32_t>((r * p.k_sn + cp_chunk) * sizeof(T));
-          copy16_to_lds(kt, off, kdst + n * 4096);
+          copy16_to_lds(n < kPerTerm ? kt : kt_lo, off, kdst + n * 4096);
         }
       }
     };
@@ -760,6 +776,20 @@ __global__ void __launch_bounds__(kThreads) sparse_fa_kernel(const FaParams p) {
             for (int mt = 0; mt < 2; ++mt)
               s[mt] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(k8[mt][sl], qlo8[sl], s[mt], 0, 0, 0,
                                                                       0x7f7f7f7f, 0, 0x7f7f7f7f);
+        }
+        if constexpr (kKLo) {
+          // k_lo . q^T: the tile of k_lo sits behind the tile of k in the stage
+#pragma unroll
+          for (int sl = 0; sl < 2; ++sl)
+#pragma unroll
+            for (int mt = 0; mt < 2; ++mt) {
+              const uint8_t* rowp = ks_base + kTileKV * kRowBytes8 + mt * 32 * kRowBytes8 + k_rd_base;
+              const i32x4 lo = *reinterpret_cast<const i32x4*>(rowp + (k_rd_x ^ (sl << 6)));
+              const i32x4 hi = *reinterpret_cast<const i32x4*>(rowp + ((k_rd_x ^ (sl << 6)) ^ 16));
+              const i32x8 kl = i32x8{lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
+              s[mt] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(kl, qreg8[sl], s[mt], 0, 0, 0,
+                                                                      0x7f7f7f7f, 0, 0x7f7f7f7f);
+            }
         }
       }
     };
@@ -1152,16 +1182,16 @@ __global__ void __launch_bounds__(kThreads) sparse_fa_kernel(const FaParams p) {
   }
 }
 
-template <typename T, bool kFp8, bool kQLo>
+template <typename T, bool kFp8, bool kQLo, bool kKLo>
 int launch(const FaParams& p, int64_t max_rows, hipStream_t stream) {
-  constexpr int kSmemBytes = Geom<kFp8>::kSmemBytes;
+  constexpr int kSmemBytes = Geom<kFp8, kKLo>::kSmemBytes;
   // (the attribute belongs to the kernel's code object on one device: set once per device; the flags
   // are atomic because host threads may launch concurrently, and setting it twice is harmless)
   static std::atomic<bool> attr_set[64] = {};
   int dev = 0;
   FO_HIP_CALL(hipGetDevice(&dev));
   if (dev < 0 || dev >= 64 || !attr_set[dev].load(std::memory_order_acquire)) {
-    FO_HIP_CALL(hipFuncSetAttribute(reinterpret_cast<const void*>(&sparse_fa_kernel<T, kFp8, kQLo>),
+    FO_HIP_CALL(hipFuncSetAttribute(reinterpret_cast<const void*>(&sparse_fa_kernel<T, kFp8, kQLo, kKLo>),
                                     hipFuncAttributeMaxDynamicSharedMemorySize, kSmemBytes));
     if (dev >= 0 && dev < 64) attr_set[dev].store(true, std::memory_order_release);
   }
@@ -1170,7 +1200,7 @@ int launch(const FaParams& p, int64_t max_rows, hipStream_t stream) {
   int64_t grid = num_cu;  // one persistent workgroup per CU (LDS bound)
   // (with even shares every workgroup may hold a part of a row; otherwise at most one row each)
   if (!(p.split_ws && p.shares) && grid > max_rows) grid = max_rows;
-  sparse_fa_kernel<T, kFp8, kQLo><<<static_cast<unsigned>(grid), kThreads, kSmemBytes, stream>>>(p);
+  sparse_fa_kernel<T, kFp8, kQLo, kKLo><<<static_cast<unsigned>(grid), kThreads, kSmemBytes, stream>>>(p);
   FO_CHECK_LAUNCH();
   return FO_OK;
 }
@@ -1183,7 +1213,8 @@ extern "C" int64_t fo_sparse_fa_split_workspace_bytes(void) {
 }
 
 extern "C" int fo_sparse_fa_run(const void* q, const void* k, const void* v, void* o, float* lse,
-                                int dtype, const void* q_lo, const float* q_scale, const float* k_scale,
+                                int dtype, const void* q_lo, const void* k_lo, const float* q_scale,
+                                const float* k_scale,
                                 int64_t q_stride_n, int64_t q_stride_h, int64_t k_stride_n,
                                 int64_t k_stride_h, int64_t v_stride_n, int64_t v_stride_h,
                                 int64_t o_stride_n, int64_t o_stride_h, const int32_t* qo_indptr,
@@ -1221,13 +1252,14 @@ extern "C" int fo_sparse_fa_run(const void* q, const void* k, const void* v, voi
     FO_REQUIRE(q_scale && k_scale && q_blk_base && kv_blk_base && n_q_blocks > 0 && n_kv_blocks > 0,
                "sparse_fa: fp8 q/k need q_scale, k_scale, the block numbering and the scale row lengths");
   FO_REQUIRE(q_lo == nullptr || dtype == FO_FP8_E4M3, "sparse_fa: q_lo is the second term of an fp8 q");
-  for (const void* ptr : {q, k, v, static_cast<const void*>(o), q_lo})
+  FO_REQUIRE(k_lo == nullptr || q_lo != nullptr, "sparse_fa: k_lo (second term of an fp8 k) needs q_lo as well");
+  for (const void* ptr : {q, k, v, static_cast<const void*>(o), q_lo, k_lo})
     FO_REQUIRE((reinterpret_cast<uintptr_t>(ptr) & 15) == 0,
                "sparse_fa: q/k/v/o must be 16-byte aligned");
 
   FaParams p;
   p.q = q; p.k = k; p.v = v; p.o = o; p.lse = lse;
-  p.q_lo = q_lo; p.q_scale = q_scale; p.k_scale = k_scale;
+  p.q_lo = q_lo; p.k_lo = k_lo; p.q_scale = q_scale; p.k_scale = k_scale;
   p.q_sn = q_stride_n; p.q_sh = q_stride_h; p.k_sn = k_stride_n; p.k_sh = k_stride_h;
   p.v_sn = v_stride_n; p.v_sh = v_stride_h; p.o_sn = o_stride_n; p.o_sh = o_stride_h;
   p.qo_indptr = qo_indptr; p.kv_indptr = kv_indptr;
@@ -1250,8 +1282,9 @@ extern "C" int fo_sparse_fa_run(const void* q, const void* k, const void* v, voi
   p.num_heads = num_heads; p.kv_group = num_heads / num_kv_heads; p.n_q_blocks = n_q_blocks; p.n_kv_blocks = n_kv_blocks;
   p.sm_scale_log2 = sm_scale * 1.44269504088896340736f;
   hipStream_t s = static_cast<hipStream_t>(stream);
-  if (dtype == FO_BF16) return launch<__bf16, false, false>(p, max_rows, s);
-  if (dtype == FO_F16) return launch<_Float16, false, false>(p, max_rows, s);
-  if (q_lo != nullptr) return launch<__bf16, true, true>(p, max_rows, s);
-  return launch<__bf16, true, false>(p, max_rows, s);
+  if (dtype == FO_BF16) return launch<__bf16, false, false, false>(p, max_rows, s);
+  if (dtype == FO_F16) return launch<_Float16, false, false, false>(p, max_rows, s);
+  if (k_lo != nullptr) return launch<__bf16, true, true, true>(p, max_rows, s);
+  if (q_lo != nullptr) return launch<__bf16, true, true, false>(p, max_rows, s);
+  return launch<__bf16, true, false, false>(p, max_rows, s);
 }

@@ -49,18 +49,23 @@ def _symbols(sparse_info, sparse_info_indptr, device, name, batch, m, num_qo_hea
     return info, indptr
 
 
-# scratch of the GEMMs (GEMM-Q's tile list, GEMM-O's work-item cursors), one buffer per (device, stream): calls on one stream run in order, so
-# they can share it; calls on different streams may overlap and get their own
+# Scratch of the GEMMs (GEMM-Q's tile list, GEMM-O's work-item cursors).  Eager calls share one
+# buffer per (device, stream): calls on one stream run in order, calls on different streams may
+# overlap and get their own.  A call made while its stream is being captured into a graph gets a
+# buffer of its own from the allocator (the graph's memory pool then owns it for as long as the
+# graph lives), and a buffer that has become too small is kept, not freed, when a larger one
+# replaces it: a launch already recorded or in flight may still hold its address.  Sizes are
+# rounded up to powers of two, so a stream retires at most a few dozen small buffers.
 _workspaces = {}
 
 
 def _gemm_workspace(device, stream, nbytes):
-    key = (device.index, stream)
-    ws = _workspaces.get(key)
-    if ws is None or ws.numel() < nbytes:
-        ws = torch.empty(max(nbytes, 1), dtype=torch.uint8, device=device)
-        _workspaces[key] = ws
-    return ws
+    if torch.cuda.is_current_stream_capturing():
+        return torch.empty(max(nbytes, 256), dtype=torch.uint8, device=device)
+    bufs = _workspaces.setdefault((device.index, stream), [])
+    if not bufs or bufs[-1].numel() < nbytes:
+        bufs.append(torch.empty(1 << (max(nbytes, 4096) - 1).bit_length(), dtype=torch.uint8, device=device))
+    return bufs[-1]
 
 
 def flashomni_gemm(

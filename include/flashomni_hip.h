@@ -19,7 +19,7 @@
 extern "C" {
 #endif
 
-#define FO_ABI_VERSION 2
+#define FO_ABI_VERSION 3
 
 enum {
   FO_OK = 0,
@@ -164,7 +164,13 @@ int fo_decode_sparse_static(const uint8_t* sparse_info, const uint8_t* sparse_kv
  * block); v and o are bf16.  q_lo (optional, else NULL): a second e4m3fn tensor laid out like q, the
  * rounding residual of q under the same scale (fo_quant_fp8_block / fo_gemm_q_quant write it);
  * the logits are then K.(q + q_lo)^T, two fp8 products at the cost of one 16-bit one, and only k's
- * rounding error is left in them.  (The fp8 form has no counterpart in the reference.)
+ * rounding error is left in them.  k_lo (optional, else NULL; needs q_lo): the same for k, laid out
+ * like k under k's scales; the logits are then k.q^T + k.q_lo^T + k_lo.q^T (the product of the two
+ * residuals is left out), as accurate as 16-bit logits at three fp8 products per tile: the
+ * accuracy form for data on which one e4m3 byte per element of k is too coarse, not a fast one.
+ * A request may hold at most 524 288 kv tokens (4096 kv blocks, the list of one row is staged in
+ * LDS), with k_lo 262 144: the caller checks that (the lengths live on the device).
+ * (The fp8 form has no counterpart in the reference.)
  * Rows of the list write every output row of their q-block; q-blocks not in the list are left
  * untouched; a listed row with no kv block writes zeros and lse = -5e4.  lse (optional, fp32
  * [nnz_q,H]) is base 2: log2(sum 2^(s*c - m*c)) + m*c, c = sm_scale*log2(e).
@@ -182,7 +188,8 @@ int fo_decode_sparse_static(const uint8_t* sparse_info, const uint8_t* sparse_kv
  * ------------------------------------------------------------------------------------------- */
 int64_t fo_sparse_fa_split_workspace_bytes(void);
 int fo_sparse_fa_run(const void* q, const void* k, const void* v, void* o, float* lse, int dtype,
-                     const void* q_lo, const float* q_scale, const float* k_scale, int64_t q_stride_n,
+                     const void* q_lo, const void* k_lo, const float* q_scale, const float* k_scale,
+                     int64_t q_stride_n,
                      int64_t q_stride_h, int64_t k_stride_n, int64_t k_stride_h,
                      int64_t v_stride_n, int64_t v_stride_h, int64_t o_stride_n,
                      int64_t o_stride_h, const int32_t* qo_indptr, const int32_t* kv_indptr,

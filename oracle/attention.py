@@ -24,14 +24,14 @@ NEG_INF = -5e4
 def sparse_attention(q, k, v, sparse_info, sparse_kv_info, sparse_info_indptr,
                      sparse_kv_info_indptr, qo_indptr, kv_indptr, block_q=128, block_kv=128,
                      sm_scale=None, is_full=False, out=None, lse=None, rows=None,
-                     q_scale=None, k_scale=None, q_lo=None):
+                     q_scale=None, k_scale=None, q_lo=None, k_lo=None):
     """q [nnz_q,H,D], k/v [nnz_kv,H,D] (any float dtype; math is fp32 on the given values).
 
     `out` (same dtype as q unless q is fp8, then bf16) is updated in place for active rows only; allocated
     as zeros when None (flashomni/attention.py:779-785).  `rows`: optional iterable of
     row-list positions to evaluate (sampling for the big configs); others are left untouched.
     q_scale/k_scale: optional fp32 [H, n_blocks] dequantisation scales for fp8 q/k; q_lo: optional
-    second fp8 term added to q before scaling (no reference counterpart)."""
+    second fp8 term added to q before scaling; k_lo: the same for k (no reference counterpart)."""
     H, D = q.shape[1], q.shape[2]
     group = H // k.shape[1]   # q heads per kv head (prefill.cuh:410-413); 1 without grouped-query attention
     if sm_scale is None:
@@ -68,6 +68,8 @@ def sparse_attention(q, k, v, sparse_info, sparse_kv_info, sparse_info_indptr,
         if q_lo is not None:
             qf = qf + q_lo[q0:q1, h].float()
         kf = k[tok_t, h // group].float()
+        if k_lo is not None:
+            kf = kf + k_lo[tok_t, h // group].float()
         vf = v[tok_t, h // group].float()
         if q_scale is not None:
             qf = qf * float(q_scale[h, int(q_blk_base[r]) + qb])

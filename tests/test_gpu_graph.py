@@ -119,3 +119,55 @@ def test_captured_long_gemm_o_replays(dev):
         torch.cuda.synchronize()
         for name, a, r in zip(("cache pass", "final pass"), got, ref):
             assert torch.equal(a, r), "replay %d: %s differs from the eager call" % (replay, name)
+
+
+def test_graph_captured_on_a_warm_stream_survives_workspace_growth(dev):
+    """GEMM-Q keeps its tile list in a scratch buffer cached per stream.  A graph captured on a stream
+    that already ran the GEMM eagerly must not record that cached buffer: a later, larger eager GEMM on
+    the same stream replaces it, and a replay would then write its list into memory that may belong to
+    someone else.  Capture on the warm stream, grow the scratch eagerly on it, replay, compare."""
+    import flashomni_amd as fo
+    from flashomni_amd import gemm as gemm_mod
+    heads, hidden = 4, 512
+    g = torch.Generator(device=dev).manual_seed(17)
+    rng = np.random.default_rng(17)
+
+    def problem(m):
+        x = torch.randn(1, m, hidden, generator=g, device=dev).to(torch.bfloat16)
+        info = fo.packbits(torch.from_numpy(rng.random(-(-m // 128) * heads) < 0.6).to(dev), "little")
+        ip = torch.tensor([0, info.numel()], dtype=torch.int32, device=dev)
+        return x, info, ip
+
+    w = (torch.randn(hidden, hidden, generator=g, device=dev) * 0.05).to(torch.bfloat16)
+    # (large enough that the tile list is built by the list kernel into the scratch buffer)
+    x, info, ip = problem(128 * 300)
+    out = torch.zeros(1, x.size(1), hidden, dtype=torch.bfloat16, device=dev)
+    s = torch.cuda.Stream(device=dev)
+    s.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(s):
+        fo.flashomni_gemm(x, w, heads, info, ip, 0, None, out=out)   # eager warm-up on s
+    s.synchronize()
+    eager_bufs = {b.data_ptr() for b in gemm_mod._workspaces[(dev.index, s.cuda_stream)]}
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph, stream=s):
+        fo.flashomni_gemm(x, w, heads, info, ip, 0, None, out=out)
+    # a much larger GEMM on the same stream: the stream's scratch buffer is replaced
+    xb, infob, ipb = problem(128 * 3000)
+    with torch.cuda.stream(s):
+        big = fo.flashomni_gemm(xb, w, heads, infob, ipb, 0, None)
+    s.synchronize()
+    bufs = gemm_mod._workspaces[(dev.index, s.cuda_stream)]
+    assert len(bufs) >= 2 and eager_bufs <= {b.data_ptr() for b in bufs}, "superseded scratch must stay alive"
+    del big, xb
+    torch.cuda.empty_cache()
+    junk = [torch.full((1 << 20,), 0x5a, dtype=torch.uint8, device=dev) for _ in range(8)]  # reuse freed memory
+    for replay in range(3):
+        x.copy_(torch.randn(1, x.size(1), hidden, generator=g, device=dev).to(torch.bfloat16))
+        out.zero_()
+        graph.replay()
+        torch.cuda.synchronize()
+        ref = torch.zeros_like(out)
+        fo.flashomni_gemm(x, w, heads, info, ip, 0, None, out=ref)
+        torch.cuda.synchronize()
+        assert torch.equal(out, ref), "replay %d differs from the eager call" % replay
+        assert all(bool((j == 0x5a).all()) for j in junk), "a replay wrote outside its own scratch"
