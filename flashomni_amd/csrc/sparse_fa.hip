@@ -41,6 +41,13 @@
 // leaves in 16-byte pieces, 16 consecutive lanes per 256-byte output row.  (Both were measured:
 // fetched or stored from the accumulator layout, a wavefront instruction is 64 scattered pieces.)
 //
+// Long lists (eight rows per CU or more) run in a second form of the same kernel: a workgroup is
+// 4 wavefronts that own a whole row, two such workgroups share a CU, and the main loop is software-
+// pipelined in steps of 32 keys: the MFMAs of S(t+1) and P(t-1).V(t-1) are interleaved, instruction
+// by instruction, with the softmax of S(t), the operand reads four slots ahead and the copies two
+// steps ahead (see the kPipe branch of the kernel).  Measured on the video-sized lists it is ~5 %
+// faster than the two-phase form; on short lists a row's doubled latency costs more than that.
+//
 // Numerics follow the reference kernel (include/flashomni/attention/prefill.cuh:759-962): base-2
 // softmax p = exp2(s*c - m*c) with c = sm_scale*log2(e), P rounded to the activation type before
 // P.V, row sum d over the rounded p, O = acc * rcp(d) with one round-to-nearest cast, a row with no
@@ -48,6 +55,7 @@
 // lse = log2(d) + m*c.  Two liberties inside the stated tolerances: for 16-bit inputs c is
 // multiplied into Q once per row (one extra rounding of q), and the reference point m is the exact
 // row max of the first tile and afterwards raised only when exceeded by more than 2^8.
+#include <cstdlib>
 #include <type_traits>
 
 #include "fo_common.h"
@@ -61,6 +69,7 @@ typedef __attribute__((ext_vector_type(4))) _Float16 f16x4;
 typedef __attribute__((ext_vector_type(4))) short s16x4;
 typedef __attribute__((ext_vector_type(16))) float f32x16;
 typedef __attribute__((ext_vector_type(4))) float f32x4;
+typedef __attribute__((ext_vector_type(2))) float f32x2;
 typedef __attribute__((ext_vector_type(4))) unsigned int u32x4;
 typedef __attribute__((ext_vector_type(8))) int i32x8;
 typedef __attribute__((ext_vector_type(4))) int i32x4;
@@ -79,21 +88,23 @@ constexpr int kOutTileOff = kMergeOBytes + 4 * 64 * 8;  // behind the merge area
 constexpr int kOutRowBytes = 256 + 16;                  // one output row of 128 16-bit elements, padded
 constexpr int kOutTileBytes = 128 * kOutRowBytes;
 // LDS geometry of one kv group: two stages of (K tile, V tile); K is 16-bit or fp8
-template <bool kFp8, bool kKLo = false>
+template <bool kFp8, bool kKLo = false, int kGroups = 2>
 struct Geom {
   // (fp8 K with a second term: the tile of k, then the tile of k_lo)
   static constexpr int kKBytes = kTileKV * (kFp8 ? (kKLo ? 2 : 1) * kRowBytes8 : kRowBytes);
   static constexpr int kStageBytes = kKBytes + kVBytes;
   static constexpr int kGroupBytes = 2 * kStageBytes;
-  static constexpr int kTilesBytes = 2 * kGroupBytes;
+  static constexpr int kTilesBytes = kGroups * kGroupBytes;
   // the epilogue reuses the tile buffers: kv group 1's partial O (64 KB fp32) + its (max, sum)
-  // pairs (2 KB), then the finished row as a padded tile for the coalesced store
-  static constexpr int kSmemBytes = kTilesBytes > kOutTileOff + kOutTileBytes ? kTilesBytes
-                                                                              : kOutTileOff + kOutTileBytes;
+  // pairs (2 KB), then the finished row as a padded tile for the coalesced store (one kv group:
+  // no merge area, the output tile starts at 0)
+  static constexpr int kOutOff = kGroups == 2 ? kOutTileOff : 0;
+  static constexpr int kSmemBytes = kTilesBytes > kOutOff + kOutTileBytes ? kTilesBytes : kOutOff + kOutTileBytes;
 };
 constexpr int kXcds = 8;
 constexpr int kMaxRowBlocks = 4096;  // kv blocks of one row held in LDS (512 Ki tokens per request)
 constexpr int kMaxRowBlocksKLo = 2048;  // the same for the two-term k, whose tiles leave less LDS
+constexpr int kMaxRowBlocksOneGroup = 3072;  // and for the one-group form (two workgroups share a CU's LDS)
 constexpr float kLazyLog2 = 8.0f;  // the running max is raised only past a 2^8 overshoot
 // merge area (reuses the tile buffers): O^T of kv group 1, then its (m, d)
 static_assert(kOutTileOff + kOutTileBytes <= Geom<true>::kSmemBytes, "merge area must fit");
@@ -260,17 +271,29 @@ __device__ __forceinline__ int pop_row(const FaParams& p, int xcd, const int* q,
 // kKLo: k comes as two e4m3 terms as well, k + k_lo; S^T = k.q^T + k.q_lo^T + k_lo.q^T (the product
 // of the two residuals, 2^-8 of the logit, is left out): both operands then carry ~7 significant
 // bits and the logits are as accurate as 16-bit ones.  This is the accuracy form, not a fast one.
-template <typename T, bool kFp8, bool kQLo, bool kKLo>
-__global__ void __launch_bounds__(kThreads) sparse_fa_kernel(const FaParams p) {
+//
+// kGroups: kv groups of a workgroup.  2: the form described at the top of this file (8 wavefronts).
+// 1: a workgroup is 4 wavefronts (q sub-tiles 0..3) that walk all tiles of the row, two such
+// workgroups share a CU (one wavefront of each per SIMD) and run independent rows: nothing ties
+// their phases together, there is no merge, and one's row prologue / epilogue overlaps the other's
+// main loop.  A row takes twice as long, so this is the form for long lists (many rows per CU).
+template <typename T, bool kFp8, bool kQLo, bool kKLo, int kGroups, bool kPipe = false>
+__global__ void __launch_bounds__(kGroups * kGroupThreads) __attribute__((amdgpu_waves_per_eu(2, 2)))
+sparse_fa_kernel(const FaParams p) {
+  static_assert(kPipe == (kGroups == 1), "one kv group runs the software-pipelined loop, two the two-phase loop");
+  static_assert(!kPipe || !kFp8, "the software-pipelined loop is built for 16-bit operands");
   static_assert(kFp8 || !kQLo, "the two-term q is an fp8 form");
   static_assert(kQLo || !kKLo, "the two-term k is built on the two-term q");
+  constexpr int kWaves = 4 * kGroups;
+  constexpr int kFetchWave = kGroups == 2 ? 4 : 0;  // the wavefront that fetches the next item
   using TT = Types<T>;
   using x8 = typename TT::x8;
   using x4 = typename TT::x4;
-  using G = Geom<kFp8, kKLo>;
+  using G = Geom<kFp8, kKLo, kGroups>;
   using TQK = typename std::conditional<kFp8, uint8_t, T>::type;
   constexpr int kStageBytes = G::kStageBytes, kKBytes = G::kKBytes, kGroupBytes = G::kGroupBytes;
-  extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
+  // (256-byte aligned: lane offsets with XOR-swizzled low bits can then carry the array's base)
+  extern __shared__ __attribute__((aligned(256))) uint8_t smem[];
   // this item / the next one, with everything the row's prologue needs: fetched by the popping lane
   // while the rest of the workgroup finishes the current row
   struct RowInfo {
@@ -293,7 +316,7 @@ __global__ void __launch_bounds__(kThreads) sparse_fa_kernel(const FaParams p) {
   __shared__ int s_queue[16];  // queue bounds and even-share words of `sched`, read once
   __shared__ int s_share[1];   // even shares: items of this workgroup's share handed out so far
   __shared__ RowInfo s_items[kItemBatch];  // even shares: records of the share's next items
-  constexpr int kRowBlocks = kKLo ? kMaxRowBlocksKLo : kMaxRowBlocks;
+  constexpr int kRowBlocks = kGroups == 1 ? kMaxRowBlocksOneGroup : kKLo ? kMaxRowBlocksKLo : kMaxRowBlocks;
   __shared__ uint16_t s_blk2[2][kRowBlocks];  // kv block list of this row / the next one
   // fp8: the k dequantisation scales of the listed blocks (read per tile: from global memory the
   // compiler would wait for every tile copy in flight along with them)
@@ -351,7 +374,7 @@ __global__ void __launch_bounds__(kThreads) sparse_fa_kernel(const FaParams p) {
   // the start: their records are gathered sixteen at a time, all in parallel, so that between two
   // rows only the kv block list has to be fetched.
   const int ev_share = s_queue[10], ev_total = s_queue[11], ev_n = s_queue[12], ev_rows = s_queue[13];
-  const bool even = s_queue[9] != 0 && p.shares != nullptr && p.split_ws != nullptr &&
+  const bool even = kGroups == 2 && s_queue[9] != 0 && p.shares != nullptr && p.split_ws != nullptr &&
                     static_cast<int>(gridDim.x) == ev_n;
   const int ev_j = (ev_n & (kXcds - 1)) == 0 ? (blockIdx.x & (kXcds - 1)) * (ev_n / kXcds) + blockIdx.x / kXcds
                                              : static_cast<int>(blockIdx.x);
@@ -501,10 +524,312 @@ __global__ void __launch_bounds__(kThreads) sparse_fa_kernel(const FaParams p) {
         for (int j = 0; j < 8; ++j) reinterpret_cast<u32x4*>(dst)[j] = z;
         if (p.lse && g == 0) p.lse[q_tok * p.num_heads + head] = kNegInf;
       }
-      if (wv == 4) fetch_next((row_it + 1) & 1);
+      if (wv == kFetchWave) fetch_next((row_it + 1) & 1);
       continue;
     }
 
+    f32x16 o_acc[4];
+#pragma unroll
+    for (int dt = 0; dt < 4; ++dt)
+#pragma unroll
+      for (int i = 0; i < 16; ++i) o_acc[dt][i] = 0.f;
+    float m_run = 0.f, d_part = 0.f;
+    if constexpr (kPipe) {
+      // ---- software-pipelined row (one kv group) ----
+      // A step is 32 keys.  In step t a wavefront issues the MFMAs of S(t+1) = K(t+1).Q^T and of
+      // O^T += V(t-1)^T.P(t-1)^T, and between them, instruction by instruction, the softmax of S(t)
+      // (max, exp2, rounding, row sum -> P(t)), the operand reads of later MFMAs and the copies of
+      // later steps: the vector ALU work of a step runs in the shadow of its own MFMAs instead of in
+      // a phase of its own.  LDS holds four K and four V buffers of 32 keys (8 KB each).  The K
+      // operands of a step are read one step ahead (K(t) in step t-2), the V^T operands four slots
+      // ahead (V(t) in the second half of step t and the first half of step t+1); a copy is issued as
+      // soon as its buffer is dead: K three steps, V two steps before its first read.  One barrier
+      // per step.
+      constexpr int kStep = 32, kBuf = kStep * kRowBytes;
+      // K buffers 0..2 | V buffer 0 | K buffer 3 | V buffers 1..3; Q is staged in the upper 32 KB, so
+      // that K(0..2) and V(0) can be requested together with it
+      auto kbuf = [&](int i) { return static_cast<uint32_t>(i * kBuf + (i == 3 ? kBuf : 0)); };
+      auto vbuf = [&](int i) { return static_cast<uint32_t>((4 + i) * kBuf - (i == 0 ? kBuf : 0)); };
+      const uint32_t lds0 = static_cast<uint32_t>(reinterpret_cast<uintptr_t>((lds_void*)smem));
+      const int last_valid = min(kBlockKV, kv_len - s_blk[nb - 1] * kBlockKV);
+      const int n_steps = 4 * (nb - 1) + ((last_valid + kStep - 1) / kStep);
+      const int kv_head = head / p.kv_group;
+      const uint8_t* k_head = reinterpret_cast<const uint8_t*>(
+          kp + static_cast<int64_t>(kv_begin) * p.k_sn + static_cast<int64_t>(kv_head) * p.k_sh);
+      const uint8_t* v_head = reinterpret_cast<const uint8_t*>(
+          vp + static_cast<int64_t>(kv_begin) * p.v_sn + static_cast<int64_t>(kv_head) * p.v_sh);
+      // K and V copies go through buffer descriptors that end with the request's last key: a copy
+      // that reaches past it (the ragged last 32 keys, or the copies a row's last steps issue for steps
+      // that do not exist) touches no memory there, so the loop issues its copies unconditionally.
+      // Offsets are 32 bits: the launcher picks this kernel only for kv spans below 4 GiB.
+      const uint32_t k_sn2 = static_cast<uint32_t>(p.k_sn) * sizeof(T), v_sn2 = static_cast<uint32_t>(p.v_sn) * sizeof(T);
+      const __amdgpu_buffer_rsrc_t k_rsrc = __builtin_amdgcn_make_buffer_rsrc(
+          const_cast<uint8_t*>(k_head), 0, static_cast<uint32_t>(kv_len - 1) * k_sn2 + kRowBytes, 0x00020000);
+      const __amdgpu_buffer_rsrc_t v_rsrc = __builtin_amdgcn_make_buffer_rsrc(
+          const_cast<uint8_t*>(v_head), 0, static_cast<uint32_t>(kv_len - 1) * v_sn2 + kRowBytes, 0x00020000);
+      // a lane's part of a copy: row 4 * qs + lane / 16 of a 16-row group, swizzled 16-byte chunk
+      uint32_t k_voff = static_cast<uint32_t>(4 * qs + cp_row) * k_sn2 + cp_chunk * static_cast<uint32_t>(sizeof(T));
+      uint32_t v_voff = static_cast<uint32_t>(4 * qs + cp_row) * v_sn2 + cp_chunk * static_cast<uint32_t>(sizeof(T));
+      asm volatile("" : "+v"(k_voff), "+v"(v_voff));
+      const uint32_t m0_base = lds0 + qs * 1024;  // LDS address of this wavefront's part of buffer offset 0
+      // 64 lanes x 16 bytes of 4 rows, global -> LDS (see copy16_to_lds), addressed through a descriptor:
+      // lane offset + scalar offset
+      auto copy_desc = [&](__amdgpu_buffer_rsrc_t rsrc, uint32_t voff, uint32_t soff, uint32_t lds_addr) __attribute__((always_inline)) {
+        asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tbuffer_load_dwordx4 %1, %2, %3 offen lds"
+                     :
+                     : "s"(lds_addr), "v"(voff), "s"(rsrc), "s"(soff)
+                     : "memory", "m0");
+      };
+      auto step_start = [&](int t) { return s_blk[t >> 2] * kBlockKV + (t & 3) * kStep; };
+      // the 32 keys of step t (two copy instructions per wavefront) -> their LDS buffer
+      auto copy_k = [&](int t) __attribute__((always_inline)) {
+        const uint32_t soff = static_cast<uint32_t>(__builtin_amdgcn_readfirstlane(step_start(t))) * k_sn2;
+#pragma unroll
+        for (int j = 0; j < 2; ++j) copy_desc(k_rsrc, k_voff, soff + j * 16 * k_sn2, m0_base + kbuf(t & 3) + j * 4096);
+      };
+      auto copy_v = [&](int t) __attribute__((always_inline)) {
+        const uint32_t soff = static_cast<uint32_t>(__builtin_amdgcn_readfirstlane(step_start(t))) * v_sn2;
+#pragma unroll
+        for (int j = 0; j < 2; ++j) copy_desc(v_rsrc, v_voff, soff + j * 16 * v_sn2, m0_base + vbuf(t & 3) + j * 4096);
+      };
+
+      // prologue: Q, K(0..2), V(0) requested together
+      {
+        const uint8_t* q_head = reinterpret_cast<const uint8_t*>(
+            qp + static_cast<int64_t>(q_begin) * p.q_sn + static_cast<int64_t>(head) * p.q_sh);
+#pragma unroll
+        for (int n = 0; n < 8; ++n) {
+          int r = 4 * (4 * n + qs) + cp_row;
+          r = r < q_rows ? r : q_rows - 1;  // ragged last q block: re-read the last row
+          copy16_to_lds(q_head, static_cast<uint32_t>((r * p.q_sn + cp_chunk) * sizeof(T)),
+                        lds0 + 4 * kBuf + qs * 1024 + n * 4096);
+        }
+      }
+      copy_k(0);
+      if (n_steps > 1) copy_k(1);
+      if (n_steps > 2) copy_k(2);
+      copy_v(0);
+      __builtin_amdgcn_s_waitcnt(0x0f70);  // vmcnt(0)
+      __builtin_amdgcn_s_barrier();
+      x8 qreg[8], kop[4], vop[4];
+      u32x4 pA[2], pB[2];  // P of a step: 2 x 8 rounded values, as 32-bit pairs
+      f32x16 sA, sB;
+      {
+        int q_rd_base = k_rd_base, q_rd_x = k_rd_x;
+        asm volatile("" : "+v"(q_rd_base), "+v"(q_rd_x));
+        const uint8_t* qt = smem + 4 * kBuf + qs * 32 * kRowBytes + q_rd_base;
+#pragma unroll
+        for (int ks = 0; ks < 8; ++ks) qreg[ks] = *reinterpret_cast<const x8*>(qt + (q_rd_x ^ (ks << 5)));
+        // the softmax scale (log2 domain) is folded into Q, so S^T needs no multiply
+#pragma unroll
+        for (int ks = 0; ks < 8; ++ks)
+#pragma unroll
+          for (int e = 0; e < 8; ++e) qreg[ks][e] = static_cast<T>(static_cast<float>(qreg[ks][e]) * c);
+      }
+      // LDS address of the K operand reads of a step, without the buffer's offset (an immediate of the
+      // read): read i is at kx0 ^ (i << 5) (row bits, chunk bits and the 256-byte aligned base of
+      // the array do not overlap)
+      typedef __attribute__((address_space(3))) const x8 lds_x8;
+      uint32_t kx0 = lds0 + static_cast<uint32_t>(k_rd_base | k_rd_x);
+      asm volatile("" : "+v"(kx0));
+      // K operand slice i (16 d) of the step whose K is in buffer `buf`
+      auto read_k = [&](uint32_t kx, int buf, int i) __attribute__((always_inline)) {
+        return *reinterpret_cast<lds_x8*>(static_cast<uintptr_t>((kx ^ (i << 5)) + kbuf(buf)));
+      };
+      // the same for the V^T operand reads: the eight lane offsets with the array's base added
+      uint32_t vrd[4][2];
+#pragma unroll
+      for (int dt = 0; dt < 4; ++dt)
+#pragma unroll
+        for (int hi = 0; hi < 2; ++hi) {
+          vrd[dt][hi] = lds0 + static_cast<uint32_t>(v_rd_off[dt][hi]);
+          asm volatile("" : "+v"(vrd[dt][hi]));
+        }
+      // V^T operand (kk, dt) of the step whose V is in buffer `buf`: 16 keys x 32 d, transposed
+      auto read_v = [&](int buf, int kk, int dt) __attribute__((always_inline)) {
+        union {
+          s16x4 h[2];
+          x8 v;
+        } a;
+        const uint32_t off = vbuf(buf) + kk * 16 * kRowBytes;
+        a.h[0] = __builtin_amdgcn_ds_read_tr16_b64_v4i16(reinterpret_cast<lds_s16x4*>(static_cast<uintptr_t>(vrd[dt][0] + off)));
+        a.h[1] = __builtin_amdgcn_ds_read_tr16_b64_v4i16(reinterpret_cast<lds_s16x4*>(static_cast<uintptr_t>(vrd[dt][1] + off)));
+        return a.v;
+      };
+#pragma unroll
+      for (int i = 0; i < 16; ++i) sA[i] = 0.f;
+      {
+        x8 k0[8];
+#pragma unroll
+        for (int i = 0; i < 8; ++i) k0[i] = read_k(kx0, 0, i);
+#pragma unroll
+        for (int i = 0; i < 8; ++i) sA = TT::mfma(k0[i], qreg[i], sA);
+      }
+      __builtin_amdgcn_sched_barrier(0);
+      // (a row of one step reads a buffer nobody filled: the result is never used)
+#pragma unroll
+      for (int i = 0; i < 4; ++i) kop[i] = read_k(kx0, 1, i);
+      // (a row's first step multiplies P(-1) = 0 by what vop holds and by what its first half reads
+      // from V buffer 3, where Q was staged: both must be finite whatever Q holds)
+#pragma unroll
+      for (int i = 0; i < 4; ++i)
+#pragma unroll
+        for (int e = 0; e < 8; ++e) vop[i][e] = static_cast<T>(0.f);
+#pragma unroll
+      for (int e = 0; e < 4; ++e) pA[0][e] = pA[1][e] = pB[0][e] = pB[1][e] = 0u;
+      __builtin_amdgcn_s_waitcnt(0xc07f);  // lgkmcnt(0): Q and K(0) are in registers
+      __builtin_amdgcn_s_barrier();        // ... of every wavefront: their LDS space is free
+      {
+        // V buffer 3 (read by the first step as "V(-1)"), and for a row of fewer than four steps
+        // every V buffer it does not fill (read by its padded steps), must not hold Q any more
+        const u32x4 z = {0u, 0u, 0u, 0u};
+        for (int b = min(n_steps, 3); b < 4; ++b) {
+          u32x4* vb = reinterpret_cast<u32x4*>(smem + vbuf(b));
+          vb[tid] = z;
+          vb[tid + kGroupThreads] = z;
+        }
+      }
+      if (n_steps > 1) {
+        copy_v(1);
+        copy_k(min(3, n_steps - 1));  // (kept to four instructions per group: the loop's waits count them)
+      }
+
+#pragma unroll
+      for (int i = 0; i < 16; ++i) sB[i] = 0.f;  // S(1) accumulates from the reference point 0, moved by the first step
+      // Block numbers of the row's list as scalars: blk0 = the block of the current four steps, blk1
+      // the one after it.  They come from a register that holds 64 consecutive entries of the list,
+      // one per lane, refilled every 64 blocks: the loop itself reads no list from LDS (the wait
+      // for such a read would also wait for the operand reads in flight).
+      int blk_win = s_blk[min(lane, nb - 1)];
+      int blk0 = 0, blk1 = 0;
+      typedef __attribute__((ext_vector_type(2))) T x2;
+      const x2 ones2 = {static_cast<T>(1.0f), static_cast<T>(1.0f)};
+      // One step (kB = t % 4 picks the LDS buffers).  Straight-line code apart from small
+      // wavefront-uniform branches, so that the accumulators stay where they are.  Eight slots, each:
+      // one MFMA of S(t+1), one K operand read of step t+2, one MFMA of P(t-1).V(t-1), the V^T operand
+      // needed four slots later, and the softmax of two values of S(t): exp2, rounding, row sum; the
+      // accumulator that held them is set to the reference point for its next use (S(t+2)
+      // accumulates onto -m_run, so that p = exp2(S) with no subtraction).
+      auto do_step = [&](int t, auto buf_tag, f32x16& s_cur, f32x16& s_next, u32x4 (&p_prev)[2], u32x4 (&p_cur)[2]) __attribute__((always_inline)) {
+        constexpr int kB = decltype(buf_tag)::value;
+        // V(t) and K(t+2), first read in this step, were requested two barriers ago: they have landed
+        // once only the four copies of the last barrier are outstanding; after the barrier that holds
+        // for every wavefront
+        __builtin_amdgcn_s_waitcnt(0x0f70 | 4);  // vmcnt(4)
+        // (the buffers that this step's copies overwrite were last read in the first half of step t-1:
+        // the twelve operand reads of its second half may still be in flight)
+        __builtin_amdgcn_s_waitcnt(0xcc7f);  // lgkmcnt(12)
+        __builtin_amdgcn_s_barrier();
+        // this step's copies: V(t+2) into the buffer of V(t-2) and K(t+4) into the buffer of K(t), both
+        // last read in step t-1.  Their scalar offsets are worked out here from the block numbers held
+        // in scalar registers; the four instructions go out between the MFMAs below (V first, then
+        // K).  Steps past the row's end copy a block again or nothing (see the descriptors).
+        const uint32_t v_soff = static_cast<uint32_t>(((kB + 2) < 4 ? blk0 : blk1) * kBlockKV + ((kB + 2) & 3) * kStep) * v_sn2;
+        const uint32_t k_soff = static_cast<uint32_t>(blk1 * kBlockKV + kB * kStep) * k_sn2;
+        // (a row is padded to a multiple of four steps; a padded step has no keys: p = 0, against V
+        // operands read from buffers that hold earlier steps of the same row)
+        const int valid = t < n_steps ? min(kStep, kv_len - (blk0 * kBlockKV + kB * kStep)) : 0;
+        if (valid < kStep) {
+#pragma unroll
+          for (int i = 0; i < 16; ++i) {
+            const int kv = (i >> 2) * 8 + g * 4 + (i & 3);
+            if (kv >= valid) s_cur[i] = -INFINITY;  // p = 0
+          }
+        }
+        float mx = s_cur[0];
+#pragma unroll
+        for (int i = 1; i < 16; ++i) mx = fmaxf(mx, s_cur[i]);
+        mx = max_across_halves(mx);  // row max relative to m_run
+        const bool first = t == 0;
+        // The reference point moves always on a row's first step, afterwards only past a 2^8
+        // overshoot (a rare, wavefront-uniform branch that changes registers in place): S(t), the
+        // accumulator of S(t+1), which holds the old point, and the row sum move now; O, which still
+        // receives P(t-1).V(t-1) at the old point in this step, is rescaled at the step's end.
+        const bool moved = first || __builtin_expect(__any(mx > kLazyLog2), 0);
+        float o_scale = 1.f;
+        if (moved) {
+          const float delta = first ? mx : fmaxf(mx, 0.f);
+          if (!first) {
+            o_scale = __builtin_amdgcn_exp2f(-delta);
+            d_part *= o_scale;
+          }
+          m_run += delta;
+#pragma unroll
+          for (int i = 0; i < 16; ++i) s_cur[i] -= delta;
+#pragma unroll
+          for (int i = 0; i < 16; ++i) s_next[i] -= delta;
+        }
+        const f32x2 neg_m2 = {-m_run, -m_run};
+        // (made opaque once per step: otherwise the eight read offsets are worked out once per
+        // kernel and live in eight registers, which the loop does not have)
+        uint32_t kx = kx0;
+        asm volatile("" : "+v"(kx));
+        float psum = 0.f;
+        __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+        for (int i = 0; i < 8; ++i) {
+          s_next = TT::mfma(kop[i & 3], qreg[i], s_next);
+          // the operand of the S MFMA four slots on: second half of K(t+1), then first half of K(t+2)
+          kop[i & 3] = i < 4 ? read_k(kx, (kB + 1) & 3, i + 4) : read_k(kx, (kB + 2) & 3, i - 4);
+          o_acc[i & 3] = TT::mfma(vop[i & 3], __builtin_bit_cast(x8, p_prev[i >> 2]), o_acc[i & 3]);
+          // the operand of the P.V MFMA four slots on: second half of V(t-1), then first half of V(t)
+          vop[i & 3] = i < 4 ? read_v((kB + 3) & 3, 1, i) : read_v(kB, 0, i - 4);
+          // (the two values are pinned to this slot: without the empty statements the compiler
+          // gathers all exponentials of a step in front of its MFMAs)
+          float e0 = s_cur[2 * i], e1 = s_cur[2 * i + 1];
+          asm volatile("" : "+v"(e0), "+v"(e1));
+          const x2 pk = {static_cast<T>(__builtin_amdgcn_exp2f(e0)), static_cast<T>(__builtin_amdgcn_exp2f(e1))};
+          uint32_t pu = __builtin_bit_cast(uint32_t, pk);
+          // the row sum is taken over the rounded p, as the reference does
+          if constexpr (std::is_same<T, __bf16>::value) {
+            psum = __builtin_amdgcn_fdot2_f32_bf16(pk, ones2, psum, false);
+          } else {
+            psum = __builtin_amdgcn_fdot2(pk, ones2, psum, false);
+          }
+          // (the accumulator that held the two values is set to the reference point for its next use)
+          f32x2 r01 = neg_m2;
+          asm volatile("" : "+v"(pu), "+v"(psum), "+v"(r01));
+          p_cur[i >> 2][i & 3] = pu;
+          s_cur[2 * i] = r01[0];
+          s_cur[2 * i + 1] = r01[1];
+          if (i == 1 || i == 3) {
+            copy_desc(v_rsrc, v_voff, v_soff + (i >> 1) * 16 * v_sn2, m0_base + vbuf((kB + 2) & 3) + (i >> 1) * 4096);
+          } else if (i == 5 || i == 7) {
+            copy_desc(k_rsrc, k_voff, k_soff + ((i - 4) >> 1) * 16 * k_sn2, m0_base + kbuf(kB) + ((i - 4) >> 1) * 4096);
+          }
+          __builtin_amdgcn_sched_barrier(0);
+        }
+        d_part += psum;
+        if (moved && !first) {
+#pragma unroll
+          for (int dt = 0; dt < 4; ++dt)
+#pragma unroll
+            for (int i = 0; i < 16; ++i) o_acc[dt][i] *= o_scale;
+        }
+      };
+      using B0 = std::integral_constant<int, 0>;
+      using B1 = std::integral_constant<int, 1>;
+      using B2 = std::integral_constant<int, 2>;
+      using B3 = std::integral_constant<int, 3>;
+      for (int t = 0; t < n_steps; t += 4) {
+        const int bi = t >> 2;
+        blk0 = __builtin_amdgcn_readlane(blk_win, bi & 63);
+        if (((bi + 1) & 63) == 0) blk_win = s_blk[min(bi + 1 + lane, nb - 1)];
+        blk1 = __builtin_amdgcn_readlane(blk_win, (bi + 1) & 63);
+        do_step(t, B0{}, sA, sB, pB, pA);
+        do_step(t + 1, B1{}, sB, sA, pA, pB);
+        do_step(t + 2, B2{}, sA, sB, pB, pA);
+        do_step(t + 3, B3{}, sB, sA, pA, pB);
+      }
+      // P.V of the last step (real or padded; its V is in buffer 3, vop holds the first half)
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        o_acc[i] = TT::mfma(vop[i], __builtin_bit_cast(x8, pB[0]), o_acc[i]);
+        vop[i] = read_v(3, 1, i);
+      }
+#pragma unroll
+      for (int i = 0; i < 4; ++i) o_acc[i] = TT::mfma(vop[i], __builtin_bit_cast(x8, pB[1]), o_acc[i]);
+    } else {
     // Q operand.  A lane needs q row l32 of its sub-tile, 16 bytes out of every 32 (fp8: 32 of 64):
     // fetched straight from memory that is 64 scattered pieces per instruction (measured: ~4 k
     // cycles per row).  The 128 q rows are copied into LDS like a K tile instead (64 rows per kv
@@ -559,17 +884,11 @@ __global__ void __launch_bounds__(kThreads) sparse_fa_kernel(const FaParams p) {
     const int kv_head = head / p.kv_group;
     const float* const s_ksc = s_ksc2[row_it & 1];
 
-    f32x16 o_acc[4];
-#pragma unroll
-    for (int dt = 0; dt < 4; ++dt)
-#pragma unroll
-      for (int i = 0; i < 16; ++i) o_acc[dt][i] = 0.f;
     // Running reference point m_run of the softmax (log2 domain), partial sum d_part.  S^T is formed
     // relative to m_run: the MFMA accumulator starts at -m_run (c_init), so p = exp2(S^T) directly.
     // m_run is set to the tile's exact row max on the first tile and afterwards only raised when a
     // row's new max exceeds it by more than kLazyLog2 (p then stays <= 2^kLazyLog2, harmless in
     // fp32 / bf16 / fp16): the rescale of O leaves the steady-state path.
-    float m_run = 0.f, d_part = 0.f;
     f32x16 c_init;
 #pragma unroll
     for (int i = 0; i < 16; ++i) c_init[i] = 0.f;
@@ -976,35 +1295,53 @@ __global__ void __launch_bounds__(kThreads) sparse_fa_kernel(const FaParams p) {
     }
     for (int i = calls_mine; i < calls_all; ++i) __builtin_amdgcn_s_barrier();
     if (my_tiles == 0) m_run = kNegInf;  // nothing seen: weight 0 in the merge
+    }  // !kPipe
 
     // ---- merge the two kv groups through LDS, then write the row ----
     __syncthreads();  // all tile reads done: the tile buffers can be reused
     f32x4* mo = reinterpret_cast<f32x4*>(smem);
     float* md = reinterpret_cast<float*>(smem + kMergeOBytes);
-    if (kg == 1) {
+    if constexpr (kGroups == 2) {
+      if (kg == 1) {
 #pragma unroll
-      for (int dt = 0; dt < 4; ++dt)
+        for (int dt = 0; dt < 4; ++dt)
 #pragma unroll
-        for (int i4 = 0; i4 < 4; ++i4) {
-          f32x4 t4;
+          for (int i4 = 0; i4 < 4; ++i4) {
+            f32x4 t4;
 #pragma unroll
-          for (int j = 0; j < 4; ++j) t4[j] = o_acc[dt][i4 * 4 + j];
-          mo[(qs * 16 + dt * 4 + i4) * 64 + lane] = t4;
-        }
-      md[(qs * 64 + lane) * 2 + 0] = m_run;
-      md[(qs * 64 + lane) * 2 + 1] = d_part;
+            for (int j = 0; j < 4; ++j) t4[j] = o_acc[dt][i4 * 4 + j];
+            mo[(qs * 16 + dt * 4 + i4) * 64 + lane] = t4;
+          }
+        md[(qs * 64 + lane) * 2 + 0] = m_run;
+        md[(qs * 64 + lane) * 2 + 1] = d_part;
+      }
+      __syncthreads();
     }
-    __syncthreads();
-    if (wv == 4) fetch_next((row_it + 1) & 1);
+    if (wv == kFetchWave) fetch_next((row_it + 1) & 1);
     float m_all = 0.f, d_all = 0.f;  // kv group 0: row maximum and row sum over both groups
     // A lane owns one q row and runs of four d: stored from here, a row would leave as 32 scattered
     // 8-byte pieces per instruction (measured: ~12 k cycles per row).  The finished row goes through
     // a padded LDS tile instead and leaves in 16-byte pieces, 16 consecutive lanes per 256-byte row.
     int ln_out = l32;
     asm volatile("" : "+v"(ln_out));  // (not hoisted out of the row loop and spilled)
-    uint8_t* const out_row = smem + kOutTileOff + (qs * 32 + ln_out) * kOutRowBytes;
+    uint8_t* const out_row = smem + G::kOutOff + (qs * 32 + ln_out) * kOutRowBytes;
     bool store_row = parts == 1;
-    if (kg == 0) {
+    if constexpr (kGroups == 1) {
+      // one kv group: the accumulators hold the whole row
+      const float d_tot = d_part + __shfl_xor(d_part, 32, 64);
+      const float inv = __builtin_amdgcn_rcpf(d_tot);
+#pragma unroll
+      for (int dt = 0; dt < 4; ++dt)
+#pragma unroll
+        for (int i4 = 0; i4 < 4; ++i4) {
+          x4 out;
+#pragma unroll
+          for (int j = 0; j < 4; ++j) out[j] = static_cast<T>(o_acc[dt][i4 * 4 + j] * inv);
+          *reinterpret_cast<x4*>(out_row + (dt * 32 + i4 * 8 + g * 4) * sizeof(T)) = out;
+        }
+      if (row_ok && p.lse && g == 0) p.lse[q_tok * p.num_heads + head] = __builtin_amdgcn_logf(d_tot) + m_run;
+    }
+    if (kGroups == 2 && kg == 0) {
       const float m1 = md[(qs * 64 + lane) * 2 + 0], d1 = md[(qs * 64 + lane) * 2 + 1];
       const float m = fmaxf(m_run, m1);
       const float a0 = __builtin_amdgcn_exp2f(m_run - m);
@@ -1048,7 +1385,7 @@ __global__ void __launch_bounds__(kThreads) sparse_fa_kernel(const FaParams p) {
         d_all = d_tot;
       }
     }
-    if (parts > 1) {
+    if (kGroups == 2 && parts > 1) {
       // Whoever comes last combines the parts and writes the row.  A workgroup that finds every
       // other part arrived already need not publish its own; otherwise it publishes, then counts
       // itself in, and may still turn out to be the last.
@@ -1159,14 +1496,15 @@ __global__ void __launch_bounds__(kThreads) sparse_fa_kernel(const FaParams p) {
       // per kernel, spilled, and every reload waits for the store before it)
       int ln = lane;
       asm volatile("" : "+v"(ln));
-      const int r0 = wv * 16 + (ln >> 4), chunk = ln & 15;
-      u32x4 v[4];
+      constexpr int kRowsPerWave = kBlockQ / kWaves;
+      const int r0 = wv * kRowsPerWave + (ln >> 4), chunk = ln & 15;
+      u32x4 v[kRowsPerWave / 4];
 #pragma unroll
-      for (int i = 0; i < 4; ++i)
-        v[i] = *reinterpret_cast<const u32x4*>(smem + kOutTileOff + (r0 + i * 4) * kOutRowBytes + chunk * 16);
+      for (int i = 0; i < kRowsPerWave / 4; ++i)
+        v[i] = *reinterpret_cast<const u32x4*>(smem + G::kOutOff + (r0 + i * 4) * kOutRowBytes + chunk * 16);
       T* d0 = dst + static_cast<int64_t>(r0) * p.o_sn + chunk * 8;
 #pragma unroll
-      for (int i = 0; i < 4; ++i)
+      for (int i = 0; i < kRowsPerWave / 4; ++i)
         if (r0 + i * 4 < q_rows) *reinterpret_cast<u32x4*>(d0 + i * 4 * p.o_sn) = v[i];
     }
   }
@@ -1182,30 +1520,40 @@ __global__ void __launch_bounds__(kThreads) sparse_fa_kernel(const FaParams p) {
   }
 }
 
-template <typename T, bool kFp8, bool kQLo, bool kKLo>
+template <typename T, bool kFp8, bool kQLo, bool kKLo, int kGroups = 2, bool kPipe = false>
 int launch(const FaParams& p, int64_t max_rows, hipStream_t stream) {
-  constexpr int kSmemBytes = Geom<kFp8, kKLo>::kSmemBytes;
+  constexpr int kSmemBytes = Geom<kFp8, kKLo, kGroups>::kSmemBytes;
   // (the attribute belongs to the kernel's code object on one device: set once per device; the flags
   // are atomic because host threads may launch concurrently, and setting it twice is harmless)
   static std::atomic<bool> attr_set[64] = {};
   int dev = 0;
   FO_HIP_CALL(hipGetDevice(&dev));
   if (dev < 0 || dev >= 64 || !attr_set[dev].load(std::memory_order_acquire)) {
-    FO_HIP_CALL(hipFuncSetAttribute(reinterpret_cast<const void*>(&sparse_fa_kernel<T, kFp8, kQLo, kKLo>),
+    FO_HIP_CALL(hipFuncSetAttribute(reinterpret_cast<const void*>(&sparse_fa_kernel<T, kFp8, kQLo, kKLo, kGroups, kPipe>),
                                     hipFuncAttributeMaxDynamicSharedMemorySize, kSmemBytes));
     if (dev >= 0 && dev < 64) attr_set[dev].store(true, std::memory_order_release);
   }
   int num_cu = fo_num_cu();
   if (num_cu <= 0) return fo::fail(FO_ERR_HIP, "sparse_fa: no device");
-  int64_t grid = num_cu;  // one persistent workgroup per CU (LDS bound)
+  int64_t grid = num_cu * (3 - kGroups);  // persistent workgroups: one per CU, or two of one kv group each (LDS bound)
   // (with even shares every workgroup may hold a part of a row; otherwise at most one row each)
   if (!(p.split_ws && p.shares) && grid > max_rows) grid = max_rows;
-  sparse_fa_kernel<T, kFp8, kQLo, kKLo><<<static_cast<unsigned>(grid), kThreads, kSmemBytes, stream>>>(p);
+  sparse_fa_kernel<T, kFp8, kQLo, kKLo, kGroups, kPipe><<<static_cast<unsigned>(grid), kGroups * kGroupThreads, kSmemBytes, stream>>>(p);
   FO_CHECK_LAUNCH();
   return FO_OK;
 }
 
 }  // namespace
+
+namespace {
+std::atomic<int> g_variant{0};
+}
+
+extern "C" int fo_sparse_fa_set_variant(int variant) {
+  FO_REQUIRE(variant >= 0 && variant <= 2, "sparse_fa: variant must be 0 (automatic), 1 or 2");
+  g_variant.store(variant, std::memory_order_relaxed);
+  return FO_OK;
+}
 
 extern "C" int64_t fo_sparse_fa_split_workspace_bytes(void) {
   // two areas per share, one share per workgroup = per CU
@@ -1282,8 +1630,24 @@ extern "C" int fo_sparse_fa_run(const void* q, const void* k, const void* v, voi
   p.num_heads = num_heads; p.kv_group = num_heads / num_kv_heads; p.n_q_blocks = n_q_blocks; p.n_kv_blocks = n_kv_blocks;
   p.sm_scale_log2 = sm_scale * 1.44269504088896340736f;
   hipStream_t s = static_cast<hipStream_t>(stream);
-  if (dtype == FO_BF16) return launch<__bf16, false, false, false>(p, max_rows, s);
-  if (dtype == FO_F16) return launch<_Float16, false, false, false>(p, max_rows, s);
+  // Long lists (many rows per CU) run as two independent 4-wavefront workgroups per CU with the
+  // software-pipelined loop; short ones as one 8-wavefront workgroup whose two kv groups share a row
+  // (half the latency per row, and rows can be cut into even shares).  The list's length lives on the
+  // device: the choice is made from its upper bound max_rows, unless fo_sparse_fa_set_variant() fixed
+  // it.  The one-group form needs 16-bit operands, at most 3072 kv blocks per request and kv spans
+  // below 4 GiB (32-bit copy offsets): n_kv_blocks, the batch's total, bounds both.
+  const int64_t span = static_cast<int64_t>(n_kv_blocks) * kBlockKV * 2;
+  const bool one_group_ok = (dtype == FO_BF16 || dtype == FO_F16) && n_kv_blocks > 0 &&
+                            n_kv_blocks <= kMaxRowBlocksOneGroup && span * k_stride_n < (int64_t(1) << 32) &&
+                            span * v_stride_n < (int64_t(1) << 32);
+  const int variant = g_variant.load(std::memory_order_relaxed);
+  const bool one_group = one_group_ok && (variant == 1 || (variant == 0 && max_rows >= static_cast<int64_t>(8) * fo_num_cu()));
+  if (dtype == FO_BF16)
+    return one_group ? launch<__bf16, false, false, false, 1, true>(p, max_rows, s)
+                     : launch<__bf16, false, false, false, 2>(p, max_rows, s);
+  if (dtype == FO_F16)
+    return one_group ? launch<_Float16, false, false, false, 1, true>(p, max_rows, s)
+                     : launch<_Float16, false, false, false, 2>(p, max_rows, s);
   if (k_lo != nullptr) return launch<__bf16, true, true, true>(p, max_rows, s);
   if (q_lo != nullptr) return launch<__bf16, true, true, false>(p, max_rows, s);
   return launch<__bf16, true, false, false>(p, max_rows, s);

@@ -187,6 +187,14 @@ int fo_decode_sparse_static(const uint8_t* sparse_info, const uint8_t* sparse_kv
  * Supported: D = 128, block_q = 128, block_kv = 128.  max_rows bounds the number of rows.
  * ------------------------------------------------------------------------------------------- */
 int64_t fo_sparse_fa_split_workspace_bytes(void);
+/* Which form of the kernel fo_sparse_fa_run launches (process-wide; no counterpart in the reference):
+ * 0 = automatic (the default): lists whose upper bound max_rows is at least 8 rows per CU run as two
+ * independent 4-wavefront workgroups per CU, one row each, with a software-pipelined loop; shorter
+ * ones as one 8-wavefront workgroup per CU whose two halves share a row.  1 / 2 force the first /
+ * second form where it applies (the first needs 16-bit q, k, v, at most 3072 kv blocks in the batch
+ * and kv strides that keep a request's keys within 4 GiB).  Results agree within the stated
+ * tolerances, not bit for bit.  For tests and measurements. */
+int fo_sparse_fa_set_variant(int variant);
 int fo_sparse_fa_run(const void* q, const void* k, const void* v, void* o, float* lse, int dtype,
                      const void* q_lo, const void* k_lo, const float* q_scale, const float* k_scale,
                      int64_t q_stride_n,

@@ -16,6 +16,18 @@ pytestmark = pytest.mark.gpu
 MAX_ABS, REL_L2 = 2e-2, 1e-2
 
 
+@pytest.fixture(autouse=True, params=["auto", "one_group"])
+def kernel_variant(request):
+    """Every test of this module runs twice: with the kernel form chosen from the list's size (short
+    lists: one 8-wavefront workgroup per CU shares a row) and with the form for long lists forced
+    (two 4-wavefront workgroups per CU, software-pipelined loop), which these small cases would not
+    reach on their own.  Inputs the second form does not take (fp8) run the first one either way."""
+    from flashomni_amd import _lib
+    _lib.check(_lib.lib().fo_sparse_fa_set_variant(1 if request.param == "one_group" else 0))
+    yield request.param
+    _lib.check(_lib.lib().fo_sparse_fa_set_variant(0))
+
+
 def _run_case(dev, ql, kl, heads, dtype, seed, pa=0.75, pk=0.5, force=None, is_full=False,
               return_lse=False, layout="NHD"):
     import flashomni_amd as fo
