@@ -11,7 +11,12 @@ The JSON line also carries
     fraction of the MI355X peak that bounds it,
   * ``roofline``: the dominant kernel (sparse FlashAttention at the FLUX shape) measured with HIP
     events on the launch stream,
-  * ``cpu_baseline``: the fp32 dense-masked CPU path (the oracle) timed on this box's host cores.
+  * ``cpu_baseline``: the fp32 CPU path (the oracle) timed on this box's host cores: the whole FLUX
+    layer, and under ``c3`` / ``c4`` a sample of the big configs' attention rows and token blocks
+    with the extrapolation to the whole config labelled as such.
+
+Every attention config also carries ``run_dropin``: the reference's call sequence
+``wrapper.run(q, k, v, sparse_info, sparse_kv_info, indptrs)`` with a fresh decode in every call.
 
 Usage: python bench.py [--gpus 1] [--steps K] [--warmup W] [--configs 0,1,2,3,4] [--no-cpu]
 """
@@ -37,16 +42,32 @@ def log(*a):
     print(*a, file=sys.stderr, flush=True)
 
 
+def kernel_source_hash():
+    import hashlib
+    with open(os.path.join(ROOT, "flashomni_amd", "csrc", "sparse_fa.hip"), "rb") as f:
+        return hashlib.sha256(f.read()).hexdigest()[:16]
+
+
 def traffic_from_profile():
     """HBM bytes per sparse-FA launch at config 0, as recorded in the committed rocprofv3 summary
-    (line ``traffic_bytes_per_launch <kernel> = <bytes>``); None when the summary has no such line."""
+    (line ``traffic_bytes_per_launch <kernel> = <bytes>``), and whether that summary was taken from the
+    kernel source this run uses (line ``kernel_source_sha256 sparse_fa.hip = <first 16 hex digits>``).
+    (None, reason) when the summary has no such line or describes another version of the kernel: a
+    counter reading of other code is not this run's traffic."""
+    value = recorded = None
     try:
         for line in open(TRAFFIC_PROFILE):
             if line.startswith("traffic_bytes_per_launch sparse_fa_kernel<bf16>"):
-                return float(line.split("=")[1].split()[0])
+                value = float(line.split("=")[1].split()[0])
+            if line.startswith("kernel_source_sha256 sparse_fa.hip"):
+                recorded = line.split("=")[1].split()[0]
     except OSError:
-        pass
-    return None
+        return None, "no counter summary"
+    if value is None:
+        return None, "no counter summary"
+    if recorded != kernel_source_hash():
+        return None, "the counter summary was taken from another version of the kernel source"
+    return value, "current"
 
 
 def time_gpu(fn, iters, warmup):
@@ -134,9 +155,10 @@ class FluxLayer:
         return self.w1.gemm_q_flops() + self.w0.attention_flops() + self.w2.gemm_o_flops(False)
 
 
-def bench_big_attention(dev, index, iters, warmup):
+def bench_big_attention(dev, index, iters, warmup, with_cpu=False):
     """Configs 3 / 4 attention at full size (tensors drawn on the GPU: the CPU draw of 10^9 normals
-    would dominate the run; masks are the seeded CPU ones)."""
+    would dominate the run; masks are the seeded CPU ones).  with_cpu: also time the oracle on a sample
+    of the same rows (second return value)."""
     import flashomni_amd as fo
     from flashomni_amd.workloads import make_workload
     wl = make_workload(index, tensors=False)
@@ -159,6 +181,10 @@ def bench_big_attention(dev, index, iters, warmup):
     ms = time_gpu(lambda: w.run(q, k, v, *args, out=out, reuse_decoded=True), iters, warmup)
     res["sparse_fa_bf16"] = entry(ms, flops=wl.attention_flops())
     res["sparse_fa_bf16"]["computed_blocks"] = wl.computed_blocks
+    # the call a user of the reference makes: decode of the symbols + attention, every time
+    ms = time_gpu(lambda: w.run(q, k, v, *args, out=out), iters, warmup)
+    res["run_dropin"] = entry(ms, flops=wl.attention_flops())
+    cpu = cpu_baseline_attention(wl, q.cpu(), k.cpu(), v.cpu()) if with_cpu else None
     if index == 4:
         # fp8 e4m3 Q.K^T (per-(head, 128-token block) absmax scales), bf16 P.V.  q as two e4m3 terms
         # (q + residual: the form that meets the fp8 accuracy contract) and as one term (faster, outside it)
@@ -168,29 +194,32 @@ def bench_big_attention(dev, index, iters, warmup):
         ms_q = time_gpu(lambda: fo.quant_fp8_block(q, wl.qo_indptr, blocks=blocks, residual=True), iters, warmup)
         res["quant_fp8_two_term"] = entry(ms_q, nbytes=4 * q.numel() + 4 * s.heads * s.n_blocks)
         q8, qs, q_lo = fo.quant_fp8_block(q, wl.qo_indptr, blocks=blocks, residual=True)
-        k8, ks = fo.quant_fp8_block(k, wl.kv_indptr, blocks=blocks)
+        k8, ks, k_lo = fo.quant_fp8_block(k, wl.kv_indptr, blocks=blocks, residual=True)
         w8 = fo.BatchFlashOmniFAWithRaggedKVWrapper(ws)
         w8.plan(wl.qo_indptr, wl.kv_indptr, s.heads, s.heads, 128, q_data_type=torch.float8_e4m3fn)
         out8 = torch.zeros_like(q)
         w8.decode(*args)
         w.run(q, k, v, *args, out=out)
-        for name, lo, peak in (("sparse_fa_fp8qk", q_lo, PEAK_BF16),
-                               # one term: QK^T half at the fp8 peak, PV half at the bf16 peak
-                               ("sparse_fa_fp8qk_one_term", None, 2.0 / (1 / PEAK_FP8 + 1 / PEAK_BF16))):
+        # two terms of q and of k (value + rounding residual under one scale): the form that meets the
+        # fp8 accuracy contract of the whole chain; two terms of q only; one term each (fastest)
+        for name, lo, klo, peak in (("sparse_fa_fp8qk", q_lo, k_lo, PEAK_BF16),
+                                    ("sparse_fa_fp8qk_q_two_term", q_lo, None, PEAK_BF16),
+                                    # one term: QK^T half at the fp8 peak, PV half at the bf16 peak
+                                    ("sparse_fa_fp8qk_one_term", None, None, 2.0 / (1 / PEAK_FP8 + 1 / PEAK_BF16))):
             ms8 = time_gpu(lambda: w8.run(q8, k8, v, *args, out=out8, q_scale=qs, k_scale=ks, q_lo=lo,
-                                          reuse_decoded=True), iters, warmup)
+                                          k_lo=klo, reuse_decoded=True), iters, warmup)
             res[name] = entry(ms8, flops=wl.attention_flops(), peak=peak)
             res[name]["frac_of_bf16_peak"] = round(res[name]["tflops"] / PEAK_BF16, 4)
             # error of the fp8 output against the bf16 kernel's output on the same inputs
             num = (out8.float() - out.float()).norm()
             res[name]["rel_l2_vs_bf16_kernel"] = round(float(num / out.float().norm()), 4)
-        del q8, k8, out8, q_lo
+        del q8, k8, out8, q_lo, k_lo
     del q, k, v, out
     torch.cuda.empty_cache()
-    return res
+    return res, cpu
 
 
-def bench_big_gemms(dev, index, iters, warmup):
+def bench_big_gemms(dev, index, iters, warmup, with_cpu=False):
     import flashomni_amd as fo
     from flashomni_amd.workloads import make_workload
     wl = make_workload(index, tensors=False)
@@ -225,15 +254,16 @@ def bench_big_gemms(dev, index, iters, warmup):
     # context, not a product path: the vendor library's dense bf16 GEMM of the same shape on this device
     ms = time_gpu(lambda: torch.matmul(x[0], wq.t()), iters, warmup)
     res["vendor_dense_gemm_same_shape"] = entry(ms, flops=2.0 * s.seq * s.hidden * s.hidden)
+    cpu = cpu_baseline_gemms(wl, x.cpu(), wq.cpu(), bq.cpu()) if with_cpu else None
     del x, wq, out, cache
     torch.cuda.empty_cache()
-    return res
+    return res, cpu
 
 
 def bench_wan_chain(dev, iters, warmup):
-    """Config 4 end to end: GEMM-Q (two-term fp8 result from its epilogue) -> fp8 quantisation of K ->
-    symbol decode + sparse FA (fp8 Q.K^T) -> GEMM-O final pass; and the same chain in bf16 without any
-    quantisation.  K, V drawn directly (the chain of the task has no K/V projection)."""
+    """Config 4 end to end: GEMM-Q (two-term fp8 result from its epilogue) -> two-term fp8 quantisation
+    of K -> symbol decode + sparse FA (fp8 Q.K^T) -> GEMM-O final pass; and the same chain in bf16 without
+    any quantisation.  K, V drawn directly (the chain of the task has no K/V projection)."""
     import flashomni_amd as fo
     from flashomni_amd.workloads import make_workload
     wl = make_workload(4, tensors=False)
@@ -271,13 +301,13 @@ def bench_wan_chain(dev, iters, warmup):
         side.wait_stream(cur)
         with torch.cuda.stream(side):
             w8.decode(info, kv_info, ip, kv_ip)
-            k8, ks = fo.quant_fp8_block(k, wl.kv_indptr, blocks=blocks)
+            k8, ks, k8lo = fo.quant_fp8_block(k, wl.kv_indptr, blocks=blocks, residual=True)
         fo.flashomni_gemm(x, wq, s.heads, info, ip, 0, bq, out=False, quant_out=(q8, q8s, q8lo))
         cur.wait_stream(side)
-        k8.record_stream(cur)
-        ks.record_stream(cur)
+        for t in (k8, ks, k8lo):
+            t.record_stream(cur)
         w8.run(q8.view(s.seq, s.heads, 128), k8, v, info, kv_info, ip, kv_ip, out=o, q_scale=q8s, k_scale=ks,
-               q_lo=q8lo.view(s.seq, s.heads, 128), reuse_decoded=True)
+               q_lo=q8lo.view(s.seq, s.heads, 128), k_lo=k8lo, reuse_decoded=True)
         return fo.flashomni_gemm_reduction(o.view(1, s.seq, s.hidden), wo, s.heads, info, ip, 0, bias=cache,
                                            is_for_cache=False)
 
@@ -342,6 +372,82 @@ def cpu_baseline(layer):
         "ms_per_step": round((t_q + t_fa + t_o) * 1e3, 2),
         "gemm_q_tflops": round(f_q / t_q / 1e12, 4), "sparse_fa_tflops": round(f_fa / t_fa / 1e12, 4),
         "gemm_o_tflops": round(f_o / t_o / 1e12, 4),
+    }
+
+
+def cpu_baseline_attention(wl, q, k, v, n_random=2048):
+    """The oracle on a sample of a big config's attention rows: the first and last q block of every
+    head that has them active (short last block, first / last kv range) plus n_random rows drawn with
+    a fixed seed.  Reports the measured time and, labelled as an extrapolation, the whole config's time
+    = symbol decode (measured in full) + row time scaled by computed kv blocks."""
+    import numpy as np
+    import oracle
+    from oracle.symbols import decode_kv_csr
+    s = wl.shape
+    n = lambda t: t.numpy()
+    t0 = time.perf_counter()
+    row_req, row_qb, row_head, ptr, _ = decode_kv_csr(
+        n(wl.packed_info), n(wl.packed_kv_info), n(wl.info_indptr), n(wl.kv_info_indptr),
+        n(wl.qo_indptr).astype(np.int64), n(wl.kv_indptr).astype(np.int64), s.heads, 128, 128, False)
+    t_decode = time.perf_counter() - t0
+    n_rows = len(row_req)
+    edge = [i for i in range(n_rows) if row_qb[i] in (0, s.n_blocks - 1)]
+    rng = np.random.default_rng(5000 + s.index)
+    rows = sorted(set(edge) | set(int(i) for i in rng.choice(n_rows, min(n_random, n_rows), replace=False)))
+    out = torch.zeros(s.seq, s.heads, 128, dtype=torch.bfloat16)
+    call = lambda r: oracle.sparse_attention(q, k, v, wl.packed_info, wl.packed_kv_info, wl.info_indptr,
+                                             wl.kv_info_indptr, wl.qo_indptr, wl.kv_indptr, out=out, rows=r)
+    call(rows[:8])  # warm-up
+    t0 = time.perf_counter()
+    call(rows)
+    t_rows = time.perf_counter() - t0 - t_decode  # (every call decodes the symbols first)
+    blocks = int(sum(int(ptr[i + 1] - ptr[i]) for i in rows))
+    total_blocks = int(ptr[n_rows])
+    t_full = t_decode + t_rows * total_blocks / blocks
+    return {
+        "kind": "port", "cores": torch.get_num_threads(),
+        "sample": "%d of %d attention rows (%d edge rows: first / last q block; %d random, seeded), %d of %d "
+                  "computed kv blocks; symbol decode in full" % (len(rows), n_rows, len(edge), len(rows) - len(edge),
+                                                                blocks, total_blocks),
+        "measured_s": round(t_rows, 3), "decode_s": round(t_decode, 3),
+        "extrapolated_full_s": round(t_full, 2),
+        "extrapolated_tflops": round(wl.attention_flops() / t_full / 1e12, 4),
+        "extrapolation": "decode_s + measured_s * total kv blocks / sampled kv blocks",
+    }
+
+
+def cpu_baseline_gemms(wl, x, w, bias, n_sample=64):
+    """The oracle's GEMM-Q and GEMM-O (final pass) on a sample of a big config's token blocks (the first
+    n_sample / 2 and the last n_sample / 2, which includes the short last block); the whole config's time
+    is extrapolated by the computed (token block, head) tiles."""
+    import oracle
+    s = wl.shape
+    half = n_sample // 2
+    spans = [(0, half * 128), ((s.n_blocks - half) * 128, s.seq)]
+    info = wl.sparse_info.to(torch.float64)
+    lens = torch.full((s.n_blocks,), 128.0, dtype=torch.float64)
+    lens[-1] = s.seq - (s.n_blocks - 1) * 128
+    work = (info * lens[:, None]).sum(dim=1)  # active heads x tokens per token block
+    sample_work = float(work[:half].sum() + work[s.n_blocks - half:].sum())
+    t_q = t_o = 0.0
+    for r0, r1 in spans:
+        xs = x[:, r0:r1]
+        cache = torch.zeros(1, r1 - r0, s.hidden, dtype=torch.bfloat16)
+        t0 = time.perf_counter()
+        oracle.gemm_q(xs, w, s.heads, wl.packed_info, wl.info_indptr, r0, bias)
+        t1 = time.perf_counter()
+        oracle.gemm_o(xs, w, s.heads, wl.packed_info, wl.info_indptr, r0, bias=cache, is_for_cache=False)
+        t2 = time.perf_counter()
+        t_q += t1 - t0
+        t_o += t2 - t1
+    scale = float(work.sum()) / sample_work
+    return {
+        "sample": "%d of %d token blocks (first %d, last %d)" % (2 * half, s.n_blocks, half, half),
+        "gemm_q_measured_s": round(t_q, 3), "gemm_o_final_measured_s": round(t_o, 3),
+        "gemm_q_extrapolated_full_s": round(t_q * scale, 2), "gemm_o_final_extrapolated_full_s": round(t_o * scale, 2),
+        "gemm_q_extrapolated_tflops": round(wl.gemm_q_flops() / (t_q * scale) / 1e12, 4),
+        "gemm_o_final_extrapolated_tflops": round(wl.gemm_o_flops(False) / (t_o * scale) / 1e12, 4),
+        "extrapolation": "measured_s * active (token block, head) tiles of the config / of the sample",
     }
 
 
@@ -423,6 +529,8 @@ def main():
     c0["decode"]["rows"], c0["decode"]["kv_blocks"] = rows, nnz
     c0["sparse_fa_bf16"] = entry(fa_ms, flops=w0.attention_flops())
     c0["sparse_fa_bf16"]["computed_blocks"] = w0.computed_blocks
+    # the call a user of the reference makes: decode of the symbols + attention, every time
+    c0["run_dropin"] = entry(time_gpu(lambda: layer.attention(fresh_decode=True), KK, WW), flops=w0.attention_flops())
     kernels[w0.shape.name] = c0
     ms = time_gpu(layer.gemm_q, KK, WW)
     kernels[layer.w1.shape.name] = {"gemm_q": entry(ms, flops=layer.w1.gemm_q_flops())}
@@ -458,13 +566,19 @@ def main():
         log("[bench]", name, json.dumps(d))
 
     big_iters, big_warm = max(3, min(K, 10)), 2
+    cpu_big = {}
     for idx in (3, 4):
         if idx in configs:
             log("[bench] config %d attention (bf16)" % idx)
-            res = bench_big_attention(dev, idx, big_iters, big_warm)
+            res, cpu_fa = bench_big_attention(dev, idx, big_iters, big_warm, with_cpu=not args.no_cpu)
+            if cpu_fa is not None:
+                cpu_big["c%d" % idx] = {"sparse_fa": cpu_fa}
             if idx == 4:
                 log("[bench] config 4 GEMMs + quantiser")
-                res.update(bench_big_gemms(dev, idx, big_iters, big_warm))
+                res_g, cpu_g = bench_big_gemms(dev, idx, big_iters, big_warm, with_cpu=not args.no_cpu)
+                res.update(res_g)
+                if cpu_g is not None:
+                    cpu_big["c4"]["gemms"] = cpu_g
                 log("[bench] config 4 chain end to end")
                 res.update(bench_wan_chain(dev, big_iters, big_warm))
             kernels[SHAPES[idx].name] = res
@@ -474,6 +588,7 @@ def main():
     kernel_sum_ms = (kernels[layer.w1.shape.name]["gemm_q"]["ms"] + fa_ms
                      + kernels[layer.w2.shape.name]["gemm_o_final"]["ms"])
     fa_flops = w0.attention_flops()
+    traffic, traffic_state = traffic_from_profile()
     roofline = {
         "kernel": "sparse_fa_kernel<bf16> (config 0, FLUX shape)", "bound": "mfma",
         "achieved": round(fa_flops / (fa_ms * 1e-3) / 1e12, 2), "peak": PEAK_BF16, "unit": "TFLOP/s",
@@ -481,7 +596,7 @@ def main():
         # HBM bytes per launch: read from the committed summary of two rocprofv3 --pmc runs of this
         # command (FETCH_SIZE and WRITE_SIZE, each scaled by what a 256 MiB copy kernel reads on the same
         # counter); the algorithmic bytes of the launch are 98.6e6
-        "traffic": traffic_from_profile(), "traffic_unit": "bytes/launch",
+        "traffic": traffic, "traffic_state": traffic_state, "traffic_unit": "bytes/launch",
         "traffic_source": "profiles/" + os.path.basename(TRAFFIC_PROFILE),
         "launch_ms": round(fa_ms, 5), "algorithmic_flop_per_launch": fa_flops,
     }
@@ -489,6 +604,7 @@ def main():
     if not args.no_cpu:
         log("[bench] CPU baseline (oracle, %d threads)" % torch.get_num_threads())
         cpu = cpu_baseline(layer)
+        cpu.update(cpu_big)
 
     line = {
         "metric": "sparse-FA + GEMM-Q/O effective TFLOP/s on computed blocks, FLUX-shaped sparse layer "
