@@ -193,6 +193,11 @@ def bench_big_attention(dev, index, iters, warmup, with_cpu=False):
         res["quant_fp8"] = entry(ms_q, nbytes=3 * q.numel() + 4 * s.heads * s.n_blocks)
         ms_q = time_gpu(lambda: fo.quant_fp8_block(q, wl.qo_indptr, blocks=blocks, residual=True), iters, warmup)
         res["quant_fp8_two_term"] = entry(ms_q, nbytes=4 * q.numel() + 4 * s.heads * s.n_blocks)
+        # context, not a product path: a device-to-device copy of the same tensor (what a kernel that
+        # reads and writes streams reaches on this device)
+        qc = torch.empty_like(q)
+        res["device_copy_same_tensor"] = entry(time_gpu(lambda: qc.copy_(q), iters, warmup), nbytes=4 * q.numel())
+        del qc
         q8, qs, q_lo = fo.quant_fp8_block(q, wl.qo_indptr, blocks=blocks, residual=True)
         k8, ks, k_lo = fo.quant_fp8_block(k, wl.kv_indptr, blocks=blocks, residual=True)
         w8 = fo.BatchFlashOmniFAWithRaggedKVWrapper(ws)
