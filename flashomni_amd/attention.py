@@ -91,7 +91,7 @@ class PlannedBatch:
 
     def __init__(self, float_workspace_buffer, qo_indptr_host, kv_indptr_host, qo_indptr_dev,
                  kv_indptr_dev, num_qo_heads, num_kv_heads, block_q, block_kv, share_rows=True,
-                 worklist=None):
+                 worklist=None, gqa_packed=False):
         L = _lib.lib()
         self.device = float_workspace_buffer.device
         self.float_ws = float_workspace_buffer
@@ -100,15 +100,28 @@ class PlannedBatch:
         self.block_q, self.block_kv = block_q, block_kv
         batch_size = qo_indptr_host.numel() - 1
         self.batch_size = batch_size
+        # What a work-list row is.  Packed (the reference's layout for grouped-query attention,
+        # include/flashomni/attention/prefill.cuh:410-413, 1283-1290): a request's q rows are its
+        # (token, q head of the group) pairs, token-major; a row is (request, tile of 128 pairs, kv
+        # head) and the symbols hold one bit per (tile, kv head).  For the decoder that is a batch
+        # whose requests are `group` times as long, with num_kv_heads heads.
+        self.gqa_packed = bool(gqa_packed) and num_kv_heads != num_qo_heads
+        self.symbol_heads = num_kv_heads if self.gqa_packed else num_qo_heads
+        qo_rows_host = qo_indptr_host
+        if self.gqa_packed:
+            rows = qo_indptr_host.to(torch.int64) * (num_qo_heads // num_kv_heads)
+            if int(rows[-1]) >= 2 ** 31:
+                raise RuntimeError("Failed to plan prefill with error: too many packed q rows")
+            qo_rows_host = rows.to(torch.int32).contiguous()
         n_blk = torch.zeros(3, dtype=torch.int64)
-        _lib.check(L.fo_decode_sizes(_lib.ptr(qo_indptr_host), _lib.ptr(kv_indptr_host), batch_size,
-                                     num_qo_heads, block_q, block_kv,
+        _lib.check(L.fo_decode_sizes(_lib.ptr(qo_rows_host), _lib.ptr(kv_indptr_host), batch_size,
+                                     self.symbol_heads, block_q, block_kv,
                                      n_blk[0:].data_ptr(), n_blk[1:].data_ptr(), n_blk[2:].data_ptr()))
         n_q_blk, max_rows, max_nnz = (int(v) for v in n_blk)
         if max_nnz >= 2 ** 31:
             raise RuntimeError("Failed to plan prefill with error: work list too large")
         table = torch.empty((2, max(n_q_blk, 1)), dtype=torch.int32)
-        _lib.check(L.fo_sparse_block_table(_lib.ptr(qo_indptr_host), batch_size, block_q,
+        _lib.check(L.fo_sparse_block_table(_lib.ptr(qo_rows_host), batch_size, block_q,
                                            table[0].data_ptr(), table[1].data_ptr(), n_q_blk,
                                            n_blk[0:].data_ptr()))
         self.blk_table = table.to(self.device)
@@ -127,12 +140,13 @@ class PlannedBatch:
         # token counts, and the packed bytes of the byte-aligned per-request segments
         self.total_q_rows = int(qo_indptr_host[-1]) if qo_indptr_host.numel() else 0
         self.total_kv_rows = int(kv_indptr_host[-1]) if kv_indptr_host.numel() else 0
-        nqb = q_base[1:] - q_base[:-1]
+        qrows = (qo_rows_host[1:] - qo_rows_host[:-1]).to(torch.int64)
+        nqb = (qrows + block_q - 1) // block_q   # symbol rows (q blocks or packed tiles) per request
         nkb = kv_base[1:] - kv_base[:-1]
-        self.min_info_bytes = int(((nqb * num_qo_heads + 7) // 8).sum())
-        self.min_kv_info_bytes = int(((nqb * nkb * num_qo_heads + 7) // 8).sum())
+        self.min_info_bytes = int(((nqb * self.symbol_heads + 7) // 8).sum())
+        self.min_kv_info_bytes = int(((nqb * nkb * self.symbol_heads + 7) // 8).sum())
         if worklist is None or worklist.max_rows < max_rows or worklist.max_nnz < max_nnz:
-            worklist = DecodedWorkList(max_rows, max_nnz, num_qo_heads, self.device)
+            worklist = DecodedWorkList(max_rows, max_nnz, self.symbol_heads, self.device)
         self.worklist = worklist
         self.max_rows = max_rows
         self.share_rows = share_rows
@@ -181,7 +195,7 @@ class PlannedBatch:
             _lib.check(_lib.lib().fo_decode_sparse(
                 _lib.ptr(tensors[0]), _lib.ptr(tensors[1]), _lib.ptr(tensors[2]), _lib.ptr(tensors[3]),
                 _lib.ptr(self.blk_table[0]), _lib.ptr(self.blk_table[1]), _lib.ptr(self.kv_indptr),
-                self.n_q_blk, self.num_qo_heads, self.block_kv, int(bool(is_full)),
+                self.n_q_blk, self.symbol_heads, self.block_kv, int(bool(is_full)),
                 _lib.ptr(wl.row_req), _lib.ptr(wl.row_qb), _lib.ptr(wl.row_head), _lib.ptr(wl.kv_row_ptr),
                 _lib.ptr(wl.kv_idx), _lib.ptr(wl.counts), _lib.ptr(wl.order), _lib.ptr(wl.sched),
                 _lib.ptr(wl.scratch), _lib.ptr(wl.shares if self.split_ok else None),
@@ -211,6 +225,10 @@ class PlannedBatch:
         if q.dim() != 3 or k.dim() != 3 or v.dim() != 3 or k.size(2) != 128 or v.size(2) != 128:
             raise ValueError("q, k and v must be 3-dimensional with head_dim 128")
         fp8 = is_float8(q)
+        if fp8 and self.gqa_packed:
+            raise NotImplementedError(
+                "fp8 q has one scale per (q head, 128-token block); packed tiles of several q heads "
+                "(grouped-query attention in the reference's symbol layout) take 16-bit q and k")
         if fp8:
             if q.dtype != torch.float8_e4m3fn or k.dtype != torch.float8_e4m3fn \
                     or q_scale is None or k_scale is None:
@@ -267,7 +285,7 @@ class PlannedBatch:
                 _lib.ptr(self.kv_blk_base), self.n_q_blk, self.n_kv_blk, _lib.ptr(wl.row_req),
                 _lib.ptr(wl.row_qb), _lib.ptr(wl.row_head), _lib.ptr(wl.kv_row_ptr), _lib.ptr(wl.kv_idx),
                 _lib.ptr(wl.order), _lib.ptr(wl.sched), self.max_rows, q.size(1), self.num_kv_heads,
-                q.size(2), self.block_q, self.block_kv, float(sm_scale),
+                int(self.gqa_packed), q.size(2), self.block_q, self.block_kv, float(sm_scale),
                 _lib.ptr(wl.shares if self.split_ok else None),
                 _lib.ptr(self.float_ws) if self.split_ok else None,
                 self.float_ws_bytes(), _lib.current_stream(self.device)))
@@ -381,12 +399,14 @@ class BatchFlashOmniFAWithRaggedKVWrapper:
 
         Same parameters as the reference ``plan``, plus ``gqa_symbols`` (keyword-only).  With
         ``num_kv_heads < num_qo_heads`` the reference packs the q heads of a kv head into the row
-        dimension and reads one symbol per (128 packed rows = 128 / group tokens x group heads,
-        kv head) (include/flashomni/attention/prefill.cuh:1283-1290).  That tiling is not built
-        here; grouped-query attention is available with symbols per (128-token block, q head),
-        ``bit = q_block * num_qo_heads + q_head``, and has to be asked for by name,
-        ``gqa_symbols="per_q_head"``, so that symbols laid out for the reference are never
-        misread.  The host planner tiles the batch into the
+        dimension (row r of a request = token r // group, q head kv_head * group + r % group,
+        include/flashomni/attention/prefill.cuh:410-413) and reads one symbol per (tile of 128
+        packed rows, kv head): ``bit = tile * num_kv_heads + kv_head``, followed in
+        ``sparse_kv_info`` by one bit per kv block (prefill.cuh:1283-1290).  That is the layout
+        read by default (``gqa_symbols=None`` or ``"packed_tile"``); a request then has
+        ``ceil(qo_len * group / 128)`` symbol rows.  ``gqa_symbols="per_q_head"`` instead reads
+        symbols per (128-token block, q head), ``bit = q_block * num_qo_heads + q_head`` (no
+        counterpart in the reference).  The host planner tiles the batch into the
         integer workspace; in addition the q-block table of the symbol decoder is built and the
         work-list buffers are sized for the worst case (every bit set).  Cannot be captured in a
         graph (it copies the indptrs to the host)."""
@@ -414,13 +434,8 @@ class BatchFlashOmniFAWithRaggedKVWrapper:
                 "prefill path")
         if num_kv_heads <= 0 or num_qo_heads % num_kv_heads != 0:
             raise ValueError("num_qo_heads must be a multiple of num_kv_heads")
-        if gqa_symbols not in (None, "per_q_head"):
-            raise ValueError("gqa_symbols must be None or 'per_q_head'")
-        if num_kv_heads != num_qo_heads and gqa_symbols != "per_q_head":
-            raise NotImplementedError(
-                "grouped-query attention with the reference's symbol layout (one symbol per 128 packed "
-                "rows and kv head) is not built; pass gqa_symbols='per_q_head' to use symbols per "
-                "(128-token block, q head)")
+        if gqa_symbols not in (None, "packed_tile", "per_q_head"):
+            raise ValueError("gqa_symbols must be None, 'packed_tile' or 'per_q_head'")
         if head_dim_qk != 128 or head_dim_vo != 128:
             raise NotImplementedError("only head_dim 128 is supported")
         if sparse_block_size_for_q != 128 or sparse_block_size_for_kv != 128:
@@ -478,7 +493,8 @@ class BatchFlashOmniFAWithRaggedKVWrapper:
             self._float_workspace_buffer, qo_indptr_host, kv_indptr_host, self._qo_indptr_buf,
             self._kv_indptr_buf, num_qo_heads, num_kv_heads, sparse_block_size_for_q,
             sparse_block_size_for_kv, share_rows=self._share_rows,
-            worklist=self._planned.worklist if self._planned is not None else None)
+            worklist=self._planned.worklist if self._planned is not None else None,
+            gqa_packed=gqa_symbols != "per_q_head")
 
         self._num_qo_heads = num_qo_heads
         self._num_kv_heads = num_kv_heads

@@ -135,6 +135,12 @@ struct FaParams {
   const int32_t* shares;  // even shares: first row of every share, then the rows' cost offsets (or null)
   int32_t num_heads;
   int32_t kv_group;  // q heads per kv head (grouped-query attention); 1 = one kv head per q head
+  // 0: a work-list row is (request, 128-token q block, q head).  g > 0: the reference's layout for
+  // grouped-query attention with g q heads per kv head (prefill.cuh:410-413, 1283-1290): a row is
+  // (request, tile, kv head), the tile being rows tile*128 .. +127 of the request's q tokens x the kv
+  // head's g q heads flattened token-major (row r -> token r / g, q head kv_head * g + r % g);
+  // row_head holds the kv head and kv_group is 1.
+  int32_t gqa_pack;
   int32_t n_q_blocks, n_kv_blocks;  // row lengths of q_scale / k_scale
   float sm_scale_log2;
 };
@@ -277,7 +283,7 @@ __device__ __forceinline__ int pop_row(const FaParams& p, int xcd, const int* q,
 // workgroups share a CU (one wavefront of each per SIMD) and run independent rows: nothing ties
 // their phases together, there is no merge, and one's row prologue / epilogue overlaps the other's
 // main loop.  A row takes twice as long, so this is the form for long lists (many rows per CU).
-template <typename T, bool kFp8, bool kQLo, bool kKLo, int kGroups, bool kPipe = false>
+template <typename T, bool kFp8, bool kQLo, bool kKLo, int kGroups, bool kPipe = false, bool kGqaPack = false>
 __global__ void __launch_bounds__(kGroups * kGroupThreads) __attribute__((amdgpu_waves_per_eu(2, 2)))
 sparse_fa_kernel(const FaParams p) {
   static_assert(kPipe == (kGroups == 1), "one kv group runs the software-pipelined loop, two the two-phase loop");
@@ -309,6 +315,17 @@ sparse_fa_kernel(const FaParams p) {
     if constexpr (kFp8) {
       it.q_scale = p.q_scale[static_cast<int64_t>(it.head) * p.n_q_blocks + p.q_blk_base[it.req] + it.qb];
       it.k_scale0 = (it.head / p.kv_group) * p.n_kv_blocks + p.kv_blk_base[it.req];
+    }
+  };
+  // q_begin: first token of the item's q rows; q_rows: how many of its 128 rows exist
+  auto set_q_range = [&](RowInfo& it) {
+    const int q0 = p.qo_indptr[it.req], q1 = p.qo_indptr[it.req + 1];
+    if (kGqaPack) {  // (rows are (token, q head) pairs counted from the request's first token)
+      it.q_begin = q0;
+      it.q_rows = min(kBlockQ, (q1 - q0) * p.gqa_pack - it.qb * kBlockQ);
+    } else {
+      it.q_begin = q0 + it.qb * kBlockQ;
+      it.q_rows = min(kBlockQ, q1 - it.q_begin);
     }
   };
   __shared__ RowInfo s_next_row[2];
@@ -405,8 +422,7 @@ sparse_fa_kernel(const FaParams p) {
           it.req = p.row_req[w];
           it.qb = p.row_qb[w];
           it.head = p.row_head[w];
-          it.q_begin = p.qo_indptr[it.req] + it.qb * kBlockQ;
-          it.q_rows = min(kBlockQ, p.qo_indptr[it.req + 1] - it.q_begin);
+          set_q_range(it);
           it.kv_begin = p.kv_indptr[it.req];
           it.kv_len = p.kv_indptr[it.req + 1] - it.kv_begin;
           // this share's range of the row's kv blocks
@@ -463,8 +479,7 @@ sparse_fa_kernel(const FaParams p) {
           // (a row longer than the LDS list is cut; the host side refuses such requests at plan time)
           ri.nb = min(p.kv_row_ptr[w + 1] - ri.ptr0, kRowBlocks);
         }
-        ri.q_begin = p.qo_indptr[ri.req] + ri.qb * kBlockQ;
-        ri.q_rows = min(kBlockQ, p.qo_indptr[ri.req + 1] - ri.q_begin);
+        set_q_range(ri);
         ri.kv_begin = p.kv_indptr[ri.req];
         ri.kv_len = p.kv_indptr[ri.req + 1] - ri.kv_begin;
         fill_scales(ri);
@@ -513,16 +528,40 @@ sparse_fa_kernel(const FaParams p) {
 
     const int my_row = qs * 32 + l32;  // q row of this lane inside the block
     const bool row_ok = my_row < q_rows;
-    const int64_t q_tok = q_begin + (row_ok ? my_row : q_rows - 1);
+    // row r of the item -> its token (relative to q_begin) and q head (relative to head_q0)
+    // (a compile-time variant: as a run-time branch the mapping cost the ungrouped kernel 7 % at the
+    // FLUX shape, in how the compiler arranged the code around it)
+    const int gq = kGqaPack ? p.gqa_pack : 0;
+    const int head_q0 = gq ? head * gq : head;
+    auto row_at = [&](int r, int& tok, int& hq) __attribute__((always_inline)) {
+      if (gq) {
+        const uint32_t pr = static_cast<uint32_t>(qb) * kBlockQ + r;
+        tok = static_cast<int>(pr / static_cast<uint32_t>(gq));
+        hq = static_cast<int>(pr - tok * gq);
+      } else {
+        tok = r;
+        hq = 0;
+      }
+    };
+    // element offset of row r from the item's first q (o) vector, whose strides are sn, sh
+    auto row_off = [&](int r, int64_t sn, int64_t sh) __attribute__((always_inline)) {
+      int tok, hq;
+      row_at(r, tok, hq);
+      return tok * sn + hq * sh;
+    };
+    int my_tok, my_hq;
+    row_at(row_ok ? my_row : q_rows - 1, my_tok, my_hq);
+    const int64_t q_tok = q_begin + my_tok;
+    const int my_head = head_q0 + my_hq;
 
     if (nb == 0) {
       // listed row without kv blocks: zeros, lse = -5e4
       if (row_ok && kg == 0) {
-        T* dst = op + q_tok * p.o_sn + static_cast<int64_t>(head) * p.o_sh + g * 64;
+        T* dst = op + q_tok * p.o_sn + static_cast<int64_t>(my_head) * p.o_sh + g * 64;
         const u32x4 z = {0u, 0u, 0u, 0u};
 #pragma unroll
         for (int j = 0; j < 8; ++j) reinterpret_cast<u32x4*>(dst)[j] = z;
-        if (p.lse && g == 0) p.lse[q_tok * p.num_heads + head] = kNegInf;
+        if (p.lse && g == 0) p.lse[q_tok * p.num_heads + my_head] = kNegInf;
       }
       if (wv == kFetchWave) fetch_next((row_it + 1) & 1);
       continue;
@@ -596,12 +635,12 @@ sparse_fa_kernel(const FaParams p) {
       // prologue: Q, K(0..2), V(0) requested together
       {
         const uint8_t* q_head = reinterpret_cast<const uint8_t*>(
-            qp + static_cast<int64_t>(q_begin) * p.q_sn + static_cast<int64_t>(head) * p.q_sh);
+            qp + static_cast<int64_t>(q_begin) * p.q_sn + static_cast<int64_t>(head_q0) * p.q_sh);
 #pragma unroll
         for (int n = 0; n < 8; ++n) {
           int r = 4 * (4 * n + qs) + cp_row;
           r = r < q_rows ? r : q_rows - 1;  // ragged last q block: re-read the last row
-          copy16_to_lds(q_head, static_cast<uint32_t>((r * p.q_sn + cp_chunk) * sizeof(T)),
+          copy16_to_lds(q_head, static_cast<uint32_t>((row_off(r, p.q_sn, p.q_sh) + cp_chunk) * sizeof(T)),
                         lds0 + 4 * kBuf + qs * 1024 + n * 4096);
         }
       }
@@ -842,7 +881,7 @@ sparse_fa_kernel(const FaParams p) {
     if constexpr (kFp8) {
       // (fp8 Q, half the bytes, is still fetched directly: with the LDS detour hipcc arranges the
       // main loop of this instantiation less well, which costs more than the detour saves)
-      const uint8_t* src = qp + q_tok * p.q_sn + static_cast<int64_t>(head) * p.q_sh + g * 32;
+      const uint8_t* src = qp + q_tok * p.q_sn + static_cast<int64_t>(my_head) * p.q_sh + g * 32;
 #pragma unroll
       for (int sl = 0; sl < 2; ++sl) {
         const i32x4 lo = *reinterpret_cast<const i32x4*>(src + sl * 64);
@@ -851,7 +890,7 @@ sparse_fa_kernel(const FaParams p) {
       }
       if constexpr (kQLo) {
         const uint8_t* src2 = static_cast<const uint8_t*>(p.q_lo) + q_tok * p.q_sn +
-                              static_cast<int64_t>(head) * p.q_sh + g * 32;
+                              static_cast<int64_t>(my_head) * p.q_sh + g * 32;
 #pragma unroll
         for (int sl = 0; sl < 2; ++sl) {
           const i32x4 lo = *reinterpret_cast<const i32x4*>(src2 + sl * 64);
@@ -861,13 +900,14 @@ sparse_fa_kernel(const FaParams p) {
       }
     } else {
       const uint8_t* q_head = reinterpret_cast<const uint8_t*>(
-          qp + static_cast<int64_t>(q_begin) * p.q_sn + static_cast<int64_t>(head) * p.q_sh);
+          qp + static_cast<int64_t>(q_begin) * p.q_sn + static_cast<int64_t>(head_q0) * p.q_sh);
       const uint32_t qdst = lds_group + kStageBytes + kKBytes + qs * 1024;
 #pragma unroll
       for (int n = 0; n < 4; ++n) {
         int r = kg * 64 + 4 * (4 * n + qs) + cp_row;
         r = r < q_rows ? r : q_rows - 1;  // ragged last q block: re-read the last row
-        copy16_to_lds(q_head, static_cast<uint32_t>((r * p.q_sn + cp_chunk) * sizeof(T)), qdst + n * 4096);
+        copy16_to_lds(q_head, static_cast<uint32_t>((row_off(r, p.q_sn, p.q_sh) + cp_chunk) * sizeof(T)),
+                      qdst + n * 4096);
       }
     }
     // (the row's kv block list is in LDS already: the main loop has no global loads besides the
@@ -1339,7 +1379,7 @@ sparse_fa_kernel(const FaParams p) {
           for (int j = 0; j < 4; ++j) out[j] = static_cast<T>(o_acc[dt][i4 * 4 + j] * inv);
           *reinterpret_cast<x4*>(out_row + (dt * 32 + i4 * 8 + g * 4) * sizeof(T)) = out;
         }
-      if (row_ok && p.lse && g == 0) p.lse[q_tok * p.num_heads + head] = __builtin_amdgcn_logf(d_tot) + m_run;
+      if (row_ok && p.lse && g == 0) p.lse[q_tok * p.num_heads + my_head] = __builtin_amdgcn_logf(d_tot) + m_run;
     }
     if (kGroups == 2 && kg == 0) {
       const float m1 = md[(qs * 64 + lane) * 2 + 0], d1 = md[(qs * 64 + lane) * 2 + 1];
@@ -1368,7 +1408,7 @@ sparse_fa_kernel(const FaParams p) {
             *reinterpret_cast<x4*>(out_row + (dt * 32 + i4 * 8 + g * 4) * sizeof(T)) = out;
           }
         if (row_ok && p.lse && g == 0)
-          p.lse[q_tok * p.num_heads + head] = __builtin_amdgcn_logf(d_tot) + m;
+          p.lse[q_tok * p.num_heads + my_head] = __builtin_amdgcn_logf(d_tot) + m;
       } else {
         // one part of a row cut at share boundaries: fold kv group 1 in without normalising; the
         // accumulators then hold this workgroup's partial result (reference point m, sum d_tot)
@@ -1480,7 +1520,7 @@ sparse_fa_kernel(const FaParams p) {
               *reinterpret_cast<x4*>(out_row + (dt * 32 + i4 * 8 + g * 4) * sizeof(T)) = out;
             }
           if (row_ok && p.lse && g == 0)
-            p.lse[q_tok * p.num_heads + head] = __builtin_amdgcn_logf(d_all) + m_all;
+            p.lse[q_tok * p.num_heads + my_head] = __builtin_amdgcn_logf(d_all) + m_all;
         }
         if (tid == 0) p.sched[kSchedArrived + split_slot] = 0;  // re-armed for the next launch
         store_row = true;
@@ -1491,7 +1531,7 @@ sparse_fa_kernel(const FaParams p) {
     }
     if (store_row) {
       __syncthreads();  // the row is complete in the LDS tile
-      T* dst = op + static_cast<int64_t>(q_begin) * p.o_sn + static_cast<int64_t>(head) * p.o_sh;
+      T* dst = op + static_cast<int64_t>(q_begin) * p.o_sn + static_cast<int64_t>(head_q0) * p.o_sh;
       // (the lane index is made opaque here: otherwise the per-lane address terms are computed once
       // per kernel, spilled, and every reload waits for the store before it)
       int ln = lane;
@@ -1502,10 +1542,10 @@ sparse_fa_kernel(const FaParams p) {
 #pragma unroll
       for (int i = 0; i < kRowsPerWave / 4; ++i)
         v[i] = *reinterpret_cast<const u32x4*>(smem + G::kOutOff + (r0 + i * 4) * kOutRowBytes + chunk * 16);
-      T* d0 = dst + static_cast<int64_t>(r0) * p.o_sn + chunk * 8;
+      T* d0 = dst + chunk * 8;
 #pragma unroll
       for (int i = 0; i < kRowsPerWave / 4; ++i)
-        if (r0 + i * 4 < q_rows) *reinterpret_cast<u32x4*>(d0 + i * 4 * p.o_sn) = v[i];
+        if (r0 + i * 4 < q_rows) *reinterpret_cast<u32x4*>(d0 + row_off(r0 + i * 4, p.o_sn, p.o_sh)) = v[i];
     }
   }
 
@@ -1520,7 +1560,7 @@ sparse_fa_kernel(const FaParams p) {
   }
 }
 
-template <typename T, bool kFp8, bool kQLo, bool kKLo, int kGroups = 2, bool kPipe = false>
+template <typename T, bool kFp8, bool kQLo, bool kKLo, int kGroups = 2, bool kPipe = false, bool kGqaPack = false>
 int launch(const FaParams& p, int64_t max_rows, hipStream_t stream) {
   constexpr int kSmemBytes = Geom<kFp8, kKLo, kGroups>::kSmemBytes;
   // (the attribute belongs to the kernel's code object on one device: set once per device; the flags
@@ -1529,7 +1569,7 @@ int launch(const FaParams& p, int64_t max_rows, hipStream_t stream) {
   int dev = 0;
   FO_HIP_CALL(hipGetDevice(&dev));
   if (dev < 0 || dev >= 64 || !attr_set[dev].load(std::memory_order_acquire)) {
-    FO_HIP_CALL(hipFuncSetAttribute(reinterpret_cast<const void*>(&sparse_fa_kernel<T, kFp8, kQLo, kKLo, kGroups, kPipe>),
+    FO_HIP_CALL(hipFuncSetAttribute(reinterpret_cast<const void*>(&sparse_fa_kernel<T, kFp8, kQLo, kKLo, kGroups, kPipe, kGqaPack>),
                                     hipFuncAttributeMaxDynamicSharedMemorySize, kSmemBytes));
     if (dev >= 0 && dev < 64) attr_set[dev].store(true, std::memory_order_release);
   }
@@ -1538,7 +1578,7 @@ int launch(const FaParams& p, int64_t max_rows, hipStream_t stream) {
   int64_t grid = num_cu * (3 - kGroups);  // persistent workgroups: one per CU, or two of one kv group each (LDS bound)
   // (with even shares every workgroup may hold a part of a row; otherwise at most one row each)
   if (!(p.split_ws && p.shares) && grid > max_rows) grid = max_rows;
-  sparse_fa_kernel<T, kFp8, kQLo, kKLo, kGroups, kPipe><<<static_cast<unsigned>(grid), kGroups * kGroupThreads, kSmemBytes, stream>>>(p);
+  sparse_fa_kernel<T, kFp8, kQLo, kKLo, kGroups, kPipe, kGqaPack><<<static_cast<unsigned>(grid), kGroups * kGroupThreads, kSmemBytes, stream>>>(p);
   FO_CHECK_LAUNCH();
   return FO_OK;
 }
@@ -1572,8 +1612,8 @@ extern "C" int fo_sparse_fa_run(const void* q, const void* k, const void* v, voi
                                 const int32_t* row_qb, const int32_t* row_head,
                                 const int32_t* kv_row_ptr, const int32_t* kv_idx,
                                 const int32_t* order, int32_t* sched, int64_t max_rows,
-                                int32_t num_heads, int32_t num_kv_heads, int32_t head_dim, int32_t block_q,
-                                int32_t block_kv, float sm_scale, const int32_t* shares,
+                                int32_t num_heads, int32_t num_kv_heads, int32_t gqa_packed, int32_t head_dim,
+                                int32_t block_q, int32_t block_kv, float sm_scale, const int32_t* shares,
                                 void* split_workspace, int64_t split_workspace_bytes, void* stream) {
   FO_REQUIRE(head_dim == kHeadDim, "sparse_fa: head_dim %d is not supported (only 128)", head_dim);
   FO_REQUIRE(block_q == kBlockQ && block_kv == kBlockKV,
@@ -1584,6 +1624,10 @@ extern "C" int fo_sparse_fa_run(const void* q, const void* k, const void* v, voi
   FO_REQUIRE(num_heads > 0 && max_rows >= 0, "sparse_fa: bad sizes");
   FO_REQUIRE(num_kv_heads > 0 && num_heads % num_kv_heads == 0,
              "sparse_fa: num_qo_heads %d is not a multiple of num_kv_heads %d", num_heads, num_kv_heads);
+  FO_REQUIRE(gqa_packed == 0 || gqa_packed == 1, "sparse_fa: gqa_packed must be 0 or 1");
+  FO_REQUIRE(!gqa_packed || dtype != FO_FP8_E4M3,
+             "sparse_fa: fp8 q (one scale per q head and token block) is not built for packed tiles of "
+             "several q heads");
   if (max_rows == 0) return FO_OK;
   FO_REQUIRE(q && k && v && o && qo_indptr && kv_indptr && row_req && row_qb && row_head &&
                  kv_row_ptr && kv_idx && order && sched,
@@ -1627,7 +1671,11 @@ extern "C" int fo_sparse_fa_run(const void* q, const void* k, const void* v, voi
     p.split_ws = static_cast<float*>(split_workspace);
     p.shares = shares;
   }
-  p.num_heads = num_heads; p.kv_group = num_heads / num_kv_heads; p.n_q_blocks = n_q_blocks; p.n_kv_blocks = n_kv_blocks;
+  p.num_heads = num_heads;
+  // packed tiles: row_head is the kv head already, and a tile's rows spread over its q heads
+  const bool packed = gqa_packed && num_heads != num_kv_heads;
+  p.kv_group = packed ? 1 : num_heads / num_kv_heads;
+  p.gqa_pack = packed ? num_heads / num_kv_heads : 0; p.n_q_blocks = n_q_blocks; p.n_kv_blocks = n_kv_blocks;
   p.sm_scale_log2 = sm_scale * 1.44269504088896340736f;
   hipStream_t s = static_cast<hipStream_t>(stream);
   // Long lists (many rows per CU) run as two independent 4-wavefront workgroups per CU with the
@@ -1642,6 +1690,13 @@ extern "C" int fo_sparse_fa_run(const void* q, const void* k, const void* v, voi
                             span * v_stride_n < (int64_t(1) << 32);
   const int variant = g_variant.load(std::memory_order_relaxed);
   const bool one_group = one_group_ok && (variant == 1 || (variant == 0 && max_rows >= static_cast<int64_t>(8) * fo_num_cu()));
+  if (p.gqa_pack) {  // packed tiles of several q heads: the row mapping is compiled in
+    if (dtype == FO_BF16)
+      return one_group ? launch<__bf16, false, false, false, 1, true, true>(p, max_rows, s)
+                       : launch<__bf16, false, false, false, 2, false, true>(p, max_rows, s);
+    return one_group ? launch<_Float16, false, false, false, 1, true, true>(p, max_rows, s)
+                     : launch<_Float16, false, false, false, 2, false, true>(p, max_rows, s);
+  }
   if (dtype == FO_BF16)
     return one_group ? launch<__bf16, false, false, false, 1, true>(p, max_rows, s)
                      : launch<__bf16, false, false, false, 2>(p, max_rows, s);

@@ -48,9 +48,8 @@ def batch_sparseFA_with_kv_plan(float_workspace_buffer, int_workspace_buffer,
     _check(qo_host.numel() == batch_size + 1 and kv_host.numel() == batch_size + 1,
            "batch_sparseFA_with_kv_plan: indptr arrays must have batch_size + 1 entries")
     _check(head_dim_qk == 128 and head_dim_vo == 128, "only head_dim 128 is supported")
-    _check(num_qo_heads == num_kv_heads,
-           "grouped-query attention with the reference's symbol layout (one symbol per 128 packed rows and kv "
-           "head, prefill.cuh:1283-1290) is not built; the wrapper offers plan(..., gqa_symbols='per_q_head')")
+    _check(num_kv_heads > 0 and num_qo_heads % num_kv_heads == 0,
+           "num_qo_heads must be a multiple of num_kv_heads")
     plan_info = torch.empty(15, dtype=torch.int64)
     nbytes = lambda t: t.numel() * t.element_size()
     with _lib.device_guard(dev):
@@ -67,7 +66,10 @@ def batch_sparseFA_with_kv_plan(float_workspace_buffer, int_workspace_buffer,
     old = _plans.pop(key, None)
     _plans[key] = PlannedBatch(float_workspace_buffer, qo_host, kv_host, qo_host.to(dev), kv_host.to(dev),
                                num_qo_heads, num_kv_heads, 128, 128,
-                               worklist=old.worklist if old is not None else None)
+                               worklist=old.worklist if old is not None else None,
+                               # grouped-query attention: the reference's symbols, one bit per (tile of
+                               # 128 packed rows, kv head) (prefill.cuh:1283-1290)
+                               gqa_packed=True)
     while len(_plans) > _MAX_PLANS:
         _plans.popitem(last=False)
     return plan_info

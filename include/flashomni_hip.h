@@ -19,7 +19,7 @@
 extern "C" {
 #endif
 
-#define FO_ABI_VERSION 3
+#define FO_ABI_VERSION 4
 
 enum {
   FO_OK = 0,
@@ -158,7 +158,16 @@ int fo_decode_sparse_static(const uint8_t* sparse_info, const uint8_t* sparse_kv
  *
  * q [nnz_q,H,D], k,v [nnz_kv,H_kv,D], o [nnz_q,H,D]; strides in elements (the innermost stride is
  * 1).  num_heads = H must be a multiple of num_kv_heads = H_kv: q head h reads kv head
- * h / (H / H_kv) (grouped-query attention, prefill.cuh:410-413); k_scale then has H_kv rows.  dtype FO_BF16 / FO_F16: q,k,v,o share it.  dtype FO_FP8_E4M3: q and k are e4m3fn bytes
+ * h / (H / H_kv) (grouped-query attention, prefill.cuh:410-413); k_scale then has H_kv rows.
+ * gqa_packed selects what a work-list row is when H_kv < H (it has no effect when H_kv = H):
+ *   1: the reference's layout (prefill.cuh:1283-1290 with :410-413): a request's q rows are its
+ *      (token, q head of the group) pairs, token-major, per kv head; row (request, tile t, kv head j)
+ *      covers pairs t*128 .. t*128+127, i.e. pair r is token r / g, q head j*g + r % g (g = H / H_kv),
+ *      and the symbols hold one bit per (tile, kv head) (x one per kv block): the list is decoded
+ *      with num_heads = H_kv over ceil(qo_len * g / 128) tiles per request, row_qb is the tile and
+ *      row_head the kv head.  16-bit q, k, v only.
+ *   0: a row is (request, 128-token block, q head), symbols per q head (no reference counterpart).
+ * dtype FO_BF16 / FO_F16: q,k,v,o share it.  dtype FO_FP8_E4M3: q and k are e4m3fn bytes
  * with dequantisation scales q_scale[H][n_q_blocks], k_scale[H][n_kv_blocks] (fp32, blocks
  * numbered request by request: q_blk_base / kv_blk_base [batch+1] give each request's first
  * block); v and o are bf16.  q_lo (optional, else NULL): a second e4m3fn tensor laid out like q, the
@@ -204,8 +213,8 @@ int fo_sparse_fa_run(const void* q, const void* k, const void* v, void* o, float
                      const int32_t* q_blk_base, const int32_t* kv_blk_base, int32_t n_q_blocks,
                      int32_t n_kv_blocks, const int32_t* row_req, const int32_t* row_qb, const int32_t* row_head,
                      const int32_t* kv_row_ptr, const int32_t* kv_idx, const int32_t* order,
-                     int32_t* sched, int64_t max_rows, int32_t num_heads, int32_t num_kv_heads, int32_t head_dim,
-                     int32_t block_q, int32_t block_kv, float sm_scale, const int32_t* shares,
+                     int32_t* sched, int64_t max_rows, int32_t num_heads, int32_t num_kv_heads, int32_t gqa_packed,
+                     int32_t head_dim, int32_t block_q, int32_t block_kv, float sm_scale, const int32_t* shares,
                      void* split_workspace, int64_t split_workspace_bytes, void* stream);
 
 /* ---------------------------------------------------------------------------------------------

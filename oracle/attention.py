@@ -10,6 +10,14 @@ Semantics follow include/flashomni/attention/prefill.cuh:
     (:973, :1517; include/flashomni/attention/variants.cuh:54).
 The block mask is expanded to token granularity exactly like the reference benchmark builds
 its SDPA mask (benchmark/test_flashomni_attention.py:197-199): repeat_interleave(block) and crop.
+
+Grouped-query attention (fewer kv heads than q heads, group = H / H_kv), gqa_symbols="packed_tile":
+the reference's layout.  A request's q rows are its (token, q head of the group) pairs, token-major
+per kv head: packed row p = token p // group, q head kv_head * group + p % group (:410-413 load,
+:1128, :1178 store, :1510-1511 lse).  A launch block is (tile of 128 packed rows, kv head)
+(:1273-1278); its sparse_info bit is tile * H_kv + kv_head and its kv mask starts at that bit index
+times the request's number of kv blocks (:1283-1290).  gqa_symbols="per_q_head" (no reference
+counterpart): symbols per (128-token block, q head), q head h reads kv head h // group.
 """
 import math
 
@@ -24,7 +32,7 @@ NEG_INF = -5e4
 def sparse_attention(q, k, v, sparse_info, sparse_kv_info, sparse_info_indptr,
                      sparse_kv_info_indptr, qo_indptr, kv_indptr, block_q=128, block_kv=128,
                      sm_scale=None, is_full=False, out=None, lse=None, rows=None,
-                     q_scale=None, k_scale=None, q_lo=None, k_lo=None):
+                     q_scale=None, k_scale=None, q_lo=None, k_lo=None, gqa_symbols="per_q_head"):
     """q [nnz_q,H,D], k/v [nnz_kv,H,D] (any float dtype; math is fp32 on the given values).
 
     `out` (same dtype as q unless q is fp8, then bf16) is updated in place for active rows only; allocated
@@ -42,6 +50,12 @@ def sparse_attention(q, k, v, sparse_info, sparse_kv_info, sparse_info_indptr,
     to_np = lambda t: None if t is None else (t.cpu().numpy() if torch.is_tensor(t) else np.asarray(t))
     qo = to_np(qo_indptr).astype(np.int64)
     kvp = to_np(kv_indptr).astype(np.int64)
+    packed = group > 1 and gqa_symbols == "packed_tile"
+    if packed:
+        assert q_scale is None and k_scale is None, "packed tiles take 16-bit q and k"
+        return _packed_tiles(q, k, v, to_np(sparse_info), to_np(sparse_kv_info), to_np(sparse_info_indptr),
+                             to_np(sparse_kv_info_indptr), qo, kvp, group, block_q, block_kv,
+                             sm_scale, is_full, out, lse, rows)
     row_req, row_qb, row_head, ptr, idx = decode_kv_csr(
         to_np(sparse_info), to_np(sparse_kv_info), to_np(sparse_info_indptr),
         to_np(sparse_kv_info_indptr), qo, kvp, H, block_q, block_kv, is_full)
@@ -83,4 +97,44 @@ def sparse_attention(q, k, v, sparse_info, sparse_kv_info, sparse_info_indptr,
         out[q0:q1, h] = ((p @ vf) / d).to(out.dtype)
         if lse is not None:
             lse[q0:q1, h] = (torch.log2(d) + m * c).squeeze(-1)
+    return out
+
+
+def _packed_tiles(q, k, v, sparse_info, sparse_kv_info, sparse_info_indptr, sparse_kv_info_indptr, qo, kvp,
+                  group, block_q, block_kv, sm_scale, is_full, out, lse, rows):
+    """The reference's grouped-query layout (see the module text).  The symbols of a request with
+    qo_len tokens are those of an ungrouped request with qo_len * group rows and H_kv heads
+    (prefill.cuh:1283-1290 with gridDim.z = H_kv), so the same decoder lists the (tile, kv head) rows."""
+    H_kv = k.shape[1]
+    c = sm_scale * math.log2(math.e)
+    qo_packed = qo * group
+    row_req, row_tile, row_kvh, ptr, idx = decode_kv_csr(
+        sparse_info, sparse_kv_info, sparse_info_indptr, sparse_kv_info_indptr, qo_packed, kvp, H_kv,
+        block_q, block_kv, is_full)
+    sel = range(len(row_req)) if rows is None else rows
+    for i in sel:
+        r, tile, kvh = int(row_req[i]), int(row_tile[i]), int(row_kvh[i])
+        qlen = int(qo[r + 1] - qo[r])
+        pr = np.arange(tile * block_q, min((tile + 1) * block_q, qlen * group))   # packed rows of the tile
+        tok = torch.from_numpy(int(qo[r]) + pr // group)                            # :410 divmod -> q
+        hq = torch.from_numpy(kvh * group + pr % group)                             # :410 divmod -> r, :1323
+        kv0, kv1 = int(kvp[r]), int(kvp[r + 1])
+        kept = idx[ptr[i]:ptr[i + 1]]
+        if len(kept) == 0:
+            out[tok, hq] = 0
+            if lse is not None:
+                lse[tok, hq] = NEG_INF
+            continue
+        kt = torch.from_numpy(np.concatenate([np.arange(kv0 + b * block_kv, min(kv1, kv0 + (b + 1) * block_kv))
+                                              for b in kept]))
+        qf = q[tok, hq].float()
+        kf = k[kt, kvh].float()
+        vf = v[kt, kvh].float()
+        s = qf @ kf.T
+        m = s.max(dim=-1, keepdim=True).values
+        p = torch.exp2((s - m) * c)
+        d = p.sum(dim=-1, keepdim=True)
+        out[tok, hq] = ((p @ vf) / d).to(out.dtype)
+        if lse is not None:
+            lse[tok, hq] = (torch.log2(d) + m * c).squeeze(-1)
     return out

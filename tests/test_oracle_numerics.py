@@ -9,7 +9,7 @@ import torch
 import torch.nn.functional as F
 
 import oracle
-from helpers import make_ragged_masks
+from helpers import make_ragged_masks, sentinel_like
 
 
 def _qkv(nq, nk, heads, seed):
@@ -183,3 +183,49 @@ def test_fp8_attention_oracle_applies_scales():
     ref = oracle.sparse_attention(q, k, v, m["packed_info"], m["packed_keep"], m["info_indptr"], m["keep_indptr"],
                                   m["qo_indptr"], m["kv_indptr"])
     assert 1e-2 < float((a.float() - ref.float()).norm() / ref.float().norm()) < 6e-2
+
+
+@pytest.mark.parametrize("heads", [(4, 2), (6, 1), (14, 2)])
+def test_attention_packed_tile_gqa_token_by_token(heads):
+    """Grouped-query attention in the reference's symbol layout (prefill.cuh:410-413, 1283-1290),
+    pinned by a second formulation that never forms a tile: for every (token, q head) on its own, the
+    packed row is token * group + head % group, its tile row // 128, its kv head head // group; the
+    symbol bit is tile * H_kv + kv_head and the kv bits follow at that index times the number of kv
+    blocks; the output is the float64 softmax over the kept keys (masked SDPA).  A wrong divmod order,
+    head base or bit index in the oracle moves rows between symbols and fails here."""
+    hq, hkv = heads
+    group = hq // hkv
+    ql, kl = [150, 1, 260], [77, 300, 129]
+    m = make_ragged_masks([n * group for n in ql], kl, hkv, 0.6, 0.5, seed=47)
+    qo = np.concatenate([[0], np.cumsum(ql)]).astype(np.int32)
+    kv = m["kv_indptr"]
+    g = torch.Generator().manual_seed(47)
+    q = torch.randn(sum(ql), hq, 128, generator=g)
+    k = torch.randn(sum(kl), hkv, 128, generator=g)
+    v = torch.randn(sum(kl), hkv, 128, generator=g)
+    out0 = sentinel_like((sum(ql), hq, 128), torch.float32)
+    lse = torch.full((sum(ql), hq), float("nan"))
+    out = oracle.sparse_attention(q, k, v, m["packed_info"], m["packed_keep"], m["info_indptr"], m["keep_indptr"],
+                                  qo, kv, out=out0.clone(), lse=lse, gqa_symbols="packed_tile")
+    bit = lambda buf, base, i: (int(buf[base + i // 8]) >> (i % 8)) & 1
+    c = math.log2(math.e) / math.sqrt(128)
+    for r in range(len(ql)):
+        nkv = -(-kl[r] // 128)
+        for tok in range(ql[r]):
+            for h in range(hq):
+                row = tok * group + h % group
+                sym = (row // 128) * hkv + h // group
+                got = out[qo[r] + tok, h]
+                if not bit(m["packed_info"], int(m["info_indptr"][r]), sym):
+                    assert torch.equal(got, out0[qo[r] + tok, h]) and math.isnan(float(lse[qo[r] + tok, h]))
+                    continue
+                keys = [j for b in range(nkv) if bit(m["packed_keep"], int(m["keep_indptr"][r]), sym * nkv + b)
+                        for j in range(kv[r] + b * 128, min(kv[r + 1], kv[r] + (b + 1) * 128))]
+                if not keys:
+                    assert float(got.abs().max()) == 0.0 and float(lse[qo[r] + tok, h]) == -5e4
+                    continue
+                s = (k[keys, h // group].double() @ q[qo[r] + tok, h].double()) * c
+                p = torch.exp2(s - s.max())
+                want = (p[:, None] * v[keys, h // group].double()).sum(0) / p.sum()
+                assert float((got.double() - want).abs().max()) < 1e-4
+                assert abs(float(lse[qo[r] + tok, h]) - float(torch.log2(p.sum()) + s.max())) < 1e-3
