@@ -327,8 +327,10 @@ def test_video_gemms_sampled_token_blocks(dev):
     """The 14B-video shape at full size (M=76112 with an 80-row last block, K=N=5120, 40 heads):
     GEMM-Q, the GEMM-O cache pass and the final pass run over the whole matrix; the first, the last
     and 10 seeded random token blocks are checked against the oracle, which is run on each block's
-    rows alone with the text-token offset that makes it read that block's flags.  The oracle keeps
-    fp32 outputs, so the bound covers the kernel's one bf16 rounding (outputs stay below 4)."""
+    rows alone with the text-token offset that makes it read that block's flags.  Weights ~ N(0, 0.02)
+    as the configuration states: outputs have standard deviation 1.4 and a few of the 4 * 10^8 exceed
+    8, where half a bf16 unit (2^-5) is above the 2e-2 bound: no bf16 result can be closer to the
+    oracle's fp32 value than that, so from |y| = 8 on the bound is half a unit of y plus 2e-3."""
     import flashomni_amd as fo
     from flashomni_amd.workloads import make_workload
     wl = make_workload(4, tensors=False)
@@ -336,7 +338,13 @@ def test_video_gemms_sampled_token_blocks(dev):
     M, C, H = s.seq, s.hidden, s.heads
     g = torch.Generator(device=dev).manual_seed(41)
     rand = lambda *sz, std=1.0: (torch.randn(*sz, generator=g, device=dev) * std).to(torch.bfloat16)
-    x, w_q, b_q, w_o, b_o = rand(1, M, C), rand(C, C, std=0.01), rand(C, std=0.02), rand(C, C, std=0.01), rand(C, std=0.02)
+    x, w_q, b_q, w_o, b_o = rand(1, M, C), rand(C, C, std=0.02), rand(C, std=0.02), rand(C, C, std=0.02), rand(C, std=0.02)
+
+    def within_bound(got, exp):
+        half_unit = torch.exp2(torch.floor(torch.log2(exp.abs().clamp_min(1.0))) - 8)
+        bound = torch.where(exp.abs() < 8, torch.full_like(exp, MAX_ABS), half_unit + 2e-3)
+        return bool(((got.float() - exp).abs() <= bound).all())
+
     pk, ip = wl.packed_info.to(dev), wl.info_indptr.to(dev)
     y = torch.full((1, M, C), -7.0, dtype=torch.bfloat16, device=dev)
     fo.flashomni_gemm(x, w_q, H, pk, ip, 0, b_q, out=y)
@@ -357,7 +365,7 @@ def test_video_gemms_sampled_token_blocks(dev):
         exp = oracle.gemm_q(xs, wq_c, H, wl.packed_info, wl.info_indptr, r0, bq_c,
                             out=torch.full((1, r1 - r0, C), -7.0, dtype=torch.float32))
         got = y[:, r0:r1].cpu()
-        assert max_abs(got, exp) <= MAX_ABS, iy
+        assert within_bound(got, exp), iy
         assert rel_l2(got, exp) <= REL_L2, iy
         exp_cache = oracle.gemm_o(xs, wo_c, H, wl.packed_info, wl.info_indptr, r0, bias=bo_c,
                                   is_for_cache=True, out_dtype=torch.float32)
@@ -366,7 +374,7 @@ def test_video_gemms_sampled_token_blocks(dev):
         exp_final = oracle.gemm_o(xs, wo_c, H, wl.packed_info, wl.info_indptr, r0, bias=exp_cache,
                                   is_for_cache=False, out_dtype=torch.float32)
         got_final = final[:, r0:r1].cpu()
-        assert max_abs(got_final, exp_final) <= MAX_ABS, iy
+        assert within_bound(got_final, exp_final), iy
         assert rel_l2(got_final, exp_final) <= REL_L2, iy
 
 

@@ -18,7 +18,7 @@ def _ops():
     return torch.ops.flashomni_kernels
 
 
-def _plan(dev, m, heads, float_ws=None):
+def _plan(dev, m, heads, float_ws=None, kv_heads=None):
     """What the reference's wrapper does in __init__ and plan() (flashomni/attention.py:344-352,
     :535-606): workspaces, host indptrs, the plan operator."""
     k = _ops()
@@ -29,7 +29,8 @@ def _plan(dev, m, heads, float_ws=None):
     kv_len = kv_h[1:] - kv_h[:-1]
     batch = qo_h.numel() - 1
     plan_info = k.batch_sparseFA_with_kv_plan.default(
-        float_ws, int_ws, pin_ws, qo_h, kv_h, kv_len, int(qo_h[-1]), batch, heads, heads, 1, False, 128, 128)
+        float_ws, int_ws, pin_ws, qo_h, kv_h, kv_len, int(qo_h[-1]), batch, heads, kv_heads or heads, 1, False, 128,
+        128)
     return float_ws, int_ws, plan_info, qo_h.to(dev), kv_h.to(dev)
 
 
@@ -70,6 +71,30 @@ def test_attention_ops_ragged_batch(dev, dtype):
     ok = ~torch.isnan(exp_lse)
     assert torch.equal(torch.isnan(lse.cpu()), ~ok)
     assert float((lse.cpu()[ok] - exp_lse[ok]).abs().max()) < 2e-2
+
+
+def test_attention_ops_grouped_query(dev):
+    """num_kv_heads < num_qo_heads through the operators: the symbols are the reference's, one bit per
+    (tile of 128 packed (token, q head) rows, kv head) (prefill.cuh:410-413, 1283-1290)."""
+    hq, hkv = 8, 2
+    ql, kl = [200, 129], [300, 64]
+    m = make_ragged_masks([n * (hq // hkv) for n in ql], kl, hkv, 0.7, 0.5, seed=24)
+    m["qo_indptr"] = np.concatenate([[0], np.cumsum(ql)]).astype(np.int32)
+    g = torch.Generator().manual_seed(24)
+    nq, nk = sum(ql), sum(kl)
+    q = torch.randn(nq, hq, 128, generator=g).to(torch.bfloat16)
+    k, v = (torch.randn(nk, hkv, 128, generator=g).to(torch.bfloat16) for _ in range(2))
+    state = _plan(dev, m, hq, kv_heads=hkv)
+    out0 = sentinel_like((nq, hq, 128), torch.bfloat16)
+    o = out0.clone().to(dev)
+    _run(dev, state, q.to(dev), k.to(dev), v.to(dev), m, o)
+    exp = oracle.sparse_attention(q, k, v, m["packed_info"], m["packed_keep"], m["info_indptr"], m["keep_indptr"],
+                                  m["qo_indptr"], m["kv_indptr"], out=out0.clone(), gqa_symbols="packed_tile")
+    o = o.cpu()
+    touched = (exp.view(torch.int16) != out0.view(torch.int16)).any(-1)
+    assert touched.any() and not touched.all()
+    assert torch.equal(o[~touched].view(torch.int16), out0[~touched].view(torch.int16))
+    assert max_abs(o[touched], exp[touched]) <= 2e-2 and rel_l2(o[touched], exp[touched]) <= 1e-2
 
 
 def test_attention_ops_hnd_and_is_full(dev):
