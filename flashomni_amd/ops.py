@@ -14,6 +14,7 @@ as the reference's run finds its tile arrays inside that workspace.  plan() allo
 part of a captured graph in the reference either, flashomni/attention.py:140-141); run() does not.
 """
 import collections
+import weakref
 
 import torch
 
@@ -64,12 +65,17 @@ def batch_sparseFA_with_kv_plan(float_workspace_buffer, int_workspace_buffer,
             raise RuntimeError("Failed to plan prefill with error: " + str(e)) from None
     key = (dev.index, int_workspace_buffer.data_ptr())
     old = _plans.pop(key, None)
+    if old is None:
+        # the plan goes when the workspace's memory does: another tensor at the same address later must
+        # not find it
+        weakref.finalize(int_workspace_buffer.untyped_storage(), _plans.pop, key, None)
     _plans[key] = PlannedBatch(float_workspace_buffer, qo_host, kv_host, qo_host.to(dev), kv_host.to(dev),
                                num_qo_heads, num_kv_heads, 128, 128,
                                worklist=old.worklist if old is not None else None,
                                # grouped-query attention: the reference's symbols, one bit per (tile of
                                # 128 packed rows, kv head) (prefill.cuh:1283-1290)
                                gqa_packed=True)
+    _plans[key].plan_vec = plan_info.tolist()
     while len(_plans) > _MAX_PLANS:
         _plans.popitem(last=False)
     return plan_info
@@ -88,6 +94,13 @@ def batch_sparseFA_with_ragged_kv_run(float_workspace_buffer, int_workspace_buff
     pb = _plans.get((dev.index, int_workspace_buffer.data_ptr()))
     _check(pb is not None, "batch_sparseFA_with_ragged_kv_run: no plan was made with this int workspace "
                            "(call batch_sparseFA_with_kv_plan first)")
+    # (the vector is what the caller got from that plan call: a workspace planned again since, by
+    # another owner, holds another batch's tables)
+    _check(list(plan_info_vec.tolist() if torch.is_tensor(plan_info_vec) else plan_info_vec) == pb.plan_vec,
+           "batch_sparseFA_with_ragged_kv_run: plan_info_vec is not the plan last made with this int "
+           "workspace")
+    _check(q.dim() == 3 and q.size(1) == pb.num_qo_heads,
+           "batch_sparseFA_with_ragged_kv_run: q does not have the planned number of heads")
     _check(mask_mode_code == 0 and maybe_custom_mask is None and maybe_mask_indptr is None,
            "only the non-causal mask mode is built (as in the reference's shipped kernels)")
     _check(maybe_alibi_slopes is None and logits_soft_cap <= 0.0,

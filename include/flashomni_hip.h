@@ -137,7 +137,9 @@ int fo_decode_sparse(const uint8_t* sparse_info, const uint8_t* sparse_kv_info,
  * array built into the library's device code instead (one copy per GPU, held until the process ends),
  * so n_blk * num_heads may be at most fo_decode_sparse_static_max_pairs() (126 976); larger
  * inputs are refused with FO_ERR_INVALID.  Same inputs, outputs and results as fo_decode_sparse.
- * The call allocates nothing (its first call on a device looks up the array's address).  All calls
+ * The call allocates nothing.  Its first call on a device looks up the array's address, which is not
+ * a stream operation: make one call on every device outside any capture (any small input will do)
+ * before capturing the entry point into a graph; later calls only launch kernels.  All calls
  * on one GPU share that array: calls that overlap in time on one GPU (two streams, two threads)
  * race; calls on one stream are safe.
  * ------------------------------------------------------------------------------------------- */

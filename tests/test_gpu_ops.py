@@ -127,6 +127,31 @@ def test_attention_run_without_plan_is_refused(dev):
             torch.zeros_like(q), None, 1, 0, None, None, None, 0.0, 0.1, 1.0, 1e-4)
 
 
+def test_attention_run_checks_the_plan_vector_and_plans_go_with_their_workspace(dev):
+    """run() finds its plan by the int workspace: the plan vector the caller passes must be the one
+    that plan call returned, and a plan is dropped when its workspace is freed (a later tensor at the
+    same address must not find it)."""
+    import gc
+    from flashomni_amd import ops
+    heads = 2
+    m = make_ragged_masks([256], [256], heads, seed=25)
+    float_ws, int_ws, plan_info, qo_d, kv_d = _plan(dev, m, heads)
+    q = torch.zeros(256, heads, 128, dtype=torch.bfloat16, device=dev)
+    _run(dev, (float_ws, int_ws, plan_info, qo_d, kv_d), q, q, q, m, torch.zeros_like(q))
+    other = plan_info.clone()
+    other[3] += 1
+    with pytest.raises(RuntimeError, match="plan_info_vec is not the plan"):
+        _run(dev, (float_ws, int_ws, other, qo_d, kv_d), q, q, q, m, torch.zeros_like(q))
+    with pytest.raises(RuntimeError, match="planned number of heads"):
+        q3 = torch.zeros(256, heads + 1, 128, dtype=torch.bfloat16, device=dev)
+        _run(dev, (float_ws, int_ws, plan_info, qo_d, kv_d), q3, q, q, m, torch.zeros_like(q3))
+    key = (dev.index, int_ws.data_ptr())
+    assert key in ops._plans
+    del int_ws
+    gc.collect()
+    assert key not in ops._plans
+
+
 def test_symbols_rewritten_in_place_are_decoded_again(dev):
     """The symbol buffers are rewritten through the C ABI (a writer torch does not see: the tensors'
     version counters do not move); both the operator and the wrapper must run the new symbols."""

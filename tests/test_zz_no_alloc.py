@@ -100,3 +100,52 @@ def test_static_scratch_decoder_refuses_large_inputs(dev):
     rc = L.fo_decode_sparse_static(None, None, None, None, p, p, p, limit // 8 + 1, 8, 128, 1, p, p, p, p, p, p, p, p,
                                    None, torch.cuda.current_stream(dev).cuda_stream)
     assert rc == -1 and b"built-in scratch" in L.fo_last_error()
+
+
+def test_static_scratch_decoder_in_a_captured_graph(dev):
+    """The entry point is meant for callers that cannot allocate, a captured HIP graph among them.  Its
+    first call on a device looks up the address of the built-in array (not a stream operation): that
+    call is made eagerly here, as the header asks, and the capture follows.  The graph is replayed
+    three times with eager work and synchronisations in between, on symbols rewritten in place between
+    the replays; every replay must give what fo_decode_sparse gives for the symbols of that moment."""
+    from flashomni_amd import _lib
+    L = _lib.lib()
+    heads, ql, kl = 6, [700, 129], [640, 300]
+    masks = [make_ragged_masks(ql, kl, heads, 0.7, pk, seed=60 + i) for i, pk in enumerate((0.4, 0.8))]
+    qo, kv = torch.from_numpy(masks[0]["qo_indptr"]), torch.from_numpy(masks[0]["kv_indptr"])
+    sizes = torch.zeros(3, dtype=torch.int64)
+    _lib.check(L.fo_decode_sizes(qo.data_ptr(), kv.data_ptr(), 2, heads, 128, 128, sizes[0:].data_ptr(),
+                                 sizes[1:].data_ptr(), sizes[2:].data_ptr()))
+    n_blk, max_rows, max_nnz = (int(v) for v in sizes)
+    table = torch.empty((2, n_blk), dtype=torch.int32)
+    _lib.check(L.fo_sparse_block_table(qo.data_ptr(), 2, 128, table[0].data_ptr(), table[1].data_ptr(), n_blk,
+                                       sizes[0:].data_ptr()))
+    table_d, kv_d = table.to(dev), kv.to(dev)
+    t = lambda a: torch.from_numpy(a).to(dev)
+    sym = [t(masks[0][n]) for n in ("packed_info", "packed_keep", "info_indptr", "keep_indptr")]
+    b = _buffers(dev, max_rows, max_nnz)
+    head = [s.data_ptr() for s in sym] + [table_d[0].data_ptr(), table_d[1].data_ptr(), kv_d.data_ptr(), n_blk,
+                                          heads, 128, 0]
+    names = ("row_req", "row_qb", "row_head", "kv_row_ptr", "kv_idx", "counts", "order", "sched")
+    outs = [b[n].data_ptr() for n in names]
+
+    def static_call():
+        _lib.check(L.fo_decode_sparse_static(*head, *outs, b["shares"].data_ptr(),
+                                             torch.cuda.current_stream(dev).cuda_stream))
+
+    static_call()   # eager first call: resolves the array's address on this device
+    torch.cuda.synchronize(dev)
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        static_call()
+    for which in (1, 0, 1):
+        for s, n in zip(sym, ("packed_info", "packed_keep", "info_indptr", "keep_indptr")):
+            s.copy_(t(masks[which][n]))
+        for n in names + ("shares",):
+            b[n].fill_(-7)
+        torch.cuda.synchronize(dev)
+        graph.replay()
+        torch.cuda.synchronize(dev)
+        got = {k: v.cpu().numpy() for k, v in b.items()}
+        exp, _ = _decode(dev, masks[which], heads, False, True)
+        assert _assert_same(got, exp) > 0
