@@ -85,7 +85,8 @@ constexpr int kXcds = 8;
 constexpr int kListThreads = 1024;
 constexpr int kInlineCells = 256;  // up to this many cells the GEMM-Q kernel lists its quads itself
 constexpr int kWindow = 16;   // token blocks per scheduling window
-constexpr int kQuadInts = 8;  // b, r0, r1, c0, c1, valid mask, pad, pad
+constexpr int kQuadInts = 8;  // b, r0, r1, c0, c1, valid mask, c2 (strips), pad
+constexpr int kStrip = 0x10;  // in the valid mask: the item is a strip (one token block x three column blocks)
 
 template <typename T>
 struct Types;
@@ -303,6 +304,177 @@ __global__ void __launch_bounds__(kListThreads) gemm_quads_kernel(ListArgs a, Li
   }
 }
 
+// ---------------------------------------------------------------------------------------------
+// Row-pair list (GEMM-Q of large matrices).  With the flags of about four fifths of the units set at
+// random, quads formed inside a (window, column pair) cell fill 81 % of their wavefronts: a row
+// flagged in one column of the pair only finds a partner among sixteen rows half the time.  Here
+// token blocks are paired first (2i, 2i + 1) and the pair's columns are dealt over the whole width:
+// columns flagged in both rows two at a time into full quads, one left over together with a column
+// of one row (three units), and what only one row has three columns at a time into strips (one X
+// tile, three W tiles); two single leftovers share a quad.  Measured on the flags of the 14B-video
+// configuration: 5248 work items instead of 5865, 91 % of the wavefronts hold a unit; a strip's three
+// columns lie far apart, though, and few concurrent items share its W tiles: 9.4 GB fetched per
+// launch against 6.8 GB, and the launch is 2.5 % shorter, not 10 %.
+// One workgroup: a thread per row pair counts its items, a scan places them, every thread emits
+// its pair's items in place; the list is cut into eight equal queues as before.
+// ---------------------------------------------------------------------------------------------
+constexpr int kMaskWords = 4;  // column blocks of a row as bits: up to 256
+struct ColSet {
+  uint64_t w[kMaskWords];
+  __device__ __forceinline__ int count() const {
+    int n = 0;
+#pragma unroll
+    for (int i = 0; i < kMaskWords; ++i) n += __popcll(w[i]);
+    return n;
+  }
+  __device__ __forceinline__ int pop() {  // lowest column, or -1
+#pragma unroll
+    for (int i = 0; i < kMaskWords; ++i)
+      if (w[i]) {
+        const int b = __ffsll(static_cast<unsigned long long>(w[i])) - 1;
+        w[i] &= w[i] - 1;
+        return i * 64 + b;
+      }
+    return -1;
+  }
+};
+
+// f(row_sel, c0, c1, c2, valid): row_sel 0 = both rows (a quad), 1 / 2 = a strip of the first / second row
+template <typename F>
+__device__ __forceinline__ void for_each_pair_item(const ColSet& a, const ColSet& b, F&& f) {
+  ColSet both, oa, ob;
+#pragma unroll
+  for (int i = 0; i < kMaskWords; ++i) {
+    both.w[i] = a.w[i] & b.w[i];
+    oa.w[i] = a.w[i] & ~b.w[i];
+    ob.w[i] = b.w[i] & ~a.w[i];
+  }
+  int nb = both.count(), na = oa.count(), nbb = ob.count();
+  for (; nb >= 2; nb -= 2) {
+    const int c0 = both.pop(), c1 = both.pop();
+    f(0, c0, c1, 0, 0xF);
+  }
+  if (nb == 1) {
+    // the column left over takes a single column of one row with it: of the row whose strips that
+    // shortens (a count of 1 mod 3), else of any row that has one
+    const int c0 = both.pop();
+    const bool take_a = na > 0 && (nbb == 0 || na % 3 == 1 || nbb % 3 != 1);
+    if (take_a) {
+      f(0, c0, oa.pop(), 0, 0x7);
+      --na;
+    } else if (nbb > 0) {
+      f(0, c0, ob.pop(), 0, 0xD);
+      --nbb;
+    } else {
+      f(0, c0, c0, 0, 0x5);
+    }
+  }
+  for (; na >= 3; na -= 3) {
+    const int c0 = oa.pop(), c1 = oa.pop(), c2 = oa.pop();
+    f(1, c0, c1, c2, kStrip | 0x7);
+  }
+  for (; nbb >= 3; nbb -= 3) {
+    const int c0 = ob.pop(), c1 = ob.pop(), c2 = ob.pop();
+    f(2, c0, c1, c2, kStrip | 0x7);
+  }
+  if (na == 1 && nbb == 1) {
+    f(0, oa.pop(), ob.pop(), 0, 0x9);  // (r0, c0) and (r1, c1)
+    return;
+  }
+  if (na > 0) {
+    const int c0 = oa.pop(), c1 = na > 1 ? oa.pop() : c0;
+    f(1, c0, c1, c0, kStrip | (na > 1 ? 0x3 : 0x1));
+  }
+  if (nbb > 0) {
+    const int c0 = ob.pop(), c1 = nbb > 1 ? ob.pop() : c0;
+    f(2, c0, c1, c0, kStrip | (nbb > 1 ? 0x3 : 0x1));
+  }
+}
+
+__global__ void __launch_bounds__(kListThreads) gemm_pair_list_kernel(ListArgs a, ListGeom gm,
+                                                                     int32_t* __restrict__ quads,
+                                                                     int32_t* __restrict__ qoff) {
+  __shared__ int32_t s_cnt[kListThreads / 64];
+  __shared__ int32_t s_carry;
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int pairs_per_batch = (gm.n_row_tiles + 1) / 2;
+  const int n_pairs = gm.batch * pairs_per_batch;
+  // flagged column blocks of token block `row` of batch entry b
+  auto row_cols = [&](int b, int row, ColSet* out) {
+#pragma unroll
+    for (int i = 0; i < kMaskWords; ++i) out->w[i] = 0;
+    if (row >= gm.n_row_tiles) return;
+    const uint8_t* info = a.sparse_info + a.sparse_info_indptr[b];
+    const uint32_t blk = static_cast<uint32_t>(a.num_text_tokens + row * kTile) / a.sparse_q_size;
+    for (int c = 0; c < gm.n_col_tiles; ++c) {
+      const uint32_t head = static_cast<uint32_t>(c * kTile) / a.head_dim;
+      if (flag_bit(info, blk * a.num_heads + head)) out->w[c >> 6] |= uint64_t(1) << (c & 63);
+    }
+  };
+  if (tid == 0) s_carry = 0;
+  __syncthreads();
+  for (int base = 0; base < n_pairs; base += kListThreads) {
+    const int pr = base + tid;
+    ColSet ca, cb;
+    int b = 0, r0 = 0;
+    int32_t my_cnt = 0;
+    if (pr < n_pairs) {
+      b = pr / pairs_per_batch;
+      r0 = 2 * (pr - b * pairs_per_batch);
+      row_cols(b, r0, &ca);
+      row_cols(b, r0 + 1, &cb);
+      for_each_pair_item(ca, cb, [&](int, int, int, int, int) { ++my_cnt; });
+    }
+    int32_t incl = my_cnt;
+#pragma unroll
+    for (int d = 1; d < 64; d <<= 1) {
+      const int32_t up = __shfl_up(incl, d, 64);
+      if (lane >= d) incl += up;
+    }
+    if (lane == 63) s_cnt[wave] = incl;
+    __syncthreads();
+    int32_t q = s_carry + incl - my_cnt, total = 0;
+#pragma unroll
+    for (int w = 0; w < kListThreads / 64; ++w) {
+      const int32_t t = s_cnt[w];
+      if (w < wave) q += t;
+      total += t;
+    }
+    // Order inside a window of eight row pairs (eight neighbouring lanes): item i of every pair, then
+    // item i + 1 of every pair, ...  A pair's items walk its columns in ascending order, so the
+    // workgroups of an XCD, which take neighbouring items at the same time, meet in the same few W
+    // tiles as well as in the window's X tiles (pair after pair they would share two X tiles and
+    // fetch the whole width of W for them).
+    const int wl = lane & ~7;
+    int cnts[8];
+#pragma unroll
+    for (int j = 0; j < 8; ++j) cnts[j] = __shfl(my_cnt, wl + j, 64);
+    const int32_t base_w = __shfl(q, wl, 64);
+    int item_i = 0;
+    if (pr < n_pairs) {
+      for_each_pair_item(ca, cb, [&](int row_sel, int c0, int c1, int c2, int valid) {
+        int32_t at = base_w;
+#pragma unroll
+        for (int j = 0; j < 8; ++j) at += min(cnts[j], item_i) + ((j < (lane & 7) && cnts[j] > item_i) ? 1 : 0);
+        ++item_i;
+        int32_t* e = quads + kQuadInts * static_cast<int64_t>(at);
+        e[0] = b;
+        e[1] = row_sel == 2 ? r0 + 1 : r0;
+        e[2] = row_sel == 0 ? r0 + 1 : e[1];
+        e[3] = c0;
+        e[4] = c1;
+        e[5] = valid;
+        e[6] = c2;
+      });
+    }
+    __syncthreads();  // every thread has read the carry and the wavefront totals
+    if (tid == 0) s_carry += total;
+    __syncthreads();
+  }
+  const int32_t total = s_carry;
+  if (tid <= kXcds) qoff[tid] = static_cast<int32_t>(static_cast<int64_t>(total) * tid / kXcds);
+}
+
 // (the cursors of a launch that hands out its work items dynamically; a kernel, not a memset, so that
 // a captured graph replays it faithfully)
 __global__ void gemm_cursor_clear_kernel(int32_t* cursor) { cursor[threadIdx.x] = 0; }
@@ -424,12 +596,15 @@ __global__ void __launch_bounds__(kThreads) gemm_kernel(const GemmParams p) {
   // the tiles they share.)
   constexpr int P = 16;      // pieces per wavefront and slab: rows 32*wv + 8*jj.. (jj = 0..3) of every tile
   constexpr int PS = P / 4;  // pieces per substep
+  // valid & kStrip (GEMM-Q lists of large matrices): the item is a strip, one token block r[0] x up to
+  // three column blocks c[0], c[1], c2 (tiles: X r[0], W c2, W c[0], W c[1]; wavefronts 0..2 own the
+  // units, valid bits 0..2 say which exist)
   struct Item {
-    int bz, valid, r[2], c[2];
+    int bz, valid, r[2], c[2], c2;
   };
   // (called by all threads together: the listing form hands the entry over through LDS)
   auto decode_item = [&](int work) -> Item {
-    int bz, valid, r[2], c[2];
+    int bz, valid, r[2], c[2], c2 = 0;
     if (inline_list) {
       if constexpr (!kReduce) {
         // the thread whose cell holds quad q_lo + work walks the cell's quads up to it
@@ -466,6 +641,7 @@ __global__ void __launch_bounds__(kThreads) gemm_kernel(const GemmParams p) {
       c[0] = e[3];
       c[1] = e[4];
       valid = e[5];
+      c2 = e[6];
     } else {
       const int q = q_lo + work;
       bz = q / quads_per_batch;
@@ -494,6 +670,7 @@ __global__ void __launch_bounds__(kThreads) gemm_kernel(const GemmParams p) {
     Item it;
     it.bz = __builtin_amdgcn_readfirstlane(bz);
     it.valid = __builtin_amdgcn_readfirstlane(valid);
+    it.c2 = __builtin_amdgcn_readfirstlane(c2);
 #pragma unroll
     for (int u = 0; u < 2; ++u) {
       it.r[u] = __builtin_amdgcn_readfirstlane(r[u]);
@@ -630,6 +807,11 @@ __global__ void __launch_bounds__(kThreads) gemm_kernel(const GemmParams p) {
       rsrc[2 + u] = __builtin_amdgcn_make_buffer_rsrc(
           const_cast<T*>(wg + static_cast<int64_t>(item.c[u]) * kTile * p.k), 0, kTile * p.k * 2, 0x00020000);
     }
+    if constexpr (!kReduce) {
+      if (item.valid & kStrip)  // a strip's second tile is its third W tile
+        rsrc[1] = __builtin_amdgcn_make_buffer_rsrc(
+            const_cast<T*>(wg + static_cast<int64_t>(item.c2) * kTile * p.k), 0, kTile * p.k * 2, 0x00020000);
+    }
   };
   int ld_off[4];
 #pragma unroll
@@ -686,8 +868,18 @@ __global__ void __launch_bounds__(kThreads) gemm_kernel(const GemmParams p) {
   while (have) {
     const int bz = cur.bz, valid = cur.valid;
     // (no indexing by a run-time value: the item has to stay in scalar registers)
-    const int out_r = wr ? cur.r[1] : cur.r[0], out_c = wc ? cur.c[1] : cur.c[0];
-    const bool my_valid = (valid >> (wr * 2 + wc)) & 1;
+    int out_r = wr ? cur.r[1] : cur.r[0], out_c = wc ? cur.c[1] : cur.c[0];
+    bool my_valid = (valid >> (wr * 2 + wc)) & 1;
+    int a_tile = 2 + wc, b_tile = wr;  // LDS tiles of this wavefront's W and X operands
+    if constexpr (!kReduce) {
+      if (valid & kStrip) {
+        out_r = cur.r[0];
+        out_c = wv == 0 ? cur.c[0] : wv == 1 ? cur.c[1] : cur.c2;
+        my_valid = wv < 3 && ((valid >> wv) & 1);
+        a_tile = wv == 2 ? 1 : 2 + wv;
+        b_tile = 0;
+      }
+    }
     // (the next item is looked up here, while no accumulator is live)
     int next_work = work + per_xcd;
     if (popping) {
@@ -795,8 +987,8 @@ __global__ void __launch_bounds__(kThreads) gemm_kernel(const GemmParams p) {
           for (int i = 0; i < 16; ++i) acc[nt][mt][i] = 0.f;
       if (n_iter > 0) {
         // LDS byte offsets of this wavefront's operand rows inside a stage
-        const int a_base = (2 + wc) * kUnitBytes + l32 * kRowBytes;  // W rows nt*32 + l32
-        const int b_base = wr * kUnitBytes + l32 * kRowBytes;        // X rows mt*32 + l32
+        const int a_base = a_tile * kUnitBytes + l32 * kRowBytes;  // W rows nt*32 + l32
+        const int b_base = b_tile * kUnitBytes + l32 * kRowBytes;  // X rows mt*32 + l32
         x8 a[2][NT], b[2][MT];
         // operand read idx of substep sub of the slab in `stage` into register set sub & 1, in the order
         // the MFMAs need them: W rows 0, all X rows, W rows 1..3
@@ -1131,7 +1323,14 @@ int launch_half(GemmParams& p, const ListGeom& gm, bool use_flags, void* workspa
   la.num_heads = p.num_heads;
   la.head_dim = p.head_dim;
   la.num_text_tokens = p.num_text_tokens;
-  gemm_quads_kernel<<<1, kListThreads, 0, stream>>>(la, gm, quads, qoff);
+  // GEMM-Q of a wide matrix: items by row pair (quads and strips); otherwise quads by cell.  (From
+  // eight column blocks on, a pair's items, at most n_col_tiles / 2 + 3, fit the room sized for the
+  // cells' quads.)
+  if (!kReduce && use_flags && gm.n_col_tiles >= 8 && gm.n_col_tiles <= 64 * kMaskWords) {
+    gemm_pair_list_kernel<<<1, kListThreads, 0, stream>>>(la, gm, quads, qoff);
+  } else {
+    gemm_quads_kernel<<<1, kListThreads, 0, stream>>>(la, gm, quads, qoff);
+  }
   FO_CHECK_LAUNCH();
   p.quads = quads;
   p.qoff = qoff;

@@ -62,6 +62,36 @@ def test_gemm_q_matches_oracle_and_skips_tiles(dev, dtype, shape):
     assert rel_l2(out[changed], exp[changed]) <= REL_L2
 
 
+@pytest.mark.parametrize("case", [(2, 33077, 2048, 96, 16, 0.8), (2, 66100, 1280, 128, 20, 0.5), (1, 70000, 1024, 64, 8, 0.6),
+                                  (2, 40000, 2304, 64, 9, 0.25)])
+def test_gemm_q_large_lists_pair_rows_and_use_strips(dev, case):
+    """Matrices of more than 256 (window, column pair) cells and at least eight column blocks list their
+    work by row pair: full quads for the columns both token blocks have, strips of three column blocks
+    for what one of them has alone.  Whole output against the oracle (small K keeps that cheap), skipped
+    tiles byte for byte; flag densities that give mostly quads, a mix, mostly strips; a ragged last
+    token block, an odd number of token blocks, K = 96 (the slab that counts for one half), heads of
+    64 columns (a column block reads the flag of its first head) and of 256 (two column blocks per flag)."""
+    import flashomni_amd as fo
+    batch, m, n, k, heads, dens = case
+    nqb = (m + 127) // 128
+    info, packed, indptr = _flags(batch, nqb, heads, dens, seed=m)
+    g = torch.Generator(device=dev).manual_seed(m + k)
+    x = torch.randn(batch, m, k, generator=g, device=dev).to(torch.bfloat16)
+    w = (torch.randn(n, k, generator=g, device=dev) * 0.05).to(torch.bfloat16)
+    b = (torch.randn(n, generator=g, device=dev) * 0.05).to(torch.bfloat16)
+    out = torch.full((batch, m, n), -7.0, dtype=torch.bfloat16, device=dev)
+    fo.flashomni_gemm(x, w, heads, torch.from_numpy(packed).to(dev), torch.from_numpy(indptr).to(dev), 0, b, out=out)
+    exp = oracle.gemm_q(x.cpu(), w.cpu(), heads, packed, indptr, 0, b.cpu(),
+                        out=torch.full((batch, m, n), -7.0, dtype=torch.bfloat16))
+    out = out.cpu()
+    hd = n // heads
+    tile_head = (np.arange(n // 128) * 128) // hd    # the flag a (128 x 128) tile reads (gemm.cuh:50-58)
+    active = torch.from_numpy(info[:, :, tile_head]).repeat_interleave(128, 1)[:, :m].repeat_interleave(128, 2)
+    assert bool((out[~active] == -7.0).all()) and bool((exp[~active] == -7.0).all())
+    assert max_abs(out[active], exp[active]) <= MAX_ABS
+    assert rel_l2(out[active], exp[active]) <= REL_L2
+
+
 def test_gemm_q_is_full_equals_linear(dev):
     import flashomni_amd as fo
     x, w, b = _operands(1, 384, 256, 192, torch.bfloat16, seed=9)
@@ -350,6 +380,7 @@ def test_video_gemms_sampled_token_blocks(dev):
     fo.flashomni_gemm(x, w_q, H, pk, ip, 0, b_q, out=y)
     active = wl.sparse_info.to(dev).repeat_interleave(128, 0)[:M].repeat_interleave(128, 1)[None]
     assert bool((y[~active] == -7.0).all())
+    assert bool((y.view(-1, 128)[active.view(-1, 128)[:, 0]] != -7.0).any(-1).all())   # every flagged tile row written
     del active
     cache = fo.flashomni_gemm_reduction(x, w_o, H, pk, ip, 0, bias=b_o, is_for_cache=True,
                                         out_dtype=torch.float32)
