@@ -14,10 +14,18 @@
 // units).  A wavefront owns one unit: 128 x 128 accumulators (256 registers, kept in the accumulator
 // half of the register file), sixteen MFMAs per eight 128-bit operand reads.  (With eight wavefronts
 // of 64 x 128 the same loop spent a third more LDS reads per MFMA and ran 25 % slower.)  A list
-// kernel packs the flagged units of every (16-token-block window, column pair) cell into quads: rows
-// flagged in both columns pair up into full quads, rows flagged in one column pair up among
-// themselves, leftovers are merged; a 4-bit mask says which units of a quad exist (the wavefront of
-// a missing unit only moves data).  GEMM-O (and GEMM-Q with is_full) computes every unit: no list
+// kernel packs the flagged units of every (16-token-block window, column pair) cell into work items:
+// rows flagged in both columns pair up into full quads; rows flagged in one column go three at a time
+// into *column strips* (three token blocks x that column block: three X tiles and one W tile, three
+// wavefronts busy), what is left pairs up or is merged; a mask says which units of an item exist
+// (the wavefront of a missing unit only moves data).  With four fifths of the units flagged at
+// random (the 14B-video configuration) that fills 86 % of the wavefront slots against 81 % with
+// quads alone, from the same operand tiles, and the launch is 2 % shorter.  (Measured and dropped:
+// items dealt by row pair over the whole width, full quads for the columns both token blocks have and
+// strips of one token block x three column blocks for the rest: 91 % of the slots, but a strip's
+// three columns lie far apart and few concurrent items share its W tiles, 9.4 GB fetched per launch
+// against 6.8 GB, and the launch was 1.3 % shorter.  Either way the time per round of work items
+// rises with the fill.)  GEMM-O (and GEMM-Q with is_full) computes every unit: no list
 // then, the kernel derives its quads from the shape.  GEMM-O walks the union of the two token
 // blocks' selected heads; a token block that does not select a head reads that k step's X operand
 // as zeros.
@@ -85,8 +93,9 @@ constexpr int kXcds = 8;
 constexpr int kListThreads = 1024;
 constexpr int kInlineCells = 256;  // up to this many cells the GEMM-Q kernel lists its quads itself
 constexpr int kWindow = 16;   // token blocks per scheduling window
-constexpr int kQuadInts = 8;  // b, r0, r1, c0, c1, valid mask, c2 (strips), pad
-constexpr int kStrip = 0x10;  // in the valid mask: the item is a strip (one token block x three column blocks)
+constexpr int kQuadInts = 8;  // b, r0, r1, c0, c1, valid mask, r2 (column strips), pad
+constexpr int kColStrip = 0x20;        // in the valid mask: the item is a column strip (three token blocks x one column block)
+constexpr int kColStripSecond = 0x40;  // ... of the cell's second column
 
 template <typename T>
 struct Types;
@@ -204,41 +213,54 @@ __device__ __forceinline__ int pop_lowest(uint32_t* m) {
   return r;
 }
 
-// Packs a cell's flagged units into quads and calls f(r0, r1, valid) for each; r1 < 0 = no second
-// row.  valid bits: 1 = (r0,c0), 2 = (r0,c1), 4 = (r1,c0), 8 = (r1,c1).
+// Packs a cell's flagged units into work items and calls f(r0, r1, valid, r2) for each; r1 < 0 = no
+// second row.  Quads: valid bits 1 = (r0,c0), 2 = (r0,c1), 4 = (r1,c0), 8 = (r1,c1).  Column strips
+// (col_strips: units come from flags): valid = kColStrip | 7 (| kColStripSecond for the cell's second
+// column), rows r0, r1, r2 of that column.
 template <typename F>
-__device__ __forceinline__ void for_each_quad(uint32_t m0, uint32_t m1, F&& f) {
+__device__ __forceinline__ void for_each_quad(uint32_t m0, uint32_t m1, bool col_strips, F&& f) {
   uint32_t both = m0 & m1, only0 = m0 & ~m1, only1 = m1 & ~m0;
   while (__popc(both) >= 2) {
     const int r0 = pop_lowest(&both), r1 = pop_lowest(&both);
-    f(r0, r1, 0xF);
+    f(r0, r1, 0xF, 0);
+  }
+  if (col_strips) {
+    // rows flagged in one column only: three at a time into a column strip (three X tiles, one W tile)
+    while (__popc(only0) >= 3) {
+      const int r0 = pop_lowest(&only0), r1 = pop_lowest(&only0), r2 = pop_lowest(&only0);
+      f(r0, r1, kColStrip | 0x7, r2);
+    }
+    while (__popc(only1) >= 3) {
+      const int r0 = pop_lowest(&only1), r1 = pop_lowest(&only1), r2 = pop_lowest(&only1);
+      f(r0, r1, kColStrip | kColStripSecond | 0x7, r2);
+    }
   }
   while (__popc(only0) >= 2) {
     const int r0 = pop_lowest(&only0), r1 = pop_lowest(&only0);
-    f(r0, r1, 0x5);
+    f(r0, r1, 0x5, 0);
   }
   while (__popc(only1) >= 2) {
     const int r0 = pop_lowest(&only1), r1 = pop_lowest(&only1);
-    f(r0, r1, 0xA);
+    f(r0, r1, 0xA, 0);
   }
   // at most one row left in each class: merge them two by two
   if (both) {
     const int r0 = pop_lowest(&both);
     if (only0) {
-      f(r0, pop_lowest(&only0), 0x3 | 0x4);
+      f(r0, pop_lowest(&only0), 0x3 | 0x4, 0);
     } else if (only1) {
-      f(r0, pop_lowest(&only1), 0x3 | 0x8);
+      f(r0, pop_lowest(&only1), 0x3 | 0x8, 0);
     } else {
-      f(r0, -1, 0x3);
+      f(r0, -1, 0x3, 0);
     }
   }
   if (only0 && only1) {
     const int r0 = pop_lowest(&only0);
-    f(r0, pop_lowest(&only1), 0x1 | 0x8);
+    f(r0, pop_lowest(&only1), 0x1 | 0x8, 0);
   } else if (only0) {
-    f(pop_lowest(&only0), -1, 0x1);
+    f(pop_lowest(&only0), -1, 0x1, 0);
   } else if (only1) {
-    f(pop_lowest(&only1), -1, 0x2);
+    f(pop_lowest(&only1), -1, 0x2, 0);
   }
 }
 
@@ -264,7 +286,7 @@ __global__ void __launch_bounds__(kListThreads) gemm_quads_kernel(ListArgs a, Li
   for (int cell = lo; cell < hi; ++cell) {
     cell_masks(gm, cell, a.use_flags, a.sparse_info, a.sparse_info_indptr, a.sparse_q_size, a.num_heads,
                a.head_dim, a.num_text_tokens, &b, &row0, &cp, &m0, &m1);
-    for_each_quad(m0, m1, [&](int, int, int) { ++my_cnt; });
+    for_each_quad(m0, m1, a.use_flags != 0, [&](int, int, int, int) { ++my_cnt; });
   }
   // inclusive scan of the per-thread counts: inside a wavefront by lane shifts, then over the
   // sixteen wavefront totals
@@ -291,188 +313,22 @@ __global__ void __launch_bounds__(kListThreads) gemm_quads_kernel(ListArgs a, Li
     if (per > 1)  // with one cell per thread the masks of the counting pass are still at hand
       cell_masks(gm, cell, a.use_flags, a.sparse_info, a.sparse_info_indptr, a.sparse_q_size, a.num_heads,
                  a.head_dim, a.num_text_tokens, &b, &row0, &cp, &m0, &m1);
-    for_each_quad(m0, m1, [&](int r0, int r1, int valid) {
+    for_each_quad(m0, m1, a.use_flags != 0, [&](int r0, int r1, int valid, int r2) {
       int32_t* e = quads + kQuadInts * static_cast<int64_t>(q);
       e[0] = b;
       e[1] = row0 + r0;
       e[2] = row0 + (r1 < 0 ? r0 : r1);
-      e[3] = (valid & 0x5) ? 2 * cp : 2 * cp + 1;
-      e[4] = (valid & 0xA) ? 2 * cp + 1 : 2 * cp;
+      if (valid & kColStrip) {
+        e[3] = e[4] = (valid & kColStripSecond) ? 2 * cp + 1 : 2 * cp;
+      } else {
+        e[3] = (valid & 0x5) ? 2 * cp : 2 * cp + 1;
+        e[4] = (valid & 0xA) ? 2 * cp + 1 : 2 * cp;
+      }
       e[5] = valid;
+      e[6] = row0 + r2;
       ++q;
     });
   }
-}
-
-// ---------------------------------------------------------------------------------------------
-// Row-pair list (GEMM-Q of large matrices).  With the flags of about four fifths of the units set at
-// random, quads formed inside a (window, column pair) cell fill 81 % of their wavefronts: a row
-// flagged in one column of the pair only finds a partner among sixteen rows half the time.  Here
-// token blocks are paired first (2i, 2i + 1) and the pair's columns are dealt over the whole width:
-// columns flagged in both rows two at a time into full quads, one left over together with a column
-// of one row (three units), and what only one row has three columns at a time into strips (one X
-// tile, three W tiles); two single leftovers share a quad.  Measured on the flags of the 14B-video
-// configuration: 5248 work items instead of 5865, 91 % of the wavefronts hold a unit; a strip's three
-// columns lie far apart, though, and few concurrent items share its W tiles: 9.4 GB fetched per
-// launch against 6.8 GB, and the launch is 2.5 % shorter, not 10 %.
-// One workgroup: a thread per row pair counts its items, a scan places them, every thread emits
-// its pair's items in place; the list is cut into eight equal queues as before.
-// ---------------------------------------------------------------------------------------------
-constexpr int kMaskWords = 4;  // column blocks of a row as bits: up to 256
-struct ColSet {
-  uint64_t w[kMaskWords];
-  __device__ __forceinline__ int count() const {
-    int n = 0;
-#pragma unroll
-    for (int i = 0; i < kMaskWords; ++i) n += __popcll(w[i]);
-    return n;
-  }
-  __device__ __forceinline__ int pop() {  // lowest column, or -1
-#pragma unroll
-    for (int i = 0; i < kMaskWords; ++i)
-      if (w[i]) {
-        const int b = __ffsll(static_cast<unsigned long long>(w[i])) - 1;
-        w[i] &= w[i] - 1;
-        return i * 64 + b;
-      }
-    return -1;
-  }
-};
-
-// f(row_sel, c0, c1, c2, valid): row_sel 0 = both rows (a quad), 1 / 2 = a strip of the first / second row
-template <typename F>
-__device__ __forceinline__ void for_each_pair_item(const ColSet& a, const ColSet& b, F&& f) {
-  ColSet both, oa, ob;
-#pragma unroll
-  for (int i = 0; i < kMaskWords; ++i) {
-    both.w[i] = a.w[i] & b.w[i];
-    oa.w[i] = a.w[i] & ~b.w[i];
-    ob.w[i] = b.w[i] & ~a.w[i];
-  }
-  int nb = both.count(), na = oa.count(), nbb = ob.count();
-  for (; nb >= 2; nb -= 2) {
-    const int c0 = both.pop(), c1 = both.pop();
-    f(0, c0, c1, 0, 0xF);
-  }
-  if (nb == 1) {
-    // the column left over takes a single column of one row with it: of the row whose strips that
-    // shortens (a count of 1 mod 3), else of any row that has one
-    const int c0 = both.pop();
-    const bool take_a = na > 0 && (nbb == 0 || na % 3 == 1 || nbb % 3 != 1);
-    if (take_a) {
-      f(0, c0, oa.pop(), 0, 0x7);
-      --na;
-    } else if (nbb > 0) {
-      f(0, c0, ob.pop(), 0, 0xD);
-      --nbb;
-    } else {
-      f(0, c0, c0, 0, 0x5);
-    }
-  }
-  for (; na >= 3; na -= 3) {
-    const int c0 = oa.pop(), c1 = oa.pop(), c2 = oa.pop();
-    f(1, c0, c1, c2, kStrip | 0x7);
-  }
-  for (; nbb >= 3; nbb -= 3) {
-    const int c0 = ob.pop(), c1 = ob.pop(), c2 = ob.pop();
-    f(2, c0, c1, c2, kStrip | 0x7);
-  }
-  if (na == 1 && nbb == 1) {
-    f(0, oa.pop(), ob.pop(), 0, 0x9);  // (r0, c0) and (r1, c1)
-    return;
-  }
-  if (na > 0) {
-    const int c0 = oa.pop(), c1 = na > 1 ? oa.pop() : c0;
-    f(1, c0, c1, c0, kStrip | (na > 1 ? 0x3 : 0x1));
-  }
-  if (nbb > 0) {
-    const int c0 = ob.pop(), c1 = nbb > 1 ? ob.pop() : c0;
-    f(2, c0, c1, c0, kStrip | (nbb > 1 ? 0x3 : 0x1));
-  }
-}
-
-__global__ void __launch_bounds__(kListThreads) gemm_pair_list_kernel(ListArgs a, ListGeom gm,
-                                                                     int32_t* __restrict__ quads,
-                                                                     int32_t* __restrict__ qoff) {
-  __shared__ int32_t s_cnt[kListThreads / 64];
-  __shared__ int32_t s_carry;
-  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-  const int pairs_per_batch = (gm.n_row_tiles + 1) / 2;
-  const int n_pairs = gm.batch * pairs_per_batch;
-  // flagged column blocks of token block `row` of batch entry b
-  auto row_cols = [&](int b, int row, ColSet* out) {
-#pragma unroll
-    for (int i = 0; i < kMaskWords; ++i) out->w[i] = 0;
-    if (row >= gm.n_row_tiles) return;
-    const uint8_t* info = a.sparse_info + a.sparse_info_indptr[b];
-    const uint32_t blk = static_cast<uint32_t>(a.num_text_tokens + row * kTile) / a.sparse_q_size;
-    for (int c = 0; c < gm.n_col_tiles; ++c) {
-      const uint32_t head = static_cast<uint32_t>(c * kTile) / a.head_dim;
-      if (flag_bit(info, blk * a.num_heads + head)) out->w[c >> 6] |= uint64_t(1) << (c & 63);
-    }
-  };
-  if (tid == 0) s_carry = 0;
-  __syncthreads();
-  for (int base = 0; base < n_pairs; base += kListThreads) {
-    const int pr = base + tid;
-    ColSet ca, cb;
-    int b = 0, r0 = 0;
-    int32_t my_cnt = 0;
-    if (pr < n_pairs) {
-      b = pr / pairs_per_batch;
-      r0 = 2 * (pr - b * pairs_per_batch);
-      row_cols(b, r0, &ca);
-      row_cols(b, r0 + 1, &cb);
-      for_each_pair_item(ca, cb, [&](int, int, int, int, int) { ++my_cnt; });
-    }
-    int32_t incl = my_cnt;
-#pragma unroll
-    for (int d = 1; d < 64; d <<= 1) {
-      const int32_t up = __shfl_up(incl, d, 64);
-      if (lane >= d) incl += up;
-    }
-    if (lane == 63) s_cnt[wave] = incl;
-    __syncthreads();
-    int32_t q = s_carry + incl - my_cnt, total = 0;
-#pragma unroll
-    for (int w = 0; w < kListThreads / 64; ++w) {
-      const int32_t t = s_cnt[w];
-      if (w < wave) q += t;
-      total += t;
-    }
-    // Order inside a window of eight row pairs (eight neighbouring lanes): item i of every pair, then
-    // item i + 1 of every pair, ...  A pair's items walk its columns in ascending order, so the
-    // workgroups of an XCD, which take neighbouring items at the same time, meet in the same few W
-    // tiles as well as in the window's X tiles (pair after pair they would share two X tiles and
-    // fetch the whole width of W for them).
-    const int wl = lane & ~7;
-    int cnts[8];
-#pragma unroll
-    for (int j = 0; j < 8; ++j) cnts[j] = __shfl(my_cnt, wl + j, 64);
-    const int32_t base_w = __shfl(q, wl, 64);
-    int item_i = 0;
-    if (pr < n_pairs) {
-      for_each_pair_item(ca, cb, [&](int row_sel, int c0, int c1, int c2, int valid) {
-        int32_t at = base_w;
-#pragma unroll
-        for (int j = 0; j < 8; ++j) at += min(cnts[j], item_i) + ((j < (lane & 7) && cnts[j] > item_i) ? 1 : 0);
-        ++item_i;
-        int32_t* e = quads + kQuadInts * static_cast<int64_t>(at);
-        e[0] = b;
-        e[1] = row_sel == 2 ? r0 + 1 : r0;
-        e[2] = row_sel == 0 ? r0 + 1 : e[1];
-        e[3] = c0;
-        e[4] = c1;
-        e[5] = valid;
-        e[6] = c2;
-      });
-    }
-    __syncthreads();  // every thread has read the carry and the wavefront totals
-    if (tid == 0) s_carry += total;
-    __syncthreads();
-  }
-  const int32_t total = s_carry;
-  if (tid <= kXcds) qoff[tid] = static_cast<int32_t>(static_cast<int64_t>(total) * tid / kXcds);
 }
 
 // (the cursors of a launch that hands out its work items dynamically; a kernel, not a memset, so that
@@ -553,7 +409,7 @@ __global__ void __launch_bounds__(kThreads) gemm_kernel(const GemmParams p) {
         uint32_t m0, m1;
         cell_masks(gm, tid, true, p.sparse_info, p.sparse_info_indptr, p.sparse_q_size, p.num_heads,
                    p.head_dim, p.num_text_tokens, &b, &row0, &cp, &m0, &m1);
-        for_each_quad(m0, m1, [&](int, int, int) { ++cnt; });
+        for_each_quad(m0, m1, true, [&](int, int, int, int) { ++cnt; });
         s_cell_mask[2 * tid] = m0;
         s_cell_mask[2 * tid + 1] = m1;
       }
@@ -589,22 +445,21 @@ __global__ void __launch_bounds__(kThreads) gemm_kernel(const GemmParams p) {
 
   // ---- work items ----
   // A work item = a quad: four operand tiles per slab (X r0, X r1, W c0, W c1), wavefront = unit,
-  // 128 x 128 each.  (A second shape was measured and dropped: quads with two units that share a
+  // 128 x 128 each; or a column strip (X r0, X r1, W c0, X r2).  (Another shape was measured and dropped: quads with two units that share a
   // tile, computed by two wavefronts per unit at 64 x 128 each from three tiles.  Its slab takes as
   // long as a full one (nine LDS transfers per eight MFMAs saturate a wavefront's LDS path), and work
   // items of unequal length let the workgroups of an XCD drift apart in k, which costs the L2 hits on
   // the tiles they share.)
   constexpr int P = 16;      // pieces per wavefront and slab: rows 32*wv + 8*jj.. (jj = 0..3) of every tile
   constexpr int PS = P / 4;  // pieces per substep
-  // valid & kStrip (GEMM-Q lists of large matrices): the item is a strip, one token block r[0] x up to
-  // three column blocks c[0], c[1], c2 (tiles: X r[0], W c2, W c[0], W c[1]; wavefronts 0..2 own the
-  // units, valid bits 0..2 say which exist)
+  // valid & kColStrip (GEMM-Q with flags): the item is a column strip, three token blocks r[0], r[1],
+  // r2 x one column block c[0] (tiles: X r[0], X r[1], W c[0], X r2; wavefronts 0..2 own the units).
   struct Item {
-    int bz, valid, r[2], c[2], c2;
+    int bz, valid, r[2], c[2], r2;
   };
   // (called by all threads together: the listing form hands the entry over through LDS)
   auto decode_item = [&](int work) -> Item {
-    int bz, valid, r[2], c[2], c2 = 0;
+    int bz, valid, r[2], c[2], r2 = 0;
     if (inline_list) {
       if constexpr (!kReduce) {
         // the thread whose cell holds quad q_lo + work walks the cell's quads up to it
@@ -613,14 +468,19 @@ __global__ void __launch_bounds__(kThreads) gemm_kernel(const GemmParams p) {
           const int cp = tid % p.n_cp, t = tid / p.n_cp;
           const int w = t % p.n_win, b = t / p.n_win;
           int k = q - s_cell_pref[tid];
-          for_each_quad(s_cell_mask[2 * tid], s_cell_mask[2 * tid + 1], [&](int r0, int r1, int v) {
+          for_each_quad(s_cell_mask[2 * tid], s_cell_mask[2 * tid + 1], true, [&](int r0, int r1, int v, int r2) {
             if (k == 0) {
               s_entry[0] = b;
               s_entry[1] = w * kWindow + r0;
               s_entry[2] = w * kWindow + (r1 < 0 ? r0 : r1);
-              s_entry[3] = (v & 0x5) ? 2 * cp : 2 * cp + 1;
-              s_entry[4] = (v & 0xA) ? 2 * cp + 1 : 2 * cp;
+              if (v & kColStrip) {
+                s_entry[3] = s_entry[4] = (v & kColStripSecond) ? 2 * cp + 1 : 2 * cp;
+              } else {
+                s_entry[3] = (v & 0x5) ? 2 * cp : 2 * cp + 1;
+                s_entry[4] = (v & 0xA) ? 2 * cp + 1 : 2 * cp;
+              }
               s_entry[5] = v;
+              s_entry[6] = w * kWindow + r2;
             }
             --k;
           });
@@ -632,6 +492,7 @@ __global__ void __launch_bounds__(kThreads) gemm_kernel(const GemmParams p) {
         c[0] = s_entry[3];
         c[1] = s_entry[4];
         valid = s_entry[5];
+        r2 = s_entry[6];
       }
     } else if (p.quads) {
       const int32_t* e = p.quads + kQuadInts * static_cast<int64_t>(q_lo + work);
@@ -641,7 +502,7 @@ __global__ void __launch_bounds__(kThreads) gemm_kernel(const GemmParams p) {
       c[0] = e[3];
       c[1] = e[4];
       valid = e[5];
-      c2 = e[6];
+      r2 = e[6];
     } else {
       const int q = q_lo + work;
       bz = q / quads_per_batch;
@@ -670,7 +531,7 @@ __global__ void __launch_bounds__(kThreads) gemm_kernel(const GemmParams p) {
     Item it;
     it.bz = __builtin_amdgcn_readfirstlane(bz);
     it.valid = __builtin_amdgcn_readfirstlane(valid);
-    it.c2 = __builtin_amdgcn_readfirstlane(c2);
+    it.r2 = __builtin_amdgcn_readfirstlane(r2);
 #pragma unroll
     for (int u = 0; u < 2; ++u) {
       it.r[u] = __builtin_amdgcn_readfirstlane(r[u]);
@@ -808,9 +669,12 @@ __global__ void __launch_bounds__(kThreads) gemm_kernel(const GemmParams p) {
           const_cast<T*>(wg + static_cast<int64_t>(item.c[u]) * kTile * p.k), 0, kTile * p.k * 2, 0x00020000);
     }
     if constexpr (!kReduce) {
-      if (item.valid & kStrip)  // a strip's second tile is its third W tile
-        rsrc[1] = __builtin_amdgcn_make_buffer_rsrc(
-            const_cast<T*>(wg + static_cast<int64_t>(item.c2) * kTile * p.k), 0, kTile * p.k * 2, 0x00020000);
+      if (item.valid & kColStrip) {  // a column strip's fourth tile is its third X tile
+        const int rows_left = min(p.m - item.r2 * kTile, kTile);
+        rsrc[3] = __builtin_amdgcn_make_buffer_rsrc(
+            const_cast<T*>(xg + (static_cast<int64_t>(item.bz) * p.m + static_cast<int64_t>(item.r2) * kTile) * p.k), 0,
+            rows_left * p.k * 2, 0x00020000);
+      }
     }
   };
   int ld_off[4];
@@ -833,7 +697,7 @@ __global__ void __launch_bounds__(kThreads) gemm_kernel(const GemmParams p) {
     uint8_t* dst = smem + stage * kStageBytes + t * kUnitBytes + (32 * wv + 8 * (j & 3)) * kRowBytes + wr_off[j & 1];
     u32x4 v = stg[j];
     if constexpr (kHalf) {
-      if (t < 2) v &= keep;
+      if (t != 2) v &= keep;  // (every tile that can hold X; a W tile cleared along with its X tile changes nothing)
     }
     *reinterpret_cast<u32x4*>(dst) = v;
   };
@@ -872,12 +736,12 @@ __global__ void __launch_bounds__(kThreads) gemm_kernel(const GemmParams p) {
     bool my_valid = (valid >> (wr * 2 + wc)) & 1;
     int a_tile = 2 + wc, b_tile = wr;  // LDS tiles of this wavefront's W and X operands
     if constexpr (!kReduce) {
-      if (valid & kStrip) {
-        out_r = cur.r[0];
-        out_c = wv == 0 ? cur.c[0] : wv == 1 ? cur.c[1] : cur.c2;
+      if (valid & kColStrip) {
+        out_r = wv == 0 ? cur.r[0] : wv == 1 ? cur.r[1] : cur.r2;
+        out_c = cur.c[0];
         my_valid = wv < 3 && ((valid >> wv) & 1);
-        a_tile = wv == 2 ? 1 : 2 + wv;
-        b_tile = 0;
+        a_tile = 2;
+        b_tile = wv == 2 ? 3 : wv;
       }
     }
     // (the next item is looked up here, while no accumulator is live)
@@ -1323,14 +1187,7 @@ int launch_half(GemmParams& p, const ListGeom& gm, bool use_flags, void* workspa
   la.num_heads = p.num_heads;
   la.head_dim = p.head_dim;
   la.num_text_tokens = p.num_text_tokens;
-  // GEMM-Q of a wide matrix: items by row pair (quads and strips); otherwise quads by cell.  (From
-  // eight column blocks on, a pair's items, at most n_col_tiles / 2 + 3, fit the room sized for the
-  // cells' quads.)
-  if (!kReduce && use_flags && gm.n_col_tiles >= 8 && gm.n_col_tiles <= 64 * kMaskWords) {
-    gemm_pair_list_kernel<<<1, kListThreads, 0, stream>>>(la, gm, quads, qoff);
-  } else {
-    gemm_quads_kernel<<<1, kListThreads, 0, stream>>>(la, gm, quads, qoff);
-  }
+  gemm_quads_kernel<<<1, kListThreads, 0, stream>>>(la, gm, quads, qoff);
   FO_CHECK_LAUNCH();
   p.quads = quads;
   p.qoff = qoff;

@@ -64,10 +64,10 @@ def test_gemm_q_matches_oracle_and_skips_tiles(dev, dtype, shape):
 
 @pytest.mark.parametrize("case", [(2, 33077, 2048, 96, 16, 0.8), (2, 66100, 1280, 128, 20, 0.5), (1, 70000, 1024, 64, 8, 0.6),
                                   (2, 40000, 2304, 64, 9, 0.25)])
-def test_gemm_q_large_lists_pair_rows_and_use_strips(dev, case):
-    """Matrices of more than 256 (window, column pair) cells and at least eight column blocks list their
-    work by row pair: full quads for the columns both token blocks have, strips of three column blocks
-    for what one of them has alone.  Whole output against the oracle (small K keeps that cheap), skipped
+def test_gemm_q_large_lists_with_column_strips(dev, case):
+    """Matrices of more than 256 (window, column pair) cells get their work list from the list kernel:
+    full quads for rows flagged in both columns of a cell, column strips (three token blocks x one column
+    block) for rows flagged in one.  Whole output against the oracle (small K keeps that cheap), skipped
     tiles byte for byte; flag densities that give mostly quads, a mix, mostly strips; a ragged last
     token block, an odd number of token blocks, K = 96 (the slab that counts for one half), heads of
     64 columns (a column block reads the flag of its first head) and of 256 (two column blocks per flag)."""
