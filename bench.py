@@ -570,7 +570,9 @@ def main():
     for name, d in kernels.items():
         log("[bench]", name, json.dumps(d))
 
-    big_iters, big_warm = max(3, min(K, 10)), 2
+    # (the millisecond-scale launches of configs 3 and 4: a few tens of milliseconds of the same launch before
+    # timing, so that clocks and caches are those of a steady run)
+    big_iters, big_warm = max(3, min(K, 20)), 8
     cpu_big = {}
     for idx in (3, 4):
         if idx in configs:
