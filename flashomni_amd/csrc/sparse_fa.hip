@@ -343,6 +343,14 @@ sparse_fa_kernel(const FaParams p) {
   const int wv = __builtin_amdgcn_readfirstlane(tid >> 6);  // wavefront index, kept scalar
   const int qs = wv & 3, kg = wv >> 2;
   const int l32 = lane & 31, g = lane >> 5;
+  // The lane index, worked out again where it is called (two instructions) and opaque to the
+  // compiler: address terms derived from the kernel-wide `lane` are computed once per launch, find no
+  // register across the main loop and come back from scratch memory where they are used.
+  auto fresh_lane = [&]() __attribute__((always_inline)) {
+    int l = static_cast<int>(__builtin_amdgcn_mbcnt_hi(~0u, __builtin_amdgcn_mbcnt_lo(~0u, 0u)));
+    asm volatile("" : "+v"(l));
+    return l;
+  };
   const float c = p.sm_scale_log2;
   const TQK* __restrict__ qp = static_cast<const TQK*>(p.q);
   const TQK* __restrict__ kp = static_cast<const TQK*>(p.k);
@@ -390,12 +398,16 @@ sparse_fa_kernel(const FaParams p) {
   // shares (the same heads' K and V).  A share's items are consecutive rows of `order`, known from
   // the start: their records are gathered sixteen at a time, all in parallel, so that between two
   // rows only the kv block list has to be fetched.
-  const int ev_share = s_queue[10], ev_total = s_queue[11], ev_n = s_queue[12], ev_rows = s_queue[13];
-  const bool even = kGroups == 2 && s_queue[9] != 0 && p.shares != nullptr && p.split_ws != nullptr &&
+  // (workgroup-uniform words: made scalar, so that none of them occupies a vector register for the
+  // whole launch)
+  auto queue_word = [&](int i) { return __builtin_amdgcn_readfirstlane(s_queue[i]); };
+  const int ev_share = queue_word(10), ev_total = queue_word(11), ev_n = queue_word(12), ev_rows = queue_word(13);
+  const bool even = kGroups == 2 && queue_word(9) != 0 && p.shares != nullptr && p.split_ws != nullptr &&
                     static_cast<int>(gridDim.x) == ev_n;
   const int ev_j = (ev_n & (kXcds - 1)) == 0 ? (blockIdx.x & (kXcds - 1)) * (ev_n / kXcds) + blockIdx.x / kXcds
                                              : static_cast<int>(blockIdx.x);
   auto fill_items = [&](int batch_base) {
+    const int lane = fresh_lane();
     if (lane < kItemBatch) {
       RowInfo it;
       it.row = -1;
@@ -435,12 +447,14 @@ sparse_fa_kernel(const FaParams p) {
       s_items[lane] = it;
     }
   };
-  const bool have_records = s_queue[14] != 0 && p.shares != nullptr;
+  const bool have_records = queue_word(14) != 0 && p.shares != nullptr;
   int first_queue = 0;  // kept by the popping lane (the first pop is lane 0's, the others lane 256's)
   // One wavefront: lane 0 takes the next item (even shares: from the gathered records; otherwise it
   // pops a row and gathers its metadata, two rounds of loads), then all lanes copy the row's kv
   // block list; both go to LDS for the whole workgroup.
   auto fetch_next = [&](int slot_idx) {
+    slot_idx = __builtin_amdgcn_readfirstlane(slot_idx);
+    const int lane = fresh_lane();
     RowInfo ri;
     ri.row = -1;
     ri.ptr0 = 0;
@@ -526,7 +540,10 @@ sparse_fa_kernel(const FaParams p) {
     const int nb = __builtin_amdgcn_readfirstlane(ri.nb);
     const uint16_t* const s_blk = s_blk2[row_it & 1];
 
-    const int my_row = qs * 32 + l32;  // q row of this lane inside the block
+    // (the lane's q row, from a lane index worked out here: see fresh_lane)
+    const int lane_p = fresh_lane();
+    const int l32_p = lane_p & 31, g_p = lane_p >> 5;
+    const int my_row = qs * 32 + l32_p;  // q row of this lane inside the block
     const bool row_ok = my_row < q_rows;
     // row r of the item -> its token (relative to q_begin) and q head (relative to head_q0)
     // (a compile-time variant: as a run-time branch the mapping cost the ungrouped kernel 7 % at the
@@ -534,7 +551,7 @@ sparse_fa_kernel(const FaParams p) {
     const int gq = kGqaPack ? p.gqa_pack : 0;
     const int head_q0 = gq ? head * gq : head;
     auto row_at = [&](int r, int& tok, int& hq) __attribute__((always_inline)) {
-      if (gq) {
+      if constexpr (kGqaPack) {
         const uint32_t pr = static_cast<uint32_t>(qb) * kBlockQ + r;
         tok = static_cast<int>(pr / static_cast<uint32_t>(gq));
         hq = static_cast<int>(pr - tok * gq);
@@ -557,11 +574,11 @@ sparse_fa_kernel(const FaParams p) {
     if (nb == 0) {
       // listed row without kv blocks: zeros, lse = -5e4
       if (row_ok && kg == 0) {
-        T* dst = op + q_tok * p.o_sn + static_cast<int64_t>(my_head) * p.o_sh + g * 64;
+        T* dst = op + q_tok * p.o_sn + static_cast<int64_t>(my_head) * p.o_sh + g_p * 64;
         const u32x4 z = {0u, 0u, 0u, 0u};
 #pragma unroll
         for (int j = 0; j < 8; ++j) reinterpret_cast<u32x4*>(dst)[j] = z;
-        if (p.lse && g == 0) p.lse[q_tok * p.num_heads + my_head] = kNegInf;
+        if (p.lse && g_p == 0) p.lse[q_tok * p.num_heads + my_head] = kNegInf;
       }
       if (wv == kFetchWave) fetch_next((row_it + 1) & 1);
       continue;
@@ -636,6 +653,8 @@ sparse_fa_kernel(const FaParams p) {
       {
         const uint8_t* q_head = reinterpret_cast<const uint8_t*>(
             qp + static_cast<int64_t>(q_begin) * p.q_sn + static_cast<int64_t>(head_q0) * p.q_sh);
+        const int ln_q = fresh_lane();
+        const int cp_row = ln_q >> 4, cp_chunk = ((ln_q & 15) ^ swz(4 * qs + cp_row)) * 8;
 #pragma unroll
         for (int n = 0; n < 8; ++n) {
           int r = 4 * (4 * n + qs) + cp_row;
@@ -654,8 +673,8 @@ sparse_fa_kernel(const FaParams p) {
       u32x4 pA[2], pB[2];  // P of a step: 2 x 8 rounded values, as 32-bit pairs
       f32x16 sA, sB;
       {
-        int q_rd_base = k_rd_base, q_rd_x = k_rd_x;
-        asm volatile("" : "+v"(q_rd_base), "+v"(q_rd_x));
+        const int ln_r = fresh_lane();
+        const int q_rd_base = (ln_r & 31) * kRowBytes, q_rd_x = ((ln_r >> 5) ^ swz(ln_r & 31)) << 4;
         const uint8_t* qt = smem + 4 * kBuf + qs * 32 * kRowBytes + q_rd_base;
 #pragma unroll
         for (int ks = 0; ks < 8; ++ks) qreg[ks] = *reinterpret_cast<const x8*>(qt + (q_rd_x ^ (ks << 5)));
@@ -868,6 +887,11 @@ sparse_fa_kernel(const FaParams p) {
       }
 #pragma unroll
       for (int i = 0; i < 4; ++i) o_acc[i] = TT::mfma(vop[i], __builtin_bit_cast(x8, pB[1]), o_acc[i]);
+      // The copies of the steps past the row's end (the loop asks for K four and V two steps ahead,
+      // whatever is left of the row) are still in flight: they must have landed before the epilogue
+      // lays the finished row out in the same LDS.  (Nothing else waits for them: the barrier below
+      // orders LDS accesses, not these copies, which the compiler does not see.)
+      __builtin_amdgcn_s_waitcnt(0x0f70);  // vmcnt(0)
     } else {
     // Q operand.  A lane needs q row l32 of its sub-tile, 16 bytes out of every 32 (fp8: 32 of 64):
     // fetched straight from memory that is 64 scattered pieces per instruction (measured: ~4 k
@@ -881,7 +905,7 @@ sparse_fa_kernel(const FaParams p) {
     if constexpr (kFp8) {
       // (fp8 Q, half the bytes, is still fetched directly: with the LDS detour hipcc arranges the
       // main loop of this instantiation less well, which costs more than the detour saves)
-      const uint8_t* src = qp + q_tok * p.q_sn + static_cast<int64_t>(my_head) * p.q_sh + g * 32;
+      const uint8_t* src = qp + q_tok * p.q_sn + static_cast<int64_t>(my_head) * p.q_sh + g_p * 32;
 #pragma unroll
       for (int sl = 0; sl < 2; ++sl) {
         const i32x4 lo = *reinterpret_cast<const i32x4*>(src + sl * 64);
@@ -890,7 +914,7 @@ sparse_fa_kernel(const FaParams p) {
       }
       if constexpr (kQLo) {
         const uint8_t* src2 = static_cast<const uint8_t*>(p.q_lo) + q_tok * p.q_sn +
-                              static_cast<int64_t>(my_head) * p.q_sh + g * 32;
+                              static_cast<int64_t>(my_head) * p.q_sh + g_p * 32;
 #pragma unroll
         for (int sl = 0; sl < 2; ++sl) {
           const i32x4 lo = *reinterpret_cast<const i32x4*>(src2 + sl * 64);
@@ -902,6 +926,8 @@ sparse_fa_kernel(const FaParams p) {
       const uint8_t* q_head = reinterpret_cast<const uint8_t*>(
           qp + static_cast<int64_t>(q_begin) * p.q_sn + static_cast<int64_t>(head_q0) * p.q_sh);
       const uint32_t qdst = lds_group + kStageBytes + kKBytes + qs * 1024;
+      const int ln_q = fresh_lane();
+      const int cp_row = ln_q >> 4, cp_chunk = ((ln_q & 15) ^ swz(4 * qs + cp_row)) * 8;
 #pragma unroll
       for (int n = 0; n < 4; ++n) {
         int r = kg * 64 + 4 * (4 * n + qs) + cp_row;
@@ -971,6 +997,9 @@ sparse_fa_kernel(const FaParams p) {
           copy16_to_lds((n < kPerTerm ? kt : kt_lo) + (n % kPerTerm) * k_jstep, k_voff, kdst + n * 4096);
       } else {
         // ragged tail: re-read the last valid row, never overrun
+        const int ln_c = fresh_lane();
+        const int cp_row = ln_c >> 4, cp_chunk = ((ln_c & 15) ^ swz(4 * qs + cp_row)) * 8;
+        const int cp8_row = ln_c >> 3, cp8_chunk = ((ln_c & 7) ^ ((4 * (qs & 1) + (ln_c >> 4)) & 7)) * 16;
 #pragma unroll
         for (int n = 0; n < kKCopies; ++n) {
           int r = (kFp8 ? 8 : 4) * (4 * (n % kPerTerm) + qs) + (kFp8 ? cp8_row : cp_row);
@@ -1000,6 +1029,8 @@ sparse_fa_kernel(const FaParams p) {
       const int valid = cp_valid;
       cp_pending = valid == kTileKV;
       if (__builtin_expect(!cp_pending, 0)) {
+        const int ln_c = fresh_lane();
+        const int cp_row = ln_c >> 4, cp_chunk = ((ln_c & 15) ^ swz(4 * qs + cp_row)) * 8;
 #pragma unroll
         for (int n = 0; n < kVCopies; ++n) {
           int r = 4 * (4 * n + qs) + cp_row;
@@ -1065,8 +1096,8 @@ sparse_fa_kernel(const FaParams p) {
     if constexpr (!kFp8) {
       // (the lane terms are made opaque here: otherwise the eight read addresses are worked out once
       // per kernel, live across the main loop, and their reloads wait for every copy in flight)
-      int q_rd_base = k_rd_base, q_rd_x = k_rd_x;
-      asm volatile("" : "+v"(q_rd_base), "+v"(q_rd_x));
+      const int ln_r = fresh_lane();
+      const int q_rd_base = (ln_r & 31) * kRowBytes, q_rd_x = ((ln_r >> 5) ^ swz(ln_r & 31)) << 4;
       const uint8_t* qt = smem + (qs >> 1) * kGroupBytes + kStageBytes + kKBytes + (qs & 1) * 32 * kRowBytes +
                           q_rd_base;
 #pragma unroll
@@ -1338,6 +1369,15 @@ sparse_fa_kernel(const FaParams p) {
     }  // !kPipe
 
     // ---- merge the two kv groups through LDS, then write the row ----
+    // (this lane's row, worked out again: what the prologue derived from the lane index would have
+    // to live through the main loop, i.e. in scratch memory)
+    const int lane_m = fresh_lane();
+    const int l32_e = lane_m & 31, g_e = lane_m >> 5;
+    const bool row_ok_e = qs * 32 + l32_e < q_rows;
+    int tok_e, hq_e;
+    row_at(row_ok_e ? qs * 32 + l32_e : q_rows - 1, tok_e, hq_e);
+    const int64_t q_tok_e = q_begin + tok_e;
+    const int my_head_e = head_q0 + hq_e;
     __syncthreads();  // all tile reads done: the tile buffers can be reused
     f32x4* mo = reinterpret_cast<f32x4*>(smem);
     float* md = reinterpret_cast<float*>(smem + kMergeOBytes);
@@ -1350,10 +1390,10 @@ sparse_fa_kernel(const FaParams p) {
             f32x4 t4;
 #pragma unroll
             for (int j = 0; j < 4; ++j) t4[j] = o_acc[dt][i4 * 4 + j];
-            mo[(qs * 16 + dt * 4 + i4) * 64 + lane] = t4;
+            mo[(qs * 16 + dt * 4 + i4) * 64 + lane_m] = t4;
           }
-        md[(qs * 64 + lane) * 2 + 0] = m_run;
-        md[(qs * 64 + lane) * 2 + 1] = d_part;
+        md[(qs * 64 + lane_m) * 2 + 0] = m_run;
+        md[(qs * 64 + lane_m) * 2 + 1] = d_part;
       }
       __syncthreads();
     }
@@ -1362,7 +1402,7 @@ sparse_fa_kernel(const FaParams p) {
     // A lane owns one q row and runs of four d: stored from here, a row would leave as 32 scattered
     // 8-byte pieces per instruction (measured: ~12 k cycles per row).  The finished row goes through
     // a padded LDS tile instead and leaves in 16-byte pieces, 16 consecutive lanes per 256-byte row.
-    int ln_out = l32;
+    int ln_out = l32_e;
     asm volatile("" : "+v"(ln_out));  // (not hoisted out of the row loop and spilled)
     uint8_t* const out_row = smem + G::kOutOff + (qs * 32 + ln_out) * kOutRowBytes;
     bool store_row = parts == 1;
@@ -1377,12 +1417,12 @@ sparse_fa_kernel(const FaParams p) {
           x4 out;
 #pragma unroll
           for (int j = 0; j < 4; ++j) out[j] = static_cast<T>(o_acc[dt][i4 * 4 + j] * inv);
-          *reinterpret_cast<x4*>(out_row + (dt * 32 + i4 * 8 + g * 4) * sizeof(T)) = out;
+          *reinterpret_cast<x4*>(out_row + (dt * 32 + i4 * 8 + g_e * 4) * sizeof(T)) = out;
         }
-      if (row_ok && p.lse && g == 0) p.lse[q_tok * p.num_heads + my_head] = __builtin_amdgcn_logf(d_tot) + m_run;
+      if (row_ok_e && p.lse && g_e == 0) p.lse[q_tok_e * p.num_heads + my_head_e] = __builtin_amdgcn_logf(d_tot) + m_run;
     }
     if (kGroups == 2 && kg == 0) {
-      const float m1 = md[(qs * 64 + lane) * 2 + 0], d1 = md[(qs * 64 + lane) * 2 + 1];
+      const float m1 = md[(qs * 64 + lane_m) * 2 + 0], d1 = md[(qs * 64 + lane_m) * 2 + 1];
       const float m = fmaxf(m_run, m1);
       const float a0 = __builtin_amdgcn_exp2f(m_run - m);
       const float a1 = __builtin_amdgcn_exp2f(m1 - m);
@@ -1395,7 +1435,7 @@ sparse_fa_kernel(const FaParams p) {
         // free here), so their latencies overlap
         f32x4 t4[16];
 #pragma unroll
-        for (int e = 0; e < 16; ++e) t4[e] = mo[(qs * 16 + e) * 64 + lane];
+        for (int e = 0; e < 16; ++e) t4[e] = mo[(qs * 16 + e) * 64 + lane_m];
         __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
         for (int dt = 0; dt < 4; ++dt)
@@ -1405,16 +1445,16 @@ sparse_fa_kernel(const FaParams p) {
 #pragma unroll
             for (int j = 0; j < 4; ++j)
               out[j] = static_cast<T>(o_acc[dt][i4 * 4 + j] * w0 + t4[dt * 4 + i4][j] * w1);
-            *reinterpret_cast<x4*>(out_row + (dt * 32 + i4 * 8 + g * 4) * sizeof(T)) = out;
+            *reinterpret_cast<x4*>(out_row + (dt * 32 + i4 * 8 + g_e * 4) * sizeof(T)) = out;
           }
-        if (row_ok && p.lse && g == 0)
-          p.lse[q_tok * p.num_heads + my_head] = __builtin_amdgcn_logf(d_tot) + m;
+        if (row_ok_e && p.lse && g_e == 0)
+          p.lse[q_tok_e * p.num_heads + my_head_e] = __builtin_amdgcn_logf(d_tot) + m;
       } else {
         // one part of a row cut at share boundaries: fold kv group 1 in without normalising; the
         // accumulators then hold this workgroup's partial result (reference point m, sum d_tot)
         f32x4 t4[16];
 #pragma unroll
-        for (int e = 0; e < 16; ++e) t4[e] = mo[(qs * 16 + e) * 64 + lane];
+        for (int e = 0; e < 16; ++e) t4[e] = mo[(qs * 16 + e) * 64 + lane_m];
         __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
         for (int e = 0; e < 16; ++e)
@@ -1439,9 +1479,7 @@ sparse_fa_kernel(const FaParams p) {
           // same lane layout as the LDS merge area; two planes of 8-byte pairs, so that each store
           // instruction covers 512 contiguous bytes
           float* part_ws = p.split_ws + static_cast<int64_t>(part_area(split_slot, part)) * kSplitPartFloats;
-          // (opaque lane index: see the row store below)
-          int ln = lane;
-          asm volatile("" : "+v"(ln));
+          const int ln = fresh_lane();
           float* lane_ws = part_ws + (qs * 16 * 2 * 64 + ln) * 2;
 #pragma unroll
           for (int e = 0; e < 16; ++e) {
@@ -1472,7 +1510,7 @@ sparse_fa_kernel(const FaParams p) {
               m_p[i] = m_own;
               d_p[i] = d_own;
             } else {
-              load_pair_device(part_base(i) + 128 * 128 + (qs * 64 + lane) * 2, m_p[i], d_p[i]);
+              load_pair_device(part_base(i) + 128 * 128 + (qs * 64 + lane_m) * 2, m_p[i], d_p[i]);
             }
             m_all = fmaxf(m_all, m_p[i]);
           }
@@ -1482,8 +1520,7 @@ sparse_fa_kernel(const FaParams p) {
           for (int dt = 0; dt < 4; ++dt)
 #pragma unroll
             for (int e = 0; e < 16; ++e) acc[dt][e] = 0.f;
-          int ln = lane;
-          asm volatile("" : "+v"(ln));
+          const int ln = fresh_lane();
           for (int i = 0; i < parts; ++i) {
             const float a = __builtin_amdgcn_exp2f(m_p[i] - m_all);
             d_all = __builtin_fmaf(d_p[i], a, d_all);
@@ -1517,10 +1554,10 @@ sparse_fa_kernel(const FaParams p) {
               x4 out;
 #pragma unroll
               for (int j = 0; j < 4; ++j) out[j] = static_cast<T>(acc[dt][i4 * 4 + j] * inv);
-              *reinterpret_cast<x4*>(out_row + (dt * 32 + i4 * 8 + g * 4) * sizeof(T)) = out;
+              *reinterpret_cast<x4*>(out_row + (dt * 32 + i4 * 8 + g_e * 4) * sizeof(T)) = out;
             }
-          if (row_ok && p.lse && g == 0)
-            p.lse[q_tok * p.num_heads + my_head] = __builtin_amdgcn_logf(d_all) + m_all;
+          if (row_ok_e && p.lse && g_e == 0)
+            p.lse[q_tok_e * p.num_heads + my_head_e] = __builtin_amdgcn_logf(d_all) + m_all;
         }
         if (tid == 0) p.sched[kSchedArrived + split_slot] = 0;  // re-armed for the next launch
         store_row = true;
@@ -1532,10 +1569,9 @@ sparse_fa_kernel(const FaParams p) {
     if (store_row) {
       __syncthreads();  // the row is complete in the LDS tile
       T* dst = op + static_cast<int64_t>(q_begin) * p.o_sn + static_cast<int64_t>(head_q0) * p.o_sh;
-      // (the lane index is made opaque here: otherwise the per-lane address terms are computed once
+      // (the lane index is worked out afresh here: otherwise the per-lane address terms are computed once
       // per kernel, spilled, and every reload waits for the store before it)
-      int ln = lane;
-      asm volatile("" : "+v"(ln));
+      const int ln = fresh_lane();
       constexpr int kRowsPerWave = kBlockQ / kWaves;
       const int r0 = wv * kRowsPerWave + (ln >> 4), chunk = ln & 15;
       u32x4 v[kRowsPerWave / 4];
