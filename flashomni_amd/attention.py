@@ -151,7 +151,8 @@ class PlannedBatch:
         self.max_rows = max_rows
         self.share_rows = share_rows
         self.split_ok = self._split_ws_ok()
-        self.decoded = None  # (is_full, stream) of the list the work-list buffers hold, or None
+        # [is_full, stream, streams already ordered after it] of the list the work-list buffers hold
+        self.decoded = None
 
     def float_ws_bytes(self) -> int:
         return self.float_ws.numel() * self.float_ws.element_size()
@@ -202,21 +203,24 @@ class PlannedBatch:
                 stream.cuda_stream))
         # remembered for reuse_decoded: which stream the list was decoded on (a run on another
         # stream must be ordered after it)
-        self.decoded = (bool(is_full), stream)
+        self.decoded = (bool(is_full), stream, [])
         return wl
 
     def reuse_decoded(self, is_full: bool) -> DecodedWorkList:
         """The work list of the last decode, ordered before the current stream's work."""
         if self.decoded is None:
             raise RuntimeError("reuse_decoded=True needs an earlier decode() or run() after plan()")
-        was_full, stream = self.decoded
+        was_full, stream, ordered = self.decoded
         if was_full != bool(is_full):
             raise RuntimeError("reuse_decoded=True: the last decode was made with is_full=%s" % was_full)
         cur = torch.cuda.current_stream(self.device)
-        if cur != stream and not torch.cuda.is_current_stream_capturing():
+        # one wait per (decode, stream): later work on a stream that has waited is behind the decode
+        # already, and a wait in front of every launch costs each one 2-3 us
+        if cur != stream and cur not in ordered and not torch.cuda.is_current_stream_capturing():
             ev = torch.cuda.Event()
             ev.record(stream)
             cur.wait_event(ev)
+            ordered.append(cur)
         return self.worklist
 
     def launch(self, q, k, v, out, lse, kv_layout, sm_scale, q_scale=None, k_scale=None, q_lo=None,

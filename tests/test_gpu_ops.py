@@ -205,6 +205,42 @@ def test_symbols_rewritten_in_place_are_decoded_again(dev):
     assert max_abs(o_reuse.cpu()[touched], exp_b[touched]) <= 2e-2
 
 
+def test_reuse_decoded_from_another_stream_waits_once_per_decode(dev):
+    """A list decoded on a side stream and run from the current one: the first run waits for the
+    decode, later ones on the same stream are behind it already (no further event), and a new decode
+    is waited for again.  Each result is the oracle's for the symbols of its decode."""
+    import flashomni_amd as fo
+    heads = 2
+    ma = make_ragged_masks([384], [384], heads, 0.7, 0.6, seed=5)
+    mb = make_ragged_masks([384], [384], heads, 0.7, 0.6, seed=6)
+    g = torch.Generator().manual_seed(5)
+    q, k, v = (torch.randn(384, heads, 128, generator=g).to(torch.bfloat16) for _ in range(3))
+    qd, kd, vd = q.to(dev), k.to(dev), v.to(dev)
+    t = lambda a: torch.from_numpy(a).to(dev)
+    w = fo.BatchFlashOmniFAWithRaggedKVWrapper(torch.empty(128 << 20, dtype=torch.uint8, device=dev))
+    w.plan(t(ma["qo_indptr"]), t(ma["kv_indptr"]), heads, heads, 128, q_data_type=torch.bfloat16)
+    side = torch.cuda.Stream(device=dev)
+    out0 = sentinel_like((384, heads, 128), torch.bfloat16)
+    for m in (ma, mb):
+        sym = (t(m["packed_info"]), t(m["packed_keep"]), t(m["info_indptr"]), t(m["keep_indptr"]))
+        exp = oracle.sparse_attention(q, k, v, m["packed_info"], m["packed_keep"], m["info_indptr"],
+                                      m["keep_indptr"], m["qo_indptr"], m["kv_indptr"], out=out0.clone())
+        side.wait_stream(torch.cuda.current_stream(dev))
+        with torch.cuda.stream(side):
+            # a long fill ahead of the decode, so that a run that did not wait would read the old list
+            torch.empty(256 << 20, dtype=torch.uint8, device=dev).fill_(1)
+            w.decode(*sym)
+        assert w._planned.decoded[2] == []
+        for rep in range(3):
+            o = out0.clone().to(dev)
+            w.run(qd, kd, vd, *sym, out=o, reuse_decoded=True)
+            assert w._planned.decoded[2] == [torch.cuda.current_stream(dev)]
+            touched = (exp.view(torch.int16) != out0.view(torch.int16)).any(-1)
+            got = o.cpu()
+            assert torch.equal(got[~touched].view(torch.int16), out0[~touched].view(torch.int16))
+            assert max_abs(got[touched], exp[touched]) <= 2e-2
+
+
 def test_plan_helpers_at_config0(dev):
     """plan() leaves the reference's bit-count indptrs (flashomni/attention.py:625-642)."""
     import flashomni_amd as fo
