@@ -30,7 +30,7 @@ SIGNATURES = {
     "fo_sparse_fa_split_workspace_bytes": ([], c_i64),
     "fo_sparse_fa_set_variant": ([c_int], c_int),
     "fo_sparse_fa_run": ([c_vp] * 5 + [c_int, c_vp, c_vp, c_vp, c_vp] + [c_i64] * 8 + [c_vp] * 4 + [c_i32, c_i32]
-                         + [c_vp] * 7 + [c_i64, c_i32, c_i32, c_i32, c_i32, c_i32, c_i32, c_f32, c_vp, c_vp, c_i64, c_vp],
+                         + [c_vp] * 7 + [c_i64, c_i32, c_i32, c_i32, c_i32, c_i32, c_i32, c_f32, c_f32, c_vp, c_vp, c_i64, c_vp],
                          c_int),
     "fo_gemm_workspace_bytes": ([c_i32, c_i32, c_i32], c_i64),
     "fo_gemm_q": ([c_vp] * 4 + [c_int] + [c_i32] * 6 + [c_vp, c_vp, c_i32, c_int, c_vp, c_i64, c_vp],

@@ -11,8 +11,8 @@ The public surface (constructor, ``plan``, ``run``, ``run_return_lse``, the depr
   torch does not see; ``reuse_decoded=True`` skips it on the caller's word) and then launches the
   sparse FlashAttention kernel over that list (fo_sparse_fa_run).
 
-Only what the reference's shipped build supports is implemented: no causal / custom mask, no
-positional encoding, no logits soft cap, fp32 logits (reference: setup.py:98-111).
+Of the options the reference's shipped build supports (setup.py:30-38, :98-111) head_dim 128 and the
+logits soft cap are implemented: no causal / custom mask, no positional encoding, fp32 logits.
 """
 import functools
 import math
@@ -224,8 +224,10 @@ class PlannedBatch:
         return self.worklist
 
     def launch(self, q, k, v, out, lse, kv_layout, sm_scale, q_scale=None, k_scale=None, q_lo=None,
-               k_lo=None) -> None:
+               k_lo=None, logits_soft_cap=0.0) -> None:
         """Shape checks against the planned batch, then fo_sparse_fa_run over the decoded list."""
+        if logits_soft_cap and logits_soft_cap > 0 and is_float8(q):
+            raise NotImplementedError("the logits soft cap takes 16-bit q and k")
         if q.dim() != 3 or k.dim() != 3 or v.dim() != 3 or k.size(2) != 128 or v.size(2) != 128:
             raise ValueError("q, k and v must be 3-dimensional with head_dim 128")
         fp8 = is_float8(q)
@@ -290,6 +292,7 @@ class PlannedBatch:
                 _lib.ptr(wl.row_qb), _lib.ptr(wl.row_head), _lib.ptr(wl.kv_row_ptr), _lib.ptr(wl.kv_idx),
                 _lib.ptr(wl.order), _lib.ptr(wl.sched), self.max_rows, q.size(1), self.num_kv_heads,
                 int(self.gqa_packed), q.size(2), self.block_q, self.block_kv, float(sm_scale),
+                float(logits_soft_cap or 0.0),
                 _lib.ptr(wl.shares if self.split_ok else None),
                 _lib.ptr(self.float_ws) if self.split_ok else None,
                 self.float_ws_bytes(), _lib.current_stream(self.device)))
@@ -431,11 +434,11 @@ class BatchFlashOmniFAWithRaggedKVWrapper:
             raise NotImplementedError(
                 "causal / custom masks are not part of the sparse prefill path (the reference build "
                 "only instantiates the non-causal kernel)")
-        if PosEncodingMode[pos_encoding_mode] != PosEncodingMode.NONE or logits_soft_cap > 0 \
-                or use_fp16_qk_reduction:
+        if PosEncodingMode[pos_encoding_mode] != PosEncodingMode.NONE or use_fp16_qk_reduction:
             raise NotImplementedError(
-                "positional encoding, logits soft cap and fp16 logits are not part of the sparse "
-                "prefill path")
+                "positional encoding and fp16 logits are not part of the sparse prefill path")
+        if not (0.0 <= logits_soft_cap < float("inf")):
+            raise ValueError("logits_soft_cap must be a finite value >= 0")
         if num_kv_heads <= 0 or num_qo_heads % num_kv_heads != 0:
             raise ValueError("num_qo_heads must be a multiple of num_kv_heads")
         if gqa_symbols not in (None, "packed_tile", "per_q_head"):
@@ -607,7 +610,7 @@ class BatchFlashOmniFAWithRaggedKVWrapper:
         else:
             pb.decode(sparse_info, sparse_kv_info, sparse_info_indptr, sparse_kv_info_indptr, is_full)
         pb.launch(q, k, v, out, lse if return_lse else None, self._kv_layout, sm_scale, q_scale, k_scale, q_lo,
-                  k_lo)
+                  k_lo, logits_soft_cap=self._logits_soft_cap or 0.0)
         return (out, lse) if return_lse else out
 
     run_return_lse = functools.partialmethod(run, return_lse=True)
@@ -635,9 +638,11 @@ class BatchFlashOmniFAWithRaggedKVWrapper:
 
     def _set_forward_options(self, causal, pos_encoding_mode, use_fp16_qk_reduction,
                              logits_soft_cap, sm_scale, rope_scale, rope_theta):
-        if causal or pos_encoding_mode != "NONE" or use_fp16_qk_reduction or (logits_soft_cap or 0) > 0:
-            raise NotImplementedError("only non-causal attention without positional encoding or "
-                                      "soft cap is supported")
+        if causal or pos_encoding_mode != "NONE" or use_fp16_qk_reduction:
+            raise NotImplementedError("only non-causal attention without positional encoding is supported")
+        if not (0.0 <= (logits_soft_cap or 0.0) < float("inf")):
+            raise ValueError("logits_soft_cap must be a finite value >= 0")
+        self._logits_soft_cap = logits_soft_cap or 0.0
         self._sm_scale = sm_scale
         self._rope_scale = rope_scale
         self._rope_theta = rope_theta

@@ -143,6 +143,10 @@ struct FaParams {
   int32_t gqa_pack;
   int32_t n_q_blocks, n_kv_blocks;  // row lengths of q_scale / k_scale
   float sm_scale_log2;
+  // logits soft cap (reference: DefaultAttention, variants.cuh:43-56, :68-70): scores become
+  // cap * tanh(q.k * sm_scale / cap).  cap_log2 = cap * log2(e), and sm_scale_log2 then holds
+  // 2 * log2(e) * sm_scale / cap, so that exp2 of the scaled product is exp(2x) of tanh's argument.
+  float cap_log2;
 };
 
 template <typename T>
@@ -283,13 +287,15 @@ __device__ __forceinline__ int pop_row(const FaParams& p, int xcd, const int* q,
 // workgroups share a CU (one wavefront of each per SIMD) and run independent rows: nothing ties
 // their phases together, there is no merge, and one's row prologue / epilogue overlaps the other's
 // main loop.  A row takes twice as long, so this is the form for long lists (many rows per CU).
-template <typename T, bool kFp8, bool kQLo, bool kKLo, int kGroups, bool kPipe = false, bool kGqaPack = false>
+template <typename T, bool kFp8, bool kQLo, bool kKLo, int kGroups, bool kPipe = false, bool kGqaPack = false,
+          bool kCap = false>
 __global__ void __launch_bounds__(kGroups * kGroupThreads) __attribute__((amdgpu_waves_per_eu(2, 2)))
 sparse_fa_kernel(const FaParams p) {
   static_assert(kPipe == (kGroups == 1), "one kv group runs the software-pipelined loop, two the two-phase loop");
   static_assert(!kPipe || !kFp8, "the software-pipelined loop is built for 16-bit operands");
   static_assert(kFp8 || !kQLo, "the two-term q is an fp8 form");
   static_assert(kQLo || !kKLo, "the two-term k is built on the two-term q");
+  static_assert(!kCap || (!kFp8 && !kPipe), "the logits soft cap is built into the two-phase loop for 16-bit operands");
   constexpr int kWaves = 4 * kGroups;
   constexpr int kFetchWave = kGroups == 2 ? 4 : 0;  // the wavefront that fetches the next item
   using TT = Types<T>;
@@ -1225,6 +1231,16 @@ sparse_fa_kernel(const FaParams p) {
 #pragma unroll
           for (int i = 0; i < 16; ++i) s[mt][i] = __builtin_fmaf(s[mt][i], cs, -m_run);
       }
+      if constexpr (kCap) {
+        // s holds 2 x log2(e) of tanh's argument x (the accumulators start at zero here):
+        // tanh(x) = 1 - 2 / (1 + exp(2x)); score = cap_log2 * tanh(x), taken relative to m_run
+        const float a = -2.f * p.cap_log2, b = p.cap_log2 - m_run;
+#pragma unroll
+        for (int mt = 0; mt < 2; ++mt)
+#pragma unroll
+          for (int i = 0; i < 16; ++i)
+            s[mt][i] = __builtin_fmaf(__builtin_amdgcn_rcpf(1.f + __builtin_amdgcn_exp2f(s[mt][i])), a, b);
+      }
       if (valid < kTileKV) {
 #pragma unroll
         for (int mt = 0; mt < 2; ++mt)
@@ -1255,8 +1271,10 @@ sparse_fa_kernel(const FaParams p) {
         for (int mt = 0; mt < 2; ++mt)
 #pragma unroll
           for (int i = 0; i < 16; ++i) s[mt][i] -= delta;
+        if constexpr (!kCap) {
 #pragma unroll
-        for (int i = 0; i < 16; ++i) c_init[i] = -m_run;
+          for (int i = 0; i < 16; ++i) c_init[i] = -m_run;
+        }
       }
 #pragma unroll
       for (int mt = 0; mt < 2; ++mt)
@@ -1596,7 +1614,8 @@ sparse_fa_kernel(const FaParams p) {
   }
 }
 
-template <typename T, bool kFp8, bool kQLo, bool kKLo, int kGroups = 2, bool kPipe = false, bool kGqaPack = false>
+template <typename T, bool kFp8, bool kQLo, bool kKLo, int kGroups = 2, bool kPipe = false, bool kGqaPack = false,
+          bool kCap = false>
 int launch(const FaParams& p, int64_t max_rows, hipStream_t stream) {
   constexpr int kSmemBytes = Geom<kFp8, kKLo, kGroups>::kSmemBytes;
   // (the attribute belongs to the kernel's code object on one device: set once per device; the flags
@@ -1605,7 +1624,7 @@ int launch(const FaParams& p, int64_t max_rows, hipStream_t stream) {
   int dev = 0;
   FO_HIP_CALL(hipGetDevice(&dev));
   if (dev < 0 || dev >= 64 || !attr_set[dev].load(std::memory_order_acquire)) {
-    FO_HIP_CALL(hipFuncSetAttribute(reinterpret_cast<const void*>(&sparse_fa_kernel<T, kFp8, kQLo, kKLo, kGroups, kPipe, kGqaPack>),
+    FO_HIP_CALL(hipFuncSetAttribute(reinterpret_cast<const void*>(&sparse_fa_kernel<T, kFp8, kQLo, kKLo, kGroups, kPipe, kGqaPack, kCap>),
                                     hipFuncAttributeMaxDynamicSharedMemorySize, kSmemBytes));
     if (dev >= 0 && dev < 64) attr_set[dev].store(true, std::memory_order_release);
   }
@@ -1614,7 +1633,7 @@ int launch(const FaParams& p, int64_t max_rows, hipStream_t stream) {
   int64_t grid = num_cu * (3 - kGroups);  // persistent workgroups: one per CU, or two of one kv group each (LDS bound)
   // (with even shares every workgroup may hold a part of a row; otherwise at most one row each)
   if (!(p.split_ws && p.shares) && grid > max_rows) grid = max_rows;
-  sparse_fa_kernel<T, kFp8, kQLo, kKLo, kGroups, kPipe, kGqaPack><<<static_cast<unsigned>(grid), kGroups * kGroupThreads, kSmemBytes, stream>>>(p);
+  sparse_fa_kernel<T, kFp8, kQLo, kKLo, kGroups, kPipe, kGqaPack, kCap><<<static_cast<unsigned>(grid), kGroups * kGroupThreads, kSmemBytes, stream>>>(p);
   FO_CHECK_LAUNCH();
   return FO_OK;
 }
@@ -1649,8 +1668,9 @@ extern "C" int fo_sparse_fa_run(const void* q, const void* k, const void* v, voi
                                 const int32_t* kv_row_ptr, const int32_t* kv_idx,
                                 const int32_t* order, int32_t* sched, int64_t max_rows,
                                 int32_t num_heads, int32_t num_kv_heads, int32_t gqa_packed, int32_t head_dim,
-                                int32_t block_q, int32_t block_kv, float sm_scale, const int32_t* shares,
-                                void* split_workspace, int64_t split_workspace_bytes, void* stream) {
+                                int32_t block_q, int32_t block_kv, float sm_scale, float logits_soft_cap,
+                                const int32_t* shares, void* split_workspace, int64_t split_workspace_bytes,
+                                void* stream) {
   FO_REQUIRE(head_dim == kHeadDim, "sparse_fa: head_dim %d is not supported (only 128)", head_dim);
   FO_REQUIRE(block_q == kBlockQ && block_kv == kBlockKV,
              "sparse_fa: sparse block sizes (%d, %d) are not supported (only 128, 128)", block_q,
@@ -1661,6 +1681,9 @@ extern "C" int fo_sparse_fa_run(const void* q, const void* k, const void* v, voi
   FO_REQUIRE(num_kv_heads > 0 && num_heads % num_kv_heads == 0,
              "sparse_fa: num_qo_heads %d is not a multiple of num_kv_heads %d", num_heads, num_kv_heads);
   FO_REQUIRE(gqa_packed == 0 || gqa_packed == 1, "sparse_fa: gqa_packed must be 0 or 1");
+  FO_REQUIRE(logits_soft_cap >= 0.f && logits_soft_cap < __builtin_inff(),
+             "sparse_fa: logits_soft_cap must be a finite value >= 0 (0: no cap)");
+  FO_REQUIRE(logits_soft_cap == 0.f || dtype != FO_FP8_E4M3, "sparse_fa: the logits soft cap is not built for fp8 q/k");
   FO_REQUIRE(!gqa_packed || dtype != FO_FP8_E4M3,
              "sparse_fa: fp8 q (one scale per q head and token block) is not built for packed tiles of "
              "several q heads");
@@ -1713,7 +1736,18 @@ extern "C" int fo_sparse_fa_run(const void* q, const void* k, const void* v, voi
   p.kv_group = packed ? 1 : num_heads / num_kv_heads;
   p.gqa_pack = packed ? num_heads / num_kv_heads : 0; p.n_q_blocks = n_q_blocks; p.n_kv_blocks = n_kv_blocks;
   p.sm_scale_log2 = sm_scale * 1.44269504088896340736f;
+  p.cap_log2 = 0.f;
   hipStream_t s = static_cast<hipStream_t>(stream);
+  if (logits_soft_cap > 0.f) {
+    // (reference: soft_cap_pre_tanh_scale = sm_scale / cap, sm_scale_log2 = log2(e) * cap, variants.cuh:43-56)
+    p.cap_log2 = logits_soft_cap * 1.44269504088896340736f;
+    p.sm_scale_log2 = 2.f * 1.44269504088896340736f * sm_scale / logits_soft_cap;
+    if (p.gqa_pack)
+      return dtype == FO_BF16 ? launch<__bf16, false, false, false, 2, false, true, true>(p, max_rows, s)
+                              : launch<_Float16, false, false, false, 2, false, true, true>(p, max_rows, s);
+    return dtype == FO_BF16 ? launch<__bf16, false, false, false, 2, false, false, true>(p, max_rows, s)
+                            : launch<_Float16, false, false, false, 2, false, false, true>(p, max_rows, s);
+  }
   // Long lists (many rows per CU) run as two independent 4-wavefront workgroups per CU with the
   // software-pipelined loop; short ones as one 8-wavefront workgroup whose two kv groups share a row
   // (half the latency per row, and rows can be cut into even shares).  The list's length lives on the

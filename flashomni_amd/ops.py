@@ -103,8 +103,8 @@ def batch_sparseFA_with_ragged_kv_run(float_workspace_buffer, int_workspace_buff
            "batch_sparseFA_with_ragged_kv_run: q does not have the planned number of heads")
     _check(mask_mode_code == 0 and maybe_custom_mask is None and maybe_mask_indptr is None,
            "only the non-causal mask mode is built (as in the reference's shipped kernels)")
-    _check(maybe_alibi_slopes is None and logits_soft_cap <= 0.0,
-           "ALiBi and logits soft cap are not built (as in the reference's shipped kernels)")
+    _check(maybe_alibi_slopes is None, "ALiBi is not built (as in the reference's shipped kernels)")
+    _check(0.0 <= logits_soft_cap < float("inf"), "logits_soft_cap must be a finite value >= 0")
     _check(sparse_block_size_for_q == 128 and sparse_block_size_for_kv == 128,
            "only 128 x 128 sparse blocks are supported")
     _check(layout in (0, 1), "layout must be 0 (NHD) or 1 (HND)")
@@ -125,7 +125,8 @@ def batch_sparseFA_with_ragged_kv_run(float_workspace_buffer, int_workspace_buff
     pb.qo_indptr, pb.kv_indptr = qo_indptr, kv_indptr
     try:
         pb.decode(sparse_info, sparse_kv_info, sparse_info_indptr, sparse_kv_info_indptr, is_full)
-        pb.launch(q, k, v, o, maybe_lse, "NHD" if layout == 0 else "HND", sm_scale)
+        pb.launch(q, k, v, o, maybe_lse, "NHD" if layout == 0 else "HND", sm_scale,
+                  logits_soft_cap=logits_soft_cap)
     except ValueError as e:
         raise RuntimeError(str(e)) from None
 

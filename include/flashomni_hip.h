@@ -19,7 +19,7 @@
 extern "C" {
 #endif
 
-#define FO_ABI_VERSION 4
+#define FO_ABI_VERSION 5
 
 enum {
   FO_OK = 0,
@@ -185,6 +185,11 @@ int fo_decode_sparse_static(const uint8_t* sparse_info, const uint8_t* sparse_kv
  * Rows of the list write every output row of their q-block; q-blocks not in the list are left
  * untouched; a listed row with no kv block writes zeros and lse = -5e4.  lse (optional, fp32
  * [nnz_q,H]) is base 2: log2(sum 2^(s*c - m*c)) + m*c, c = sm_scale*log2(e).
+ * logits_soft_cap > 0 (16-bit q/k only; 0 = off): the scores become cap * tanh(q.k * sm_scale / cap)
+ * before the softmax, and lse is taken over those (reference: DefaultAttention with
+ * use_logits_soft_cap, include/flashomni/attention/variants.cuh:43-56, :68-70; tanh is formed as
+ * 1 - 2 / (1 + exp(2x)) where the reference uses tanh.approx).  Runs in the 8-wavefront form whatever
+ * the list's length.
  * Rows are taken from the queues described by `order` / `sched` (see fo_decode_sparse); the
  * kernel leaves the queue cursors rewound, so one decoded list can be run any number of times,
  * but two launches sharing one `sched` must not overlap in time.
@@ -216,8 +221,8 @@ int fo_sparse_fa_run(const void* q, const void* k, const void* v, void* o, float
                      int32_t n_kv_blocks, const int32_t* row_req, const int32_t* row_qb, const int32_t* row_head,
                      const int32_t* kv_row_ptr, const int32_t* kv_idx, const int32_t* order,
                      int32_t* sched, int64_t max_rows, int32_t num_heads, int32_t num_kv_heads, int32_t gqa_packed,
-                     int32_t head_dim, int32_t block_q, int32_t block_kv, float sm_scale, const int32_t* shares,
-                     void* split_workspace, int64_t split_workspace_bytes, void* stream);
+                     int32_t head_dim, int32_t block_q, int32_t block_kv, float sm_scale, float logits_soft_cap,
+                     const int32_t* shares, void* split_workspace, int64_t split_workspace_bytes, void* stream);
 
 /* ---------------------------------------------------------------------------------------------
  * GEMM-Q: y[b, tile] = x[b] . w^T + bias for every (128-row, 128-column) tile whose symbol bit

@@ -7,7 +7,9 @@ Semantics follow include/flashomni/attention/prefill.cuh:
   * an active row with no kept block writes zeros and lse = -5e4
     (finite "infinity" of include/flashomni/math.cuh:32; :385-386, :944-946, :1517-1520);
   * lse is base-2: log2(sum exp2(s*c - m*c)) + m*c with c = sm_scale*log2(e)
-    (:973, :1517; include/flashomni/attention/variants.cuh:54).
+    (:973, :1517; include/flashomni/attention/variants.cuh:54);
+  * logits_soft_cap > 0: the logits become tanh(q.k * sm_scale / cap) and the softmax scale
+    log2(e) * cap (variants.cuh:43-56 set-up, :68-70 transform), i.e. scores cap * tanh(q.k * sm_scale / cap).
 The block mask is expanded to token granularity exactly like the reference benchmark builds
 its SDPA mask (benchmark/test_flashomni_attention.py:197-199): repeat_interleave(block) and crop.
 
@@ -32,7 +34,8 @@ NEG_INF = -5e4
 def sparse_attention(q, k, v, sparse_info, sparse_kv_info, sparse_info_indptr,
                      sparse_kv_info_indptr, qo_indptr, kv_indptr, block_q=128, block_kv=128,
                      sm_scale=None, is_full=False, out=None, lse=None, rows=None,
-                     q_scale=None, k_scale=None, q_lo=None, k_lo=None, gqa_symbols="per_q_head"):
+                     q_scale=None, k_scale=None, q_lo=None, k_lo=None, gqa_symbols="per_q_head",
+                     logits_soft_cap=0.0):
     """q [nnz_q,H,D], k/v [nnz_kv,H,D] (any float dtype; math is fp32 on the given values).
 
     `out` (same dtype as q unless q is fp8, then bf16) is updated in place for active rows only; allocated
@@ -55,7 +58,7 @@ def sparse_attention(q, k, v, sparse_info, sparse_kv_info, sparse_info_indptr,
         assert q_scale is None and k_scale is None, "packed tiles take 16-bit q and k"
         return _packed_tiles(q, k, v, to_np(sparse_info), to_np(sparse_kv_info), to_np(sparse_info_indptr),
                              to_np(sparse_kv_info_indptr), qo, kvp, group, block_q, block_kv,
-                             sm_scale, is_full, out, lse, rows)
+                             sm_scale, is_full, out, lse, rows, logits_soft_cap)
     row_req, row_qb, row_head, ptr, idx = decode_kv_csr(
         to_np(sparse_info), to_np(sparse_kv_info), to_np(sparse_info_indptr),
         to_np(sparse_kv_info_indptr), qo, kvp, H, block_q, block_kv, is_full)
@@ -90,18 +93,28 @@ def sparse_attention(q, k, v, sparse_info, sparse_kv_info, sparse_info_indptr,
         if k_scale is not None:
             blk = torch.from_numpy((tok - kv0) // block_kv + int(kv_blk_base[r]))
             kf = kf * k_scale[h // group][blk].float()[:, None]
-        s = qf @ kf.T
-        m = s.max(dim=-1, keepdim=True).values
-        p = torch.exp2((s - m) * c)
-        d = p.sum(dim=-1, keepdim=True)
-        out[q0:q1, h] = ((p @ vf) / d).to(out.dtype)
+        o_rows, lse_rows = _softmax_pv(qf @ kf.T, vf, sm_scale, logits_soft_cap)
+        out[q0:q1, h] = o_rows.to(out.dtype)
         if lse is not None:
-            lse[q0:q1, h] = (torch.log2(d) + m * c).squeeze(-1)
+            lse[q0:q1, h] = lse_rows
     return out
 
 
+def _softmax_pv(s, vf, sm_scale, logits_soft_cap):
+    """Rows of raw logits s = q.k^T -> (softmax(s) @ v, base-2 lse), fp32."""
+    c = sm_scale * math.log2(math.e)
+    if logits_soft_cap > 0:
+        # variants.cuh:47-48: soft_cap_pre_tanh_scale = sm_scale / cap, sm_scale_log2 = log2(e) * cap
+        s = torch.tanh(s * (sm_scale / logits_soft_cap))
+        c = math.log2(math.e) * logits_soft_cap
+    m = s.max(dim=-1, keepdim=True).values
+    p = torch.exp2((s - m) * c)
+    d = p.sum(dim=-1, keepdim=True)
+    return (p @ vf) / d, (torch.log2(d) + m * c).squeeze(-1)
+
+
 def _packed_tiles(q, k, v, sparse_info, sparse_kv_info, sparse_info_indptr, sparse_kv_info_indptr, qo, kvp,
-                  group, block_q, block_kv, sm_scale, is_full, out, lse, rows):
+                  group, block_q, block_kv, sm_scale, is_full, out, lse, rows, logits_soft_cap=0.0):
     """The reference's grouped-query layout (see the module text).  The symbols of a request with
     qo_len tokens are those of an ungrouped request with qo_len * group rows and H_kv heads
     (prefill.cuh:1283-1290 with gridDim.z = H_kv), so the same decoder lists the (tile, kv head) rows."""
@@ -130,11 +143,8 @@ def _packed_tiles(q, k, v, sparse_info, sparse_kv_info, sparse_info_indptr, spar
         qf = q[tok, hq].float()
         kf = k[kt, kvh].float()
         vf = v[kt, kvh].float()
-        s = qf @ kf.T
-        m = s.max(dim=-1, keepdim=True).values
-        p = torch.exp2((s - m) * c)
-        d = p.sum(dim=-1, keepdim=True)
-        out[tok, hq] = ((p @ vf) / d).to(out.dtype)
+        o_rows, lse_rows = _softmax_pv(qf @ kf.T, vf, sm_scale, logits_soft_cap)
+        out[tok, hq] = o_rows.to(out.dtype)
         if lse is not None:
-            lse[tok, hq] = (torch.log2(d) + m * c).squeeze(-1)
+            lse[tok, hq] = lse_rows
     return out

@@ -659,3 +659,65 @@ def test_share_with_many_short_rows(dev):
     out = out.cpu()
     assert float(out[128:].abs().max()) == 0.0 and float(exp[128:].abs().max()) == 0.0
     assert max_abs(out[:128], exp[:128]) <= MAX_ABS and rel_l2(out[:128], exp[:128]) <= REL_L2
+
+
+@pytest.mark.parametrize("cap", [1.0, 30.0])
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+def test_logits_soft_cap(dev, cap, dtype):
+    """plan(..., logits_soft_cap=cap) (reference: flashomni/attention.py:421-429 -> variants.cuh:43-56,
+    :68-70): scores cap * tanh(q.k * sm_scale / cap), on a ragged batch with tails, q scaled so that the
+    raw logits reach several times the smaller cap; output within the path's tolerances of the oracle,
+    lse (base 2, over the capped scores) within 2e-2, skipped q blocks untouched.  The kernel form with
+    the cap is the 8-wavefront one whatever the list's length, so both settings of the fixture run it."""
+    import flashomni_amd as fo
+    heads = 3
+    ql, kl = [300, 1, 640], [77, 513, 700]
+    m = make_ragged_masks(ql, kl, heads, 0.8, 0.6, seed=21)
+    g = torch.Generator().manual_seed(21)
+    nq, nk = sum(ql), sum(kl)
+    q = (torch.randn(nq, heads, 128, generator=g) * 2).to(dtype)
+    k = torch.randn(nk, heads, 128, generator=g).to(dtype)
+    v = torch.randn(nk, heads, 128, generator=g).to(dtype)
+    out0 = sentinel_like((nq, heads, 128), dtype)
+    t = lambda a: torch.from_numpy(a).to(dev)
+    w = fo.BatchFlashOmniFAWithRaggedKVWrapper(torch.empty(128 << 20, dtype=torch.uint8, device=dev))
+    w.plan(t(m["qo_indptr"]), t(m["kv_indptr"]), heads, heads, 128, q_data_type=dtype, logits_soft_cap=cap)
+    out = out0.clone().to(dev)
+    _, lse = w.run(q.to(dev), k.to(dev), v.to(dev), t(m["packed_info"]), t(m["packed_keep"]), t(m["info_indptr"]),
+                   t(m["keep_indptr"]), out=out, return_lse=True)
+    exp_lse = torch.full((nq, heads), float("nan"))
+    sym = (m["packed_info"], m["packed_keep"], m["info_indptr"], m["keep_indptr"], m["qo_indptr"], m["kv_indptr"])
+    exp = oracle.sparse_attention(q, k, v, *sym, out=out0.clone(), lse=exp_lse, logits_soft_cap=cap)
+    _check(out.cpu(), exp, out0, m, heads)
+    ok = ~torch.isnan(exp_lse) & (exp_lse > -4e4)
+    assert ok.any() and float((lse.cpu()[ok] - exp_lse[ok]).abs().max()) < 2e-2
+    if cap == 1.0:   # the cap changes the result by far more than the tolerance: it was applied
+        plain = oracle.sparse_attention(q, k, v, *sym, out=out0.clone())
+        touched = _touched(m, heads, exp.shape)
+        assert max_abs(plain[touched], exp[touched]) > 10 * MAX_ABS
+
+
+def test_logits_soft_cap_packed_gqa_and_forward_options(dev):
+    """The cap with the reference's grouped-query tiles (its own kernel instantiation), and set through
+    the deprecated forward() (flashomni/attention.py:837-869), which stores it for later run() calls."""
+    import flashomni_amd as fo
+    H, Hkv, n = 4, 2, 384
+    m = make_ragged_masks([n * (H // Hkv)], [n], Hkv, 0.8, 0.6, seed=23)   # symbols over packed rows x kv heads
+    g = torch.Generator().manual_seed(23)
+    q = (torch.randn(n, H, 128, generator=g) * 2).to(torch.bfloat16)
+    k = torch.randn(n, Hkv, 128, generator=g).to(torch.bfloat16)
+    v = torch.randn(n, Hkv, 128, generator=g).to(torch.bfloat16)
+    t = lambda a: torch.from_numpy(a).to(dev)
+    ip = torch.tensor([0, n], dtype=torch.int32, device=dev)
+    w = fo.BatchFlashOmniFAWithRaggedKVWrapper(torch.empty(128 << 20, dtype=torch.uint8, device=dev))
+    w.plan(ip, ip, H, Hkv, 128, q_data_type=torch.bfloat16)
+    sym = (t(m["packed_info"]), t(m["packed_keep"]), t(m["info_indptr"]), t(m["keep_indptr"]))
+    out0 = sentinel_like((n, H, 128), torch.bfloat16)
+    exp = oracle.sparse_attention(q, k, v, m["packed_info"], m["packed_keep"], m["info_indptr"], m["keep_indptr"],
+                                  [0, n], [0, n], out=out0.clone(), gqa_symbols="packed_tile", logits_soft_cap=2.0)
+    got = w.forward(q.to(dev), k.to(dev), v.to(dev), *sym, logits_soft_cap=2.0)
+    touched = (exp.view(torch.int16) != out0.view(torch.int16)).any(-1)
+    assert touched.any()
+    assert max_abs(got.cpu()[touched], exp[touched]) <= MAX_ABS and rel_l2(got.cpu()[touched], exp[touched]) <= REL_L2
+    again = w.run(q.to(dev), k.to(dev), v.to(dev), *sym)    # the stored cap still applies
+    assert torch.equal(again, got)

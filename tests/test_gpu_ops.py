@@ -205,6 +205,39 @@ def test_symbols_rewritten_in_place_are_decoded_again(dev):
     assert max_abs(o_reuse.cpu()[touched], exp_b[touched]) <= 2e-2
 
 
+def test_attention_ops_logits_soft_cap(dev):
+    """The run operator's logits_soft_cap argument (csrc/batch_sparseFA.cu:67-201 passes it to the
+    variant, variants.cuh:43-56): equal to the wrapper planned with the same cap, and within the path's
+    tolerances of the oracle."""
+    import flashomni_amd as fo
+    heads = 2
+    m = make_ragged_masks([384, 130], [500, 256], heads, 0.8, 0.6, seed=33)
+    g = torch.Generator().manual_seed(33)
+    nq, nk = 514, 756
+    q = (torch.randn(nq, heads, 128, generator=g) * 2).to(torch.bfloat16)
+    k, v = (torch.randn(nk, heads, 128, generator=g).to(torch.bfloat16) for _ in range(2))
+    state = _plan(dev, m, heads)
+    float_ws, int_ws, plan_info, qo_d, kv_d = state
+    t = lambda a: torch.from_numpy(a).to(dev)
+    sym = (t(m["packed_info"]), t(m["packed_keep"]), t(m["info_indptr"]), t(m["keep_indptr"]))
+    out0 = sentinel_like((nq, heads, 128), torch.bfloat16)
+    o = out0.clone().to(dev)
+    _ops().batch_sparseFA_with_ragged_kv_run.default(
+        float_ws, int_ws, plan_info, q.to(dev), k.to(dev), v.to(dev), *sym, 128, 128, False,
+        qo_d, kv_d, o, None, 0, 0, None, None, None, 3.0, 128 ** -0.5, 1.0, 1.0 / 1e4)
+    exp = oracle.sparse_attention(q, k, v, m["packed_info"], m["packed_keep"], m["info_indptr"], m["keep_indptr"],
+                                  m["qo_indptr"], m["kv_indptr"], out=out0.clone(), logits_soft_cap=3.0)
+    touched = (exp.view(torch.int16) != out0.view(torch.int16)).any(-1)
+    got = o.cpu()
+    assert torch.equal(got[~touched].view(torch.int16), out0[~touched].view(torch.int16))
+    assert max_abs(got[touched], exp[touched]) <= 2e-2 and rel_l2(got[touched], exp[touched]) <= 1e-2
+    w = fo.BatchFlashOmniFAWithRaggedKVWrapper(torch.empty(128 << 20, dtype=torch.uint8, device=dev))
+    w.plan(t(m["qo_indptr"]), t(m["kv_indptr"]), heads, heads, 128, q_data_type=torch.bfloat16, logits_soft_cap=3.0)
+    o_w = out0.clone().to(dev)
+    w.run(q.to(dev), k.to(dev), v.to(dev), *sym, out=o_w)
+    assert torch.equal(o_w.cpu().view(torch.int16), got.view(torch.int16))
+
+
 def test_reuse_decoded_from_another_stream_waits_once_per_decode(dev):
     """A list decoded on a side stream and run from the current one: the first run waits for the
     decode, later ones on the same stream are behind it already (no further event), and a new decode

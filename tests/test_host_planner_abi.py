@@ -29,7 +29,7 @@ def test_library_exports_every_declared_symbol():
     for name in declared:
         assert hasattr(handle, name), name
     assert declared == set(L.SIGNATURES), declared ^ set(L.SIGNATURES)
-    assert L.lib().fo_abi_version() == 4
+    assert L.lib().fo_abi_version() == 5
 
 
 _C_SCALARS = {"int": ctypes.c_int, "int32_t": ctypes.c_int32, "uint32_t": ctypes.c_uint32,
@@ -168,8 +168,15 @@ def test_argument_checks_without_gpu():
     assert L.fo_gemm_q(1, 1, None, 1, 0, 1, 128, 100, 64, 128, 1, None, None, 0, 1, None, 0, None) == -1
     assert b"only support" in L.fo_last_error()
     assert L.fo_sparse_fa_run(*([None] * 5), 0, None, None, None, None, *([0] * 8), *([None] * 4), 0, 0, *([None] * 7), 4, 2, 2, 0, 64, 128, 128,
-                              1.0, None, None, 0, None) == -1
+                              1.0, 0.0, None, None, 0, None) == -1
     assert b"head_dim" in L.fo_last_error()
+    # the logits soft cap: finite, >= 0, 16-bit q/k only
+    tail = (None, None, 0, None)
+    head = (*([None] * 5),)
+    mid = (None, None, None, None, *([0] * 8), *([None] * 4), 0, 0, *([None] * 7), 4, 2, 2, 0, 128, 128, 128, 1.0)
+    assert L.fo_sparse_fa_run(*head, 0, *mid, -1.0, *tail) == -1 and b"logits_soft_cap" in L.fo_last_error()
+    assert L.fo_sparse_fa_run(*head, 0, *mid, float("inf"), *tail) == -1 and b"logits_soft_cap" in L.fo_last_error()
+    assert L.fo_sparse_fa_run(*head, 2, *mid, 30.0, *tail) == -1 and b"soft cap" in L.fo_last_error()
 
 
 def test_ops_fail_loudly_without_a_gpu_or_library(monkeypatch):

@@ -229,3 +229,38 @@ def test_attention_packed_tile_gqa_token_by_token(heads):
                 want = (p[:, None] * v[keys, h // group].double()).sum(0) / p.sum()
                 assert float((got.double() - want).abs().max()) < 1e-4
                 assert abs(float(lse[qo[r] + tok, h]) - float(torch.log2(p.sum()) + s.max())) < 1e-3
+
+
+def test_attention_logits_soft_cap_token_by_token():
+    """logits_soft_cap (variants.cuh:43-56, :68-70: logits -> tanh(q.k * sm_scale / cap), softmax scale
+    log2(e) * cap) against a double-precision restatement written token by token with math.tanh, on
+    logits large enough for the cap to bite; the base-2 lse with it.  Limits that a dropped factor would
+    break: a huge cap is no cap; a tiny cap is the plain mean of the kept values (all scores within
+    +-cap of each other, where a forgotten `* cap` would leave them within +-1)."""
+    heads, n = 1, 128
+    g = torch.Generator().manual_seed(9)
+    q = torch.randn(n, heads, 128, generator=g) * 3
+    k = torch.randn(2 * n, heads, 128, generator=g) * 3
+    v = torch.randn(2 * n, heads, 128, generator=g)
+    info = np.array([1], dtype=np.uint8)
+    keep = np.packbits(np.array([0, 1], dtype=np.uint8), bitorder="little")   # second kv block only
+    args = (info, keep, [0, 1], [0, 1], [0, n], [0, 2 * n])
+    sm = 1.0 / math.sqrt(128)
+    cap = 5.0
+    lse = torch.zeros(n, heads)
+    out = oracle.sparse_attention(q, k, v, *args, logits_soft_cap=cap, lse=lse)
+    raw = (q[:, 0].double() @ k[n:, 0].double().T) * sm
+    assert float(raw.abs().max()) > 2 * cap          # the cap matters on these logits
+    for i in (0, 17, 127):
+        sc = [cap * math.tanh(float(raw[i, j]) / cap) for j in range(n)]
+        mx = max(sc)
+        w = [math.exp(x - mx) for x in sc]
+        tot = sum(w)
+        ref = sum(w[j] * v[n + j, 0].double() for j in range(n)) / tot
+        assert torch.allclose(out[i, 0].double(), ref, atol=1e-5, rtol=1e-4)
+        assert abs(float(lse[i, 0]) - (math.log(tot) + mx) / math.log(2)) < 1e-4
+    plain = oracle.sparse_attention(q, k, v, *args)
+    assert not torch.allclose(out, plain, atol=1e-2)
+    assert torch.allclose(oracle.sparse_attention(q, k, v, *args, logits_soft_cap=1e6), plain, atol=1e-4, rtol=1e-3)
+    tiny = oracle.sparse_attention(q, k, v, *args, logits_soft_cap=1e-3)
+    assert torch.allclose(tiny[:, 0], v[n:, 0].mean(0).expand(n, -1), atol=5e-3)
