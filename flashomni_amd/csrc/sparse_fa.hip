@@ -1584,21 +1584,23 @@ sparse_fa_kernel(const FaParams p) {
       // the compiler would wait there for everything, the row's stores included)
       __builtin_amdgcn_s_waitcnt(0x0f70);
     }
-    if (store_row) {
-      __syncthreads();  // the row is complete in the LDS tile
+    if (store_row && kg == 0) {
+      // A wavefront stores the 32 rows it has just written to the LDS tile itself: no barrier, so
+      // the other kv group (whose first wavefront is fetching the next row's record meanwhile) is not
+      // waited for here but at the top of the next row.
+      __builtin_amdgcn_s_waitcnt(0xc07f);  // lgkmcnt(0): this wavefront's rows are in the tile
       T* dst = op + static_cast<int64_t>(q_begin) * p.o_sn + static_cast<int64_t>(head_q0) * p.o_sh;
       // (the lane index is worked out afresh here: otherwise the per-lane address terms are computed once
       // per kernel, spilled, and every reload waits for the store before it)
       const int ln = fresh_lane();
-      constexpr int kRowsPerWave = kBlockQ / kWaves;
-      const int r0 = wv * kRowsPerWave + (ln >> 4), chunk = ln & 15;
-      u32x4 v[kRowsPerWave / 4];
+      const int r0 = qs * 32 + (ln >> 4), chunk = ln & 15;
+      u32x4 v[8];
 #pragma unroll
-      for (int i = 0; i < kRowsPerWave / 4; ++i)
+      for (int i = 0; i < 8; ++i)
         v[i] = *reinterpret_cast<const u32x4*>(smem + G::kOutOff + (r0 + i * 4) * kOutRowBytes + chunk * 16);
       T* d0 = dst + chunk * 8;
 #pragma unroll
-      for (int i = 0; i < kRowsPerWave / 4; ++i)
+      for (int i = 0; i < 8; ++i)
         if (r0 + i * 4 < q_rows) *reinterpret_cast<u32x4*>(d0 + row_off(r0 + i * 4, p.o_sn, p.o_sh)) = v[i];
     }
   }
