@@ -95,6 +95,23 @@ def test_ragged_batch_with_tails(dev, layout):
     _check(out, exp, out0, m, 3)
 
 
+def test_requests_without_queries_or_without_keys(dev):
+    """A batch holding a request with no q rows (nothing to do) and one with no keys (its active rows
+    are rows without kv blocks: zeros, lse = -5e4, as prefill.cuh:385-386, :944-946 leave them), beside
+    ordinary ones and a one-token request."""
+    ql, kl = [200, 0, 128, 1], [300, 64, 0, 5]
+    out, exp, out0, m, lse, exp_lse = _run_case(dev, ql, kl, 3, torch.bfloat16, seed=8, pa=0.8, pk=0.6,
+                                                return_lse=True)
+    _check(out, exp, out0, m, 3)
+    ok = ~torch.isnan(exp_lse)
+    assert ok.any() and float((lse[ok] - exp_lse[ok]).abs().max()) < 2e-2
+    no_keys = slice(200, 328)   # the third request's rows
+    act = torch.from_numpy(m["info"][2][0])           # its one q block, per head
+    assert act.any()
+    assert float(out[no_keys][:, act].abs().max()) == 0.0
+    assert bool((lse[no_keys][:, act] == -5e4).all())
+
+
 def test_all_ones_matches_sdpa(dev):
     """is_full and an all-ones mask both reduce to plain dense attention (a library routine)."""
     heads = 2

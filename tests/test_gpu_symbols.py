@@ -69,6 +69,7 @@ CASES = [
     ([300, 1, 128, 1000], [77, 513, 128, 4096], 3, 0.6, 0.3),   # ragged, NKV not multiple of 8
     ([129], [128 * 67 + 5], 5, 0.9, 0.02),           # long rows crossing many bytes
     ([256, 256], [256, 256], 1, 0.5, 0.5),
+    ([200, 0, 128, 1], [300, 64, 0, 5], 3, 0.8, 0.6),           # a request without q rows, one without keys
 ]
 
 
