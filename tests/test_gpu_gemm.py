@@ -441,3 +441,57 @@ def test_gemm_o_cursors_and_fixed_stride_agree(dev, shape):
     # and the end result is the dense layer
     dense = F.linear(x[0, :256].float(), w.float(), b.float()).cpu()
     assert rel_l2(got[0, :256].cpu(), dense) <= REL_L2
+
+
+@pytest.mark.parametrize("seed", range(24))
+def test_random_gemm_shapes(dev, seed):
+    """Seeded random shapes through GEMM-Q (flags or is_full) and the two passes of GEMM-O (the cached
+    partial in 16 bits or fp32): batches, M with and without a tail, head widths 32 to 256, text-token
+    offsets, K = 32 mod 64, all-zero and all-one flags.  Skipped tiles keep their bytes; results within
+    max-abs 2e-2 (per unit of output magnitude above 2, where one bf16 ulp is 1.6e-2 and more) and
+    relative L2 1e-2 of the fp32 oracle."""
+    import flashomni_amd as fo
+    rng = np.random.default_rng(1000 + seed)
+    batch = int(rng.choice([1, 1, 2, 3]))
+    m = int(rng.choice([1, 100, 128, 129, 300, 512, 1000, 2176]))
+    hd = int(rng.choice([32, 64, 96, 128, 128, 256]))
+    heads = int(rng.choice([1, 2, 3, 5, 8]))
+    if (heads * hd) % 128:
+        heads *= 128 // int(np.gcd(heads * hd, 128))
+    n = heads * hd
+    text = int(rng.choice([0, 0, 128, 512]))
+    dtype = torch.bfloat16 if rng.random() < 0.6 else torch.float16
+    p = float(rng.choice([0.0, 0.25, 0.6, 1.0]))
+    kind = ["q", "q_full", "o"][seed % 3]
+    k = n if kind == "o" else int(rng.choice([64, 96, 128, 160, 256, 512, 1056]))
+    info, packed, indptr = _flags(batch, (text + m + 127) // 128, heads, p, seed=seed)
+    x, w, b = _operands(batch, m, n, k, dtype, seed=seed)
+    pk, ip = torch.from_numpy(packed).to(dev), torch.from_numpy(indptr).to(dev)
+    bound = lambda e: MAX_ABS * max(1.0, float(e.float().abs().max()) / 2)
+    if kind != "o":
+        full = kind == "q_full"
+        out0 = sentinel_like((batch, m, n), dtype)
+        out = out0.clone().to(dev)
+        fo.flashomni_gemm(x.to(dev), w.to(dev), heads, None if full else pk, None if full else ip, text, b.to(dev),
+                          out=out, is_full=full)
+        exp = oracle.gemm_q(x, w, heads, packed, indptr, text, b, out=out0.clone(), is_full=full)
+        got = out.cpu()
+        computed = torch.zeros(batch, m, n, dtype=torch.bool)
+        for bi in range(batch):
+            for iy in range((m + 127) // 128):
+                for ix in range(n // 128):
+                    if full or info[bi, (text + iy * 128) // 128, (ix * 128) // hd]:
+                        computed[bi, iy * 128:iy * 128 + 128, ix * 128:ix * 128 + 128] = True
+        assert torch.equal(got[~computed].view(torch.int16), out0[~computed].view(torch.int16))
+        if computed.any():
+            assert max_abs(got[computed], exp[computed]) <= bound(exp[computed])
+            assert rel_l2(got[computed], exp[computed]) <= REL_L2
+    else:
+        od = torch.float32 if seed % 2 else None
+        cache = fo.flashomni_gemm_reduction(x.to(dev), w.to(dev), heads, pk, ip, text, bias=b.to(dev),
+                                            is_for_cache=True, out_dtype=od)
+        final = fo.flashomni_gemm_reduction(x.to(dev), w.to(dev), heads, pk, ip, text, bias=cache, is_for_cache=False)
+        e_cache = oracle.gemm_o(x, w, heads, packed, indptr, text, bias=b, is_for_cache=True, out_dtype=od)
+        e_final = oracle.gemm_o(x, w, heads, packed, indptr, text, bias=e_cache, is_for_cache=False)
+        for got, exp in ((cache.cpu(), e_cache), (final.cpu(), e_final)):
+            assert max_abs(got, exp) <= bound(exp) and rel_l2(got, exp) <= REL_L2
