@@ -738,3 +738,60 @@ def test_logits_soft_cap_packed_gqa_and_forward_options(dev):
     assert max_abs(got.cpu()[touched], exp[touched]) <= MAX_ABS and rel_l2(got.cpu()[touched], exp[touched]) <= REL_L2
     again = w.run(q.to(dev), k.to(dev), v.to(dev), *sym)    # the stored cap still applies
     assert torch.equal(again, got)
+
+
+@pytest.mark.parametrize("seed", range(16))
+def test_random_batches_all_options(dev, seed):
+    """Seeded random batches over everything run() takes at once: 1-4 requests (now and then one without
+    q rows or without keys), ungrouped heads or the reference's packed grouped-query tiles, both dtypes
+    and kv layouts, the logits soft cap, lse.  Skipped rows keep their bytes; the rest within the path's
+    tolerances of the oracle."""
+    import flashomni_amd as fo
+    rng = np.random.default_rng(5000 + seed)
+    B = int(rng.integers(1, 5))
+    ql = [int(rng.choice([1, 5, 127, 128, 129, 200, 384, 640, 1000])) for _ in range(B)]
+    kl = [int(rng.choice([1, 64, 65, 128, 300, 513, 1024, 2048])) for _ in range(B)]
+    if seed % 4 == 1:
+        ql[int(rng.integers(0, B))] = 0
+    if seed % 4 == 2:
+        kl[int(rng.integers(0, B))] = 0
+    if sum(ql) == 0:
+        ql[0] = 130
+    if sum(kl) == 0:
+        kl[0] = 70
+    hkv, group = int(rng.choice([1, 2, 3])), int(rng.choice([1, 1, 2, 4]))
+    H = hkv * group
+    dtype = torch.bfloat16 if seed % 2 == 0 else torch.float16
+    layout = "NHD" if seed % 3 else "HND"
+    cap = 4.0 if seed % 3 == 0 else 0.0
+    pa, pk = float(rng.choice([0.3, 0.7, 1.0])), float(rng.choice([0.0, 0.1, 0.5, 1.0]))
+    packed = group > 1
+    m = make_ragged_masks([n * group for n in ql] if packed else ql, kl, hkv if packed else H, pa, pk, seed=5000 + seed)
+    qo = np.concatenate([[0], np.cumsum(ql)]).astype(np.int32)
+    g = torch.Generator().manual_seed(5000 + seed)
+    nq, nk = sum(ql), sum(kl)
+    q = torch.randn(nq, H, 128, generator=g).to(dtype)
+    k = torch.randn(nk, hkv, 128, generator=g).to(dtype)
+    v = torch.randn(nk, hkv, 128, generator=g).to(dtype)
+    out0 = sentinel_like((nq, H, 128), dtype)
+    t = lambda a: torch.from_numpy(a).to(dev)
+    w = fo.BatchFlashOmniFAWithRaggedKVWrapper(torch.empty(256 << 20, dtype=torch.uint8, device=dev), layout)
+    w.plan(t(qo), t(m["kv_indptr"]), H, hkv, 128, q_data_type=dtype, logits_soft_cap=cap or None)
+    kd, vd = k.to(dev), v.to(dev)
+    if layout == "HND":
+        kd, vd = kd.transpose(0, 1).contiguous(), vd.transpose(0, 1).contiguous()
+    out = out0.clone().to(dev)
+    _, lse = w.run(q.to(dev), kd, vd, t(m["packed_info"]), t(m["packed_keep"]), t(m["info_indptr"]),
+                   t(m["keep_indptr"]), out=out, return_lse=True)
+    exp_lse = torch.full((nq, H), float("nan"))
+    exp = oracle.sparse_attention(q, k, v, m["packed_info"], m["packed_keep"], m["info_indptr"], m["keep_indptr"], qo,
+                                  m["kv_indptr"], out=out0.clone(), lse=exp_lse,
+                                  gqa_symbols="packed_tile" if packed else "per_q_head", logits_soft_cap=cap)
+    got = out.cpu()
+    touched = ~torch.isnan(exp_lse)                     # [token, head]: rows the oracle wrote
+    assert torch.equal(got[~touched].view(torch.int16), out0[~touched].view(torch.int16))
+    if touched.any():
+        assert max_abs(got[touched], exp[touched]) <= MAX_ABS
+        if float(exp[touched].float().norm()) > 0:
+            assert rel_l2(got[touched], exp[touched]) <= REL_L2
+        assert float((lse.cpu()[touched] - exp_lse[touched]).abs().max()) < 2e-2
