@@ -338,6 +338,7 @@ sparse_fa_kernel(const FaParams p) {
   __shared__ int s_arrived;
   __shared__ int s_queue[16];  // queue bounds and even-share words of `sched`, read once
   __shared__ int s_share[1];   // even shares: items of this workgroup's share handed out so far
+  __shared__ int s_guess;      // queues: one past the position this workgroup popped last
   __shared__ RowInfo s_items[kItemBatch];  // even shares: records of the share's next items
   constexpr int kRowBlocks = kGroups == 1 ? kMaxRowBlocksOneGroup : kKLo ? kMaxRowBlocksKLo : kMaxRowBlocks;
   __shared__ uint16_t s_blk2[2][kRowBlocks];  // kv block list of this row / the next one
@@ -396,6 +397,7 @@ sparse_fa_kernel(const FaParams p) {
   // (group 1 has nothing else to do then), so the queue atomics are off the critical path.
   if (tid < 9) s_queue[tid] = p.sched[tid];
   if (tid >= 64 && tid < 64 + 6) s_queue[9 + tid - 64] = p.sched[kSchedEven + tid - 64];
+  if (tid == 128) s_guess = 0;
   __syncthreads();
   // Even shares: the decoder has laid the rows out head by head and given every row a cost
   // (kRowOverhead + its kv blocks); share j is the cost range [j * share, (j + 1) * share), and a
@@ -473,16 +475,56 @@ sparse_fa_kernel(const FaParams p) {
         s_share[0] = c + 1;
         s_next_row[slot_idx] = ri;
       }
-    } else if (lane == 0) {
-      const int at = pop_row(p, blockIdx.x & (kXcds - 1), s_queue, &first_queue);
+    } else {
+      // Queues.  The trips to memory are kept to two: the pop's atomic travels together with loads of
+      // the 64 records that follow this workgroup's last position in the queue (the 32 workgroups of an
+      // XCD pop about once per row each, so the answer is nearly always one of them; otherwise the
+      // record is read after the pop), and the row's bounds and its kv block list are asked for
+      // together once the record is known.
+      typedef __attribute__((ext_vector_type(4))) int i32x4;
+      const int xcd = blockIdx.x & (kXcds - 1);
+      i32x4 w0 = {0, 0, 0, 0}, w1 = w0;  // lane i: the record at queue position win_lo + i
+      int win_lo = 0, win_hi = 0;
+      if (have_records) {
+        const int fq = __builtin_amdgcn_readfirstlane(first_queue);
+        if (fq < kXcds) {
+          const int x = (xcd + fq) & (kXcds - 1);
+          win_lo = max(queue_word(x), __builtin_amdgcn_readfirstlane(s_guess));
+          win_hi = min(queue_word(x + 1), win_lo + 64);
+          if (win_lo + lane < win_hi) {
+            const i32x4* rec = reinterpret_cast<const i32x4*>(p.shares + kMaxShares + kRecordInts * static_cast<int64_t>(win_lo + lane));
+            w0 = rec[0];
+            w1 = rec[1];
+          }
+        }
+      }
+      int at_lane = -1;
+      if (lane == 0) at_lane = pop_row(p, xcd, s_queue, &first_queue);
+      const int at = __builtin_amdgcn_readfirstlane(at_lane);
       ri.part = 0;
       ri.parts = 1;
       ri.slot = 0;
       if (at >= 0) {
+        // (every lane forms the row's values: they are uniform, and lane 0 stores them)
         if (have_records) {
-          // one record per queue entry, left by the decoder: one round of loads after the pop
-          const i32x4* rec = reinterpret_cast<const i32x4*>(p.shares + kMaxShares + kRecordInts * static_cast<int64_t>(at));
-          const i32x4 r0 = rec[0], r1 = rec[1];
+          i32x4 r0, r1;
+          if (at >= win_lo && at < win_hi) {
+            const int d = at - win_lo;
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+              r0[j] = __builtin_amdgcn_readlane(w0[j], d);
+              r1[j] = __builtin_amdgcn_readlane(w1[j], d);
+            }
+          } else {
+            const i32x4* rec = reinterpret_cast<const i32x4*>(p.shares + kMaxShares + kRecordInts * static_cast<int64_t>(at));
+            r0 = rec[0];
+            r1 = rec[1];
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+              r0[j] = __builtin_amdgcn_readfirstlane(r0[j]);
+              r1[j] = __builtin_amdgcn_readfirstlane(r1[j]);
+            }
+          }
           ri.row = r0[0];
           ri.req = r0[1];
           ri.qb = r0[2];
@@ -490,24 +532,40 @@ sparse_fa_kernel(const FaParams p) {
           ri.ptr0 = r1[0];
           ri.nb = min(r1[1], kRowBlocks);
         } else {
-          const int w = p.order[at];
+          const int w = __builtin_amdgcn_readfirstlane(p.order[at]);
           ri.row = w;
-          ri.req = p.row_req[w];
-          ri.qb = p.row_qb[w];
-          ri.head = p.row_head[w];
-          ri.ptr0 = p.kv_row_ptr[w];
+          ri.req = __builtin_amdgcn_readfirstlane(p.row_req[w]);
+          ri.qb = __builtin_amdgcn_readfirstlane(p.row_qb[w]);
+          ri.head = __builtin_amdgcn_readfirstlane(p.row_head[w]);
+          ri.ptr0 = __builtin_amdgcn_readfirstlane(p.kv_row_ptr[w]);
           // (a row longer than the LDS list is cut; the host side refuses such requests at plan time)
-          ri.nb = min(p.kv_row_ptr[w + 1] - ri.ptr0, kRowBlocks);
+          ri.nb = min(__builtin_amdgcn_readfirstlane(p.kv_row_ptr[w + 1]) - ri.ptr0, kRowBlocks);
         }
+        // the first 64 entries of the list are asked for before the bounds are waited for
+        const int n = ri.nb, list0 = ri.ptr0;
+        int blk_first = 0;
+        if (lane < n) blk_first = p.kv_idx[list0 + lane];
         set_q_range(ri);
         ri.kv_begin = p.kv_indptr[ri.req];
         ri.kv_len = p.kv_indptr[ri.req + 1] - ri.kv_begin;
         fill_scales(ri);
+        if (lane < n) {
+          s_blk2[slot_idx][lane] = static_cast<uint16_t>(blk_first);
+          if constexpr (kFp8) s_ksc2[slot_idx][lane] = p.k_scale[ri.k_scale0 + blk_first];
+        }
+        for (int i = 64 + lane; i < n; i += 64) {
+          const int blk = p.kv_idx[list0 + i];
+          s_blk2[slot_idx][i] = static_cast<uint16_t>(blk);
+          if constexpr (kFp8) s_ksc2[slot_idx][i] = p.k_scale[ri.k_scale0 + blk];
+        }
       }
-      s_next_row[slot_idx] = ri;
+      if (lane == 0) {
+        s_next_row[slot_idx] = ri;
+        if (at >= 0) s_guess = at + 1;
+      }
     }
-    const int row = __builtin_amdgcn_readfirstlane(ri.row);
-    if (row >= 0) {
+    if (even && __builtin_amdgcn_readfirstlane(ri.row) >= 0) {
+      // (even shares: lane 0 holds the item; every lane copies its part of the kv block list)
       const int list0 = __builtin_amdgcn_readfirstlane(ri.ptr0), n = __builtin_amdgcn_readfirstlane(ri.nb);
       const int ks0 = __builtin_amdgcn_readfirstlane(ri.k_scale0);
       for (int i = lane; i < n; i += 64) {
