@@ -1050,14 +1050,16 @@ __global__ void __launch_bounds__(kThreads) gemm_kernel(const GemmParams p) {
             }
           }
           const f32x4 v = vals[i & 7];
+          // (stored with the streaming hint, cache policy 2: the output is not read again by this launch
+          // and should not push operand tiles out of the L2; 0.5-1.5 % at both sizes)
           if constexpr (kOutF32) {
-            __builtin_amdgcn_raw_buffer_store_b128(__builtin_bit_cast(u32x4, v), ry, el_off * 4, row_off(i, 4), 0);
+            __builtin_amdgcn_raw_buffer_store_b128(__builtin_bit_cast(u32x4, v), ry, el_off * 4, row_off(i, 4), 2);
           } else {
             x4 out;
 #pragma unroll
             for (int j = 0; j < 4; ++j) out[j] = static_cast<T>(v[j]);
             typedef __attribute__((ext_vector_type(2))) unsigned int u32x2;
-            __builtin_amdgcn_raw_buffer_store_b64(__builtin_bit_cast(u32x2, out), ry, el_off * 2, row_off(i, 2), 0);
+            __builtin_amdgcn_raw_buffer_store_b64(__builtin_bit_cast(u32x2, out), ry, el_off * 2, row_off(i, 2), 2);
           }
           if constexpr (kQuant) {
             float f[4];
